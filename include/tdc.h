@@ -1,0 +1,157 @@
+/*
+ * tdc.h — C ABI of the MI355X (gfx950) Tucker-convolution library.
+ *
+ * Plain C: pointers, ints and sizes only.  Every entry point returns a
+ * tdc_status (0 = success) and never terminates the process; the text of the
+ * last failure on the calling thread is available from tdc_last_error_string().
+ *
+ * Tensors are fp32, contiguous NCHW; weights are handed over in PyTorch's OIHW
+ * order and re-packed once at set-weights time.  Activations are DEVICE
+ * pointers owned by the caller; weight/bias arguments are HOST pointers.
+ * `stream` is a hipStream_t passed as void* (NULL = the default stream).
+ *
+ * What each entry point replaces in the reference (paths relative to the
+ * reference tree):
+ *   tdc_conv_*      Conv::initialize / Conv::forward
+ *                   (2080Ti-evaluation/EndToEnd/resnet18-tk/inc/common.h:38-69,
+ *                    src/Conv.cu:2-125) and the raw generated kernel
+ *                   conv2d(input, kernel, outputs)
+ *                   (2080Ti-evaluation/TDC-LAYERS-ORACLE/template_benchmark_cudnn.template:365-402,490-492)
+ *   tdc_tkconv_*    TkConv::initialize / TkConv::forward (common.h:158-166,
+ *                   src/BasicBlock.cu:14-31) and TKConv2dC.forward /
+ *                   forward_features (inference/TKConv.py:90-106)
+ *   tdc_model_*     compute_latency / compute_*_vol / modeling
+ *                   (2080Ti-evaluation/TDC-LAYERS-MODELING/model.py:136-156,209-235)
+ *                   and the occupancy probe (2080Ti-evaluation/Gen-occupancy/template.cu:277-284)
+ */
+#ifndef TDC_H
+#define TDC_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum tdc_status {
+    TDC_OK = 0,
+    TDC_ERR_INVALID = 1,     /* bad argument / inconsistent descriptor          */
+    TDC_ERR_UNSUPPORTED = 2, /* legal request the library has no kernel for     */
+    TDC_ERR_HIP = 3,         /* a HIP runtime call failed (see error string)    */
+    TDC_ERR_NOMEM = 4,       /* host or device allocation failed                */
+    TDC_ERR_STATE = 5        /* call order violated (e.g. forward before weights) */
+} tdc_status;
+
+/* One convolution: out[b,n,oy,ox] = sum_{c,r,s} w[n,c,r,s] * in[b,c,oy*stride-pad+r*dil, ox*stride-pad+s*dil]
+ * (cross-correlation, zero padding, groups = 1), then optionally + bias[n],
+ * + residual[b,n,oy,ox], then optionally ReLU — in that order. */
+typedef struct tdc_conv_desc {
+    int32_t batch;
+    int32_t C;          /* input channels                                      */
+    int32_t N;          /* OUTPUT channels (the reference's naming; not batch) */
+    int32_t H, W;       /* input height / width                                */
+    int32_t KH, KW;     /* filter height / width                               */
+    int32_t stride;
+    int32_t pad;
+    int32_t dilation;
+    int32_t has_bias;
+    int32_t relu;       /* fuse max(x,0) after bias/residual                   */
+} tdc_conv_desc;
+
+/* Tiling of one convolution on the gfx950 compute unit.  One workgroup computes
+ * an (mf*mb*wm) output-channel x (mf*nb*wn) flat-pixel tile; its wm*wn*wk
+ * wavefronts split output channels, pixels and input channels; input channels
+ * are staged through LDS `cch` at a time. */
+typedef struct tdc_tile {
+    int32_t mf;   /* MFMA block edge: 32 (v_mfma_f32_32x32x2_f32) or 16 (16x16x4) */
+    int32_t mb;   /* MFMA blocks per wave along output channels (1 or 2)        */
+    int32_t nb;   /* MFMA blocks per wave along pixels (1 or 2)                 */
+    int32_t wm;   /* waves along output channels                               */
+    int32_t wn;   /* waves along pixels                                        */
+    int32_t wk;   /* waves along input channels (in-workgroup split-K)          */
+    int32_t cch;  /* input channels staged in LDS per pass                      */
+} tdc_tile;
+
+typedef struct tdc_tile_info {
+    tdc_tile tile;
+    int32_t grid_x, grid_y, grid_z;  /* pixel tiles, channel tiles, batch      */
+    int32_t block_threads;
+    int32_t lds_bytes;
+    int32_t vgpr_estimate;           /* per lane, arch+acc                     */
+    int32_t waves_per_simd;          /* resident, limited by VGPR/LDS/slots    */
+    int32_t wg_per_cu;
+    int32_t nchunks;                 /* LDS passes over input channels         */
+    double flops;                    /* algorithmic 2*Ho*Wo*C*N*KH*KW*batch    */
+    double bytes;                    /* algorithmic: in + out + weights once   */
+    double roof_us;                  /* max(bytes/8TB/s, flops/157.3TF)        */
+    double pred_us;                  /* analytic model's predicted device time */
+    double pred_hbm_bytes;           /* modelled L2->CU traffic (re-reads incl.) */
+} tdc_tile_info;
+
+typedef struct tdc_conv_plan tdc_conv_plan;
+typedef struct tdc_tkconv tdc_tkconv;
+
+const char *tdc_last_error_string(void);
+const char *tdc_version(void);
+
+/* ---- single convolution -------------------------------------------------- */
+
+/* `forced_tile` NULL = let the analytic model choose.  Needs a HIP device. */
+int tdc_conv_plan_create(const tdc_conv_desc *desc, const tdc_tile *forced_tile,
+                         tdc_conv_plan **plan_out);
+/* Host OIHW weights [N,C,KH,KW]; bias [N] or NULL (must match has_bias). */
+int tdc_conv_plan_set_weights(tdc_conv_plan *plan, const float *w_oihw, const float *bias);
+int tdc_conv_plan_query(const tdc_conv_plan *plan, tdc_tile_info *info_out);
+/* d_residual may be NULL.  Output need not be pre-zeroed.  Asynchronous. */
+int tdc_conv_forward(tdc_conv_plan *plan, const float *d_in, const float *d_residual,
+                     float *d_out, void *stream);
+void tdc_conv_plan_destroy(tdc_conv_plan *plan);
+
+/* ---- TKConv operator: 1x1 C->R1, KxK R1->R2 (stride/pad/dilation), 1x1 R2->N (+bias) */
+
+typedef struct tdc_tkconv_desc {
+    int32_t batch;
+    int32_t C;        /* in_channels                      */
+    int32_t R1;       /* in_rank  (hp_dict.ranks[name][1]) */
+    int32_t R2;       /* out_rank (hp_dict.ranks[name][0]) */
+    int32_t N;        /* out_channels                     */
+    int32_t H, W;
+    int32_t K;        /* core kernel size (square)        */
+    int32_t stride, pad, dilation;   /* of the core conv  */
+    int32_t has_bias; /* bias of the last 1x1             */
+    int32_t relu;     /* fuse ReLU after the last 1x1     */
+} tdc_tkconv_desc;
+
+int tdc_tkconv_create(const tdc_tkconv_desc *desc, tdc_tkconv **op_out);
+/* Host pointers: first [R1,C,1,1], core [R2,R1,K,K], last [N,R2,1,1], bias [N] or NULL. */
+int tdc_tkconv_set_weights(tdc_tkconv *op, const float *first, const float *core,
+                           const float *last, const float *bias);
+/* Full operator; intermediates live in op-owned device buffers. */
+int tdc_tkconv_forward(tdc_tkconv *op, const float *d_in, const float *d_residual,
+                       float *d_out, void *stream);
+/* Same, also copying out the two intermediates (either may be NULL). */
+int tdc_tkconv_forward_features(tdc_tkconv *op, const float *d_in, float *d_feat_first,
+                                float *d_feat_core, float *d_out, void *stream);
+/* Only the KxK core conv: d_in is [batch,R1,H,W], d_out [batch,R2,Ho,Wo]. */
+int tdc_tkconv_core_forward(tdc_tkconv *op, const float *d_in, float *d_out, void *stream);
+/* which: 0 = first 1x1, 1 = core, 2 = last 1x1 */
+int tdc_tkconv_query(const tdc_tkconv *op, int which, tdc_tile_info *info_out);
+void tdc_tkconv_destroy(tdc_tkconv *op);
+
+/* ---- analytic gfx950 tile model (host only; works without a GPU) ---------- */
+
+/* Fill `info_out` (tile, launch geometry, predicted time) for a given tile;
+ * returns TDC_ERR_INVALID if the tile is not launchable for this shape. */
+int tdc_model_evaluate(const tdc_conv_desc *desc, const tdc_tile *tile, tdc_tile_info *info_out);
+/* Enumerate every launchable tile (up to `cap`) in the model's search order;
+ * *count_out receives the number written. */
+int tdc_model_enumerate(const tdc_conv_desc *desc, tdc_tile *tiles_out, int32_t cap,
+                        int32_t *count_out);
+/* The model's pick = argmin pred_us over tdc_model_enumerate. */
+int tdc_model_select(const tdc_conv_desc *desc, tdc_tile_info *info_out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TDC_H */

@@ -1,0 +1,284 @@
+// C ABI: plans, weight upload, forward calls.  See include/tdc.h for the
+// reference interfaces each entry point stands in for.
+#include <hip/hip_runtime_api.h>
+
+#include <cstdio>
+#include <cstring>
+#include <memory>
+#include <new>
+#include <string>
+#include <vector>
+
+#include "tdc_internal.hpp"
+
+namespace tdc {
+
+static thread_local std::string g_last_error;
+
+void set_error(const std::string &msg) { g_last_error = msg; }
+
+static int fail(tdc_status st, const std::string &msg) {
+    set_error(msg);
+    return (int)st;
+}
+
+static int hip_fail(const char *what, int err) {
+    return fail(TDC_ERR_HIP, std::string(what) + ": " + hipGetErrorString((hipError_t)err));
+}
+
+}  // namespace tdc
+
+using namespace tdc;
+
+struct tdc_conv_plan {
+    tdc_conv_desc desc{};
+    tdc_tile tile{};
+    tdc_tile_info info{};
+    Geometry geo{};
+    const void *kernel = nullptr;
+    float *d_wpk = nullptr;
+    float *d_bias = nullptr;
+    bool have_weights = false;
+};
+
+struct tdc_tkconv {
+    tdc_tkconv_desc desc{};
+    tdc_conv_plan *first = nullptr;
+    tdc_conv_plan *core = nullptr;
+    tdc_conv_plan *last = nullptr;
+    float *d_f1 = nullptr;  // [batch, R1, H, W]
+    float *d_f2 = nullptr;  // [batch, R2, Ho, Wo]
+    size_t f1_floats = 0, f2_floats = 0;
+};
+
+extern "C" {
+
+const char *tdc_last_error_string(void) { return g_last_error.c_str(); }
+
+const char *tdc_version(void) { return "tdc-amd 0.1 (gfx950)"; }
+
+int tdc_model_evaluate(const tdc_conv_desc *desc, const tdc_tile *tile, tdc_tile_info *info_out) {
+    if (!desc || !tile || !info_out) return fail(TDC_ERR_INVALID, "null argument");
+    std::string why;
+    if (!model_evaluate(*desc, *tile, *info_out, &why)) return fail(TDC_ERR_INVALID, why);
+    return TDC_OK;
+}
+
+int tdc_model_enumerate(const tdc_conv_desc *desc, tdc_tile *tiles_out, int32_t cap, int32_t *count_out) {
+    if (!desc || !count_out || cap < 0 || (cap > 0 && !tiles_out)) return fail(TDC_ERR_INVALID, "null argument");
+    std::string why;
+    if (!check_desc(*desc, &why)) return fail(TDC_ERR_INVALID, why);
+    std::vector<tdc_tile> v = model_enumerate(*desc);
+    int32_t n = 0;
+    for (const tdc_tile &t : v) {
+        if (n >= cap) break;
+        tiles_out[n++] = t;
+    }
+    *count_out = n;
+    return TDC_OK;
+}
+
+int tdc_model_select(const tdc_conv_desc *desc, tdc_tile_info *info_out) {
+    if (!desc || !info_out) return fail(TDC_ERR_INVALID, "null argument");
+    std::string why;
+    if (!model_select(*desc, *info_out, &why)) return fail(TDC_ERR_INVALID, why);
+    return TDC_OK;
+}
+
+int tdc_conv_plan_create(const tdc_conv_desc *desc, const tdc_tile *forced_tile, tdc_conv_plan **plan_out) {
+    if (!desc || !plan_out) return fail(TDC_ERR_INVALID, "null argument");
+    *plan_out = nullptr;
+    std::string why;
+    if (!check_desc(*desc, &why)) return fail(TDC_ERR_INVALID, why);
+    int ndev = 0;
+    hipError_t e = hipGetDeviceCount(&ndev);
+    if (e != hipSuccess || ndev < 1)
+        return fail(TDC_ERR_HIP, "no HIP device available: the convolution kernels only run on a gfx950 GPU");
+    std::unique_ptr<tdc_conv_plan> p(new (std::nothrow) tdc_conv_plan());
+    if (!p) return fail(TDC_ERR_NOMEM, "out of host memory");
+    p->desc = *desc;
+    if (forced_tile) {
+        if (!model_evaluate(*desc, *forced_tile, p->info, &why)) return fail(TDC_ERR_INVALID, "forced tile: " + why);
+    } else {
+        if (!model_select(*desc, p->info, &why)) return fail(TDC_ERR_UNSUPPORTED, why);
+    }
+    p->tile = p->info.tile;
+    if (!make_geometry(*desc, p->tile, p->geo, &why)) return fail(TDC_ERR_INVALID, why);
+    p->kernel = conv_kernel_for(p->tile, desc->KH, desc->KW);
+    if (!p->kernel) return fail(TDC_ERR_UNSUPPORTED, "no kernel instantiated for this tile");
+    int he = prepare_conv_kernel(p->kernel, p->geo);
+    if (he) return hip_fail("hipFuncSetAttribute(MaxDynamicSharedMemorySize)", he);
+    const size_t wfloats = packed_weight_floats(p->geo, p->tile.mf);
+    e = hipMalloc((void **)&p->d_wpk, wfloats * sizeof(float));
+    if (e != hipSuccess) return hip_fail("hipMalloc(packed weights)", e);
+    if (desc->has_bias) {
+        e = hipMalloc((void **)&p->d_bias, (size_t)desc->N * sizeof(float));
+        if (e != hipSuccess) {
+            (void)hipFree(p->d_wpk);
+            return hip_fail("hipMalloc(bias)", e);
+        }
+    }
+    *plan_out = p.release();
+    return TDC_OK;
+}
+
+int tdc_conv_plan_set_weights(tdc_conv_plan *plan, const float *w_oihw, const float *bias) {
+    if (!plan || !w_oihw) return fail(TDC_ERR_INVALID, "null argument");
+    if ((plan->desc.has_bias != 0) != (bias != nullptr))
+        return fail(TDC_ERR_INVALID, "bias pointer does not match desc.has_bias");
+    const size_t wfloats = packed_weight_floats(plan->geo, plan->tile.mf);
+    std::vector<float> packed;
+    try {
+        packed.resize(wfloats);
+    } catch (const std::bad_alloc &) {
+        return fail(TDC_ERR_NOMEM, "out of host memory packing weights");
+    }
+    pack_weights(plan->desc, plan->geo, plan->tile.mf, w_oihw, packed.data());
+    hipError_t e = hipMemcpy(plan->d_wpk, packed.data(), wfloats * sizeof(float), hipMemcpyHostToDevice);
+    if (e != hipSuccess) return hip_fail("hipMemcpy(packed weights)", e);
+    if (bias) {
+        e = hipMemcpy(plan->d_bias, bias, (size_t)plan->desc.N * sizeof(float), hipMemcpyHostToDevice);
+        if (e != hipSuccess) return hip_fail("hipMemcpy(bias)", e);
+    }
+    plan->have_weights = true;
+    return TDC_OK;
+}
+
+int tdc_conv_plan_query(const tdc_conv_plan *plan, tdc_tile_info *info_out) {
+    if (!plan || !info_out) return fail(TDC_ERR_INVALID, "null argument");
+    *info_out = plan->info;
+    return TDC_OK;
+}
+
+int tdc_conv_forward(tdc_conv_plan *plan, const float *d_in, const float *d_residual, float *d_out, void *stream) {
+    if (!plan || !d_in || !d_out) return fail(TDC_ERR_INVALID, "null argument");
+    if (!plan->have_weights) return fail(TDC_ERR_STATE, "tdc_conv_forward before tdc_conv_plan_set_weights");
+    const tdc_conv_desc &d = plan->desc;
+    const Geometry &g = plan->geo;
+    ConvKParams kp{};
+    kp.in = d_in;
+    kp.wpk = plan->d_wpk;
+    kp.bias = plan->d_bias;
+    kp.resid = d_residual;
+    kp.out = d_out;
+    kp.C = d.C; kp.H = d.H; kp.W = d.W; kp.N = d.N;
+    kp.Ho = g.Ho; kp.Wo = g.Wo; kp.P = g.P;
+    kp.KH = d.KH; kp.KW = d.KW; kp.stride = d.stride; kp.pad = d.pad; kp.dil = d.dilation;
+    kp.WM = plan->tile.wm; kp.WN = plan->tile.wn; kp.WK = plan->tile.wk;
+    kp.CCH = plan->tile.cch; kp.nchunks = g.nchunks; kp.CPW = g.cpw;
+    kp.RS = g.RS; kp.CS = g.CS; kp.PL = g.PL;
+    kp.relu = d.relu;
+    kp.ncg_total = g.c_pad / g.kc;
+    kp.in_bstride = (long long)d.C * d.H * d.W;
+    kp.out_bstride = (long long)d.N * g.P;
+    int he = launch_conv(plan->kernel, g, kp, stream);
+    if (he) return hip_fail("kernel launch", he);
+    return TDC_OK;
+}
+
+void tdc_conv_plan_destroy(tdc_conv_plan *plan) {
+    if (!plan) return;
+    if (plan->d_wpk) (void)hipFree(plan->d_wpk);
+    if (plan->d_bias) (void)hipFree(plan->d_bias);
+    delete plan;
+}
+
+// ---- TKConv ---------------------------------------------------------------
+
+int tdc_tkconv_create(const tdc_tkconv_desc *desc, tdc_tkconv **op_out) {
+    if (!desc || !op_out) return fail(TDC_ERR_INVALID, "null argument");
+    *op_out = nullptr;
+    if (desc->R1 < 1 || desc->R2 < 1 || desc->K < 1) return fail(TDC_ERR_INVALID, "R1, R2, K must be >= 1");
+    std::unique_ptr<tdc_tkconv> op(new (std::nothrow) tdc_tkconv());
+    if (!op) return fail(TDC_ERR_NOMEM, "out of host memory");
+    op->desc = *desc;
+    tdc_conv_desc d1{desc->batch, desc->C, desc->R1, desc->H, desc->W, 1, 1, 1, 0, 1, 0, 0};
+    tdc_conv_desc d2{desc->batch, desc->R1, desc->R2, desc->H, desc->W, desc->K, desc->K,
+                     desc->stride, desc->pad, desc->dilation, 0, 0};
+    std::string why;
+    if (!check_desc(d1, &why)) return fail(TDC_ERR_INVALID, "first 1x1: " + why);
+    if (!check_desc(d2, &why)) return fail(TDC_ERR_INVALID, "core conv: " + why);
+    const int Ho = (desc->H + 2 * desc->pad - desc->dilation * (desc->K - 1) - 1) / desc->stride + 1;
+    const int Wo = (desc->W + 2 * desc->pad - desc->dilation * (desc->K - 1) - 1) / desc->stride + 1;
+    tdc_conv_desc d3{desc->batch, desc->R2, desc->N, Ho, Wo, 1, 1, 1, 0, 1, desc->has_bias, desc->relu};
+    if (!check_desc(d3, &why)) return fail(TDC_ERR_INVALID, "last 1x1: " + why);
+    int st;
+    auto cleanup = [&]() {
+        tdc_conv_plan_destroy(op->first);
+        tdc_conv_plan_destroy(op->core);
+        tdc_conv_plan_destroy(op->last);
+        if (op->d_f1) (void)hipFree(op->d_f1);
+        if (op->d_f2) (void)hipFree(op->d_f2);
+    };
+    if ((st = tdc_conv_plan_create(&d1, nullptr, &op->first)) != TDC_OK) { cleanup(); return st; }
+    if ((st = tdc_conv_plan_create(&d2, nullptr, &op->core)) != TDC_OK) { cleanup(); return st; }
+    if ((st = tdc_conv_plan_create(&d3, nullptr, &op->last)) != TDC_OK) { cleanup(); return st; }
+    op->f1_floats = (size_t)desc->batch * desc->R1 * desc->H * desc->W;
+    op->f2_floats = (size_t)desc->batch * desc->R2 * Ho * Wo;
+    hipError_t e = hipMalloc((void **)&op->d_f1, op->f1_floats * sizeof(float));
+    if (e != hipSuccess) { cleanup(); return hip_fail("hipMalloc(first intermediate)", e); }
+    e = hipMalloc((void **)&op->d_f2, op->f2_floats * sizeof(float));
+    if (e != hipSuccess) { cleanup(); return hip_fail("hipMalloc(core intermediate)", e); }
+    *op_out = op.release();
+    return TDC_OK;
+}
+
+int tdc_tkconv_set_weights(tdc_tkconv *op, const float *first, const float *core, const float *last,
+                           const float *bias) {
+    if (!op || !first || !core || !last) return fail(TDC_ERR_INVALID, "null argument");
+    int st;
+    if ((st = tdc_conv_plan_set_weights(op->first, first, nullptr)) != TDC_OK) return st;
+    if ((st = tdc_conv_plan_set_weights(op->core, core, nullptr)) != TDC_OK) return st;
+    if ((st = tdc_conv_plan_set_weights(op->last, last, bias)) != TDC_OK) return st;
+    return TDC_OK;
+}
+
+int tdc_tkconv_forward(tdc_tkconv *op, const float *d_in, const float *d_residual, float *d_out, void *stream) {
+    if (!op || !d_in || !d_out) return fail(TDC_ERR_INVALID, "null argument");
+    int st;
+    if ((st = tdc_conv_forward(op->first, d_in, nullptr, op->d_f1, stream)) != TDC_OK) return st;
+    if ((st = tdc_conv_forward(op->core, op->d_f1, nullptr, op->d_f2, stream)) != TDC_OK) return st;
+    return tdc_conv_forward(op->last, op->d_f2, d_residual, d_out, stream);
+}
+
+int tdc_tkconv_forward_features(tdc_tkconv *op, const float *d_in, float *d_feat_first, float *d_feat_core,
+                                float *d_out, void *stream) {
+    int st = tdc_tkconv_forward(op, d_in, nullptr, d_out, stream);
+    if (st != TDC_OK) return st;
+    hipError_t e;
+    if (d_feat_first) {
+        e = hipMemcpyAsync(d_feat_first, op->d_f1, op->f1_floats * sizeof(float), hipMemcpyDeviceToDevice,
+                           (hipStream_t)stream);
+        if (e != hipSuccess) return hip_fail("hipMemcpyAsync(first feature)", e);
+    }
+    if (d_feat_core) {
+        e = hipMemcpyAsync(d_feat_core, op->d_f2, op->f2_floats * sizeof(float), hipMemcpyDeviceToDevice,
+                           (hipStream_t)stream);
+        if (e != hipSuccess) return hip_fail("hipMemcpyAsync(core feature)", e);
+    }
+    return TDC_OK;
+}
+
+int tdc_tkconv_core_forward(tdc_tkconv *op, const float *d_in, float *d_out, void *stream) {
+    if (!op) return fail(TDC_ERR_INVALID, "null argument");
+    return tdc_conv_forward(op->core, d_in, nullptr, d_out, stream);
+}
+
+int tdc_tkconv_query(const tdc_tkconv *op, int which, tdc_tile_info *info_out) {
+    if (!op || !info_out) return fail(TDC_ERR_INVALID, "null argument");
+    const tdc_conv_plan *p = which == 0 ? op->first : which == 1 ? op->core : which == 2 ? op->last : nullptr;
+    if (!p) return fail(TDC_ERR_INVALID, "which must be 0, 1 or 2");
+    return tdc_conv_plan_query(p, info_out);
+}
+
+void tdc_tkconv_destroy(tdc_tkconv *op) {
+    if (!op) return;
+    tdc_conv_plan_destroy(op->first);
+    tdc_conv_plan_destroy(op->core);
+    tdc_conv_plan_destroy(op->last);
+    if (op->d_f1) (void)hipFree(op->d_f1);
+    if (op->d_f2) (void)hipFree(op->d_f2);
+    delete op;
+}
+
+}  // extern "C"

@@ -1,0 +1,93 @@
+// Internal declarations shared by the tile model, the weight packer, the kernel
+// launcher and the C ABI.  Nothing here is exported.
+#pragma once
+
+#include <cstddef>
+#include <cstdint>
+#include <string>
+#include <vector>
+
+#include "tdc.h"
+
+namespace tdc {
+
+// ---- gfx950 (MI355X) machine description used by the analytic model -------
+struct Machine {
+    int cus = 256;                // 8 XCDs x 32 CUs
+    int xcds = 8;
+    int simds_per_cu = 4;
+    int max_waves_per_simd = 8;
+    int vgprs_per_simd_lane = 512;   // unified arch+acc file per lane
+    int lds_bytes_per_cu = 160 * 1024;
+    int max_wg_threads = 1024;
+    double clock_ghz = 2.4;
+    double hbm_tbps = 8.0;
+    double fp32_tflops = 157.3;      // MFMA fp32 dense peak
+};
+const Machine &machine();
+
+// ---- launch geometry derived from (desc, tile) ----------------------------
+struct Geometry {
+    int Ho = 0, Wo = 0, P = 0;       // output height/width, Ho*Wo
+    int kc = 0;                      // input channels consumed per MFMA (2 or 4)
+    int taps = 0;                    // KH*KW
+    int PT = 0, MT = 0;              // pixels / output channels per workgroup
+    int grid_x = 0, grid_y = 0, grid_z = 0;
+    int waves = 0, threads = 0;
+    int cpw = 0;                     // channels per wave per LDS pass (cch / wk)
+    int nchunks = 0;                 // LDS passes
+    int c_pad = 0;                   // nchunks * cch
+    int n_pad = 0;                   // grid_y * MT (rows of the packed weights)
+    int PL = 0;                      // left zero columns in an LDS row
+    int RS = 0;                      // LDS row stride (floats)
+    int nrows = 0;                   // max input rows a workgroup stages
+    int CS = 0;                      // LDS channel stride (floats)
+    int lds_bytes = 0;
+    int max_waves_kernel = 0;        // launch bound of the instantiated kernel
+};
+
+// Returns false (and a reason) when the tile cannot be launched for this shape.
+bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::string *why);
+bool check_desc(const tdc_conv_desc &d, std::string *why);
+
+// Model: fills everything in `info` except nothing device-specific.
+bool model_evaluate(const tdc_conv_desc &d, const tdc_tile &t, tdc_tile_info &info, std::string *why);
+std::vector<tdc_tile> model_enumerate(const tdc_conv_desc &d);
+bool model_select(const tdc_conv_desc &d, tdc_tile_info &info, std::string *why);
+
+// ---- weight packing --------------------------------------------------------
+// OIHW [N,C,KH,KW] -> MFMA A-operand order [n_pad/mf][c_pad/kc][taps][64 lanes]:
+// lane l of entry (mblk, cg, tap) holds w[mblk*mf + l%mf][cg*kc + l/mf][tap],
+// zero outside N x C.
+size_t packed_weight_floats(const Geometry &g, int mf);
+void pack_weights(const tdc_conv_desc &d, const Geometry &g, int mf, const float *w_oihw,
+                  float *packed);
+
+// ---- kernel arguments ------------------------------------------------------
+struct ConvKParams {
+    const float *in;
+    const float *wpk;
+    const float *bias;
+    const float *resid;
+    float *out;
+    int C, H, W, N, Ho, Wo, P;
+    int KH, KW, stride, pad, dil;
+    int WM, WN, WK;
+    int CCH, nchunks, CPW;
+    int RS, CS, PL;
+    int relu;
+    int ncg_total;        // c_pad / kc
+    long long in_bstride;   // C*H*W
+    long long out_bstride;  // N*P
+};
+
+// The instantiated kernel for a tile and filter size (nullptr if none).
+const void *conv_kernel_for(const tdc_tile &t, int KH, int KW);
+// One-time per-plan attribute setup (dynamic LDS above 64 KiB).  hipError_t as int.
+int prepare_conv_kernel(const void *fn, const Geometry &g);
+// Enqueue the kernel.  Returns a hipError_t as int.
+int launch_conv(const void *fn, const Geometry &g, const ConvKParams &kp, void *stream);
+
+void set_error(const std::string &msg);
+
+}  // namespace tdc

@@ -1,0 +1,133 @@
+"""ctypes binding of libtdc_amd.so (the C ABI declared in include/tdc.h).
+
+The library is built in-tree by ``ppopp23-tdc_amd/build.py``; nothing here falls
+back to another implementation when it is missing.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import POINTER, Structure, byref, c_char_p, c_double, c_int, c_int32, c_void_p
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libtdc_amd.so")
+
+TDC_OK, TDC_ERR_INVALID, TDC_ERR_UNSUPPORTED, TDC_ERR_HIP, TDC_ERR_NOMEM, TDC_ERR_STATE = range(6)
+
+# Every symbol include/tdc.h declares.
+EXPORTS = (
+    "tdc_last_error_string", "tdc_version",
+    "tdc_conv_plan_create", "tdc_conv_plan_set_weights", "tdc_conv_plan_query", "tdc_conv_forward",
+    "tdc_conv_plan_destroy",
+    "tdc_tkconv_create", "tdc_tkconv_set_weights", "tdc_tkconv_forward", "tdc_tkconv_forward_features",
+    "tdc_tkconv_core_forward", "tdc_tkconv_query", "tdc_tkconv_destroy",
+    "tdc_model_evaluate", "tdc_model_enumerate", "tdc_model_select",
+)
+
+
+class TdcError(RuntimeError):
+    def __init__(self, status, message):
+        super().__init__(f"tdc status {status}: {message}")
+        self.status = status
+
+
+class ConvDesc(Structure):
+    _fields_ = [(n, c_int32) for n in ("batch", "C", "N", "H", "W", "KH", "KW", "stride", "pad", "dilation",
+                                       "has_bias", "relu")]
+
+
+class Tile(Structure):
+    _fields_ = [(n, c_int32) for n in ("mf", "mb", "nb", "wm", "wn", "wk", "cch")]
+
+    def astuple(self):
+        return (self.mf, self.mb, self.nb, self.wm, self.wn, self.wk, self.cch)
+
+    def __repr__(self):
+        return "Tile(mf=%d, mb=%d, nb=%d, wm=%d, wn=%d, wk=%d, cch=%d)" % self.astuple()
+
+
+class TileInfo(Structure):
+    _fields_ = [("tile", Tile)] + [(n, c_int32) for n in (
+        "grid_x", "grid_y", "grid_z", "block_threads", "lds_bytes", "vgpr_estimate", "waves_per_simd",
+        "wg_per_cu", "nchunks")] + [(n, c_double) for n in ("flops", "bytes", "roof_us", "pred_us",
+                                                           "pred_hbm_bytes")]
+
+    def asdict(self):
+        d = {n: getattr(self, n) for n, _ in self._fields_ if n != "tile"}
+        d["tile"] = self.tile.astuple()
+        return d
+
+
+class TKConvDesc(Structure):
+    _fields_ = [(n, c_int32) for n in ("batch", "C", "R1", "R2", "N", "H", "W", "K", "stride", "pad", "dilation",
+                                       "has_bias", "relu")]
+
+
+_lib = None
+
+
+def lib():
+    """Load the shared library once; raise if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `python ppopp23-tdc_amd/build.py` "
+            "(hipcc, gfx950). There is no fallback implementation.")
+    L = ctypes.CDLL(LIB_PATH)
+    fp = POINTER(ctypes.c_float)
+    L.tdc_last_error_string.restype = c_char_p
+    L.tdc_version.restype = c_char_p
+    L.tdc_conv_plan_create.argtypes = [POINTER(ConvDesc), POINTER(Tile), POINTER(c_void_p)]
+    L.tdc_conv_plan_set_weights.argtypes = [c_void_p, c_void_p, c_void_p]
+    L.tdc_conv_plan_query.argtypes = [c_void_p, POINTER(TileInfo)]
+    L.tdc_conv_forward.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]
+    L.tdc_conv_plan_destroy.argtypes = [c_void_p]
+    L.tdc_conv_plan_destroy.restype = None
+    L.tdc_tkconv_create.argtypes = [POINTER(TKConvDesc), POINTER(c_void_p)]
+    L.tdc_tkconv_set_weights.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]
+    L.tdc_tkconv_forward.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]
+    L.tdc_tkconv_forward_features.argtypes = [c_void_p] * 6
+    L.tdc_tkconv_core_forward.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p]
+    L.tdc_tkconv_query.argtypes = [c_void_p, c_int, POINTER(TileInfo)]
+    L.tdc_tkconv_destroy.argtypes = [c_void_p]
+    L.tdc_tkconv_destroy.restype = None
+    L.tdc_model_evaluate.argtypes = [POINTER(ConvDesc), POINTER(Tile), POINTER(TileInfo)]
+    L.tdc_model_enumerate.argtypes = [POINTER(ConvDesc), POINTER(Tile), c_int32, POINTER(c_int32)]
+    L.tdc_model_select.argtypes = [POINTER(ConvDesc), POINTER(TileInfo)]
+    for name in EXPORTS:
+        fn = getattr(L, name)
+        if fn.restype is c_int:  # default restype: status code
+            fn.restype = c_int
+    _lib = L
+    return L
+
+
+def check(status):
+    if status != TDC_OK:
+        raise TdcError(status, lib().tdc_last_error_string().decode())
+
+
+def conv_desc(batch, C, N, H, W, KH, KW, stride=1, pad=0, dilation=1, has_bias=False, relu=False):
+    return ConvDesc(batch, C, N, H, W, KH, KW, stride, pad, dilation, int(has_bias), int(relu))
+
+
+# ---- analytic model (host only) ---------------------------------------------
+def model_select(desc: ConvDesc) -> TileInfo:
+    info = TileInfo()
+    check(lib().tdc_model_select(byref(desc), byref(info)))
+    return info
+
+
+def model_evaluate(desc: ConvDesc, tile: Tile) -> TileInfo:
+    info = TileInfo()
+    check(lib().tdc_model_evaluate(byref(desc), byref(tile), byref(info)))
+    return info
+
+
+def model_enumerate(desc: ConvDesc, cap: int = 8192):
+    arr = (Tile * cap)()
+    n = c_int32(0)
+    check(lib().tdc_model_enumerate(byref(desc), arr, cap, byref(n)))
+    return [Tile(*arr[i].astuple()) for i in range(n.value)]

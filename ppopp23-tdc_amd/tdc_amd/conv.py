@@ -1,0 +1,164 @@
+"""Host objects over the C ABI.  torch is used for device memory and streams only."""
+from __future__ import annotations
+
+from ctypes import byref, c_void_p
+
+import torch
+
+from . import _lib
+from ._lib import ConvDesc, Tile, TileInfo, TKConvDesc, check, lib
+
+
+def _stream_ptr():
+    return c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _host_f32(t):
+    if t is None:
+        return None
+    return t.detach().to(device="cpu", dtype=torch.float32).contiguous()
+
+
+def _dev_check(t, shape, what):
+    if not t.is_cuda:
+        raise ValueError(f"{what} must be a device tensor")
+    if t.dtype != torch.float32:
+        raise TypeError(f"{what} must be float32")
+    if tuple(t.shape) != tuple(shape):
+        raise ValueError(f"{what} has shape {tuple(t.shape)}, expected {tuple(shape)}")
+    if not t.is_contiguous():
+        raise ValueError(f"{what} must be contiguous NCHW")
+
+
+class Conv2dPlan:
+    """One convolution (optionally + bias, + residual, ReLU) on the GPU.
+
+    Counterpart of the reference's native ``Conv`` object
+    (2080Ti-evaluation/EndToEnd/resnet18-tk/inc/common.h:38-69): ``initialize``
+    = constructor + ``set_weights``; ``forward`` takes/returns device tensors.
+    """
+
+    def __init__(self, batch, C, N, H, W, KH, KW, stride=1, pad=0, dilation=1, bias=False, relu=False, tile=None):
+        self.desc = _lib.conv_desc(batch, C, N, H, W, KH, KW, stride, pad, dilation, bias, relu)
+        self._h = c_void_p()
+        tptr = byref(tile) if tile is not None else None
+        check(lib().tdc_conv_plan_create(byref(self.desc), tptr, byref(self._h)))
+        self.info = TileInfo()
+        check(lib().tdc_conv_plan_query(self._h, byref(self.info)))
+        self.Ho = _out_dim(H, KH, stride, pad, dilation)
+        self.Wo = _out_dim(W, KW, stride, pad, dilation)
+
+    def set_weights(self, weight, bias=None):
+        d = self.desc
+        w = _host_f32(weight)
+        if tuple(w.shape) != (d.N, d.C, d.KH, d.KW):
+            raise ValueError(f"weight has shape {tuple(w.shape)}, expected {(d.N, d.C, d.KH, d.KW)}")
+        b = _host_f32(bias)
+        if b is not None and tuple(b.shape) != (d.N,):
+            raise ValueError("bias must have shape [N]")
+        check(lib().tdc_conv_plan_set_weights(self._h, c_void_p(w.data_ptr()),
+                                              c_void_p(b.data_ptr()) if b is not None else None))
+        return self
+
+    def forward(self, x, residual=None, out=None):
+        d = self.desc
+        _dev_check(x, (d.batch, d.C, d.H, d.W), "input")
+        oshape = (d.batch, d.N, self.Ho, self.Wo)
+        if out is None:
+            out = torch.empty(oshape, device=x.device, dtype=torch.float32)
+        else:
+            _dev_check(out, oshape, "out")
+        rp = None
+        if residual is not None:
+            _dev_check(residual, oshape, "residual")
+            rp = c_void_p(residual.data_ptr())
+        check(lib().tdc_conv_forward(self._h, c_void_p(x.data_ptr()), rp, c_void_p(out.data_ptr()), _stream_ptr()))
+        return out
+
+    __call__ = forward
+
+    def close(self):
+        if self._h:
+            lib().tdc_conv_plan_destroy(self._h)
+            self._h = c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def _out_dim(n, k, stride, pad, dil):
+    return (n + 2 * pad - dil * (k - 1) - 1) // stride + 1
+
+
+class TKConvOp:
+    """Handle on a native tdc_tkconv (1x1 -> KxK core -> 1x1) for a fixed input shape."""
+
+    def __init__(self, batch, C, R1, R2, N, H, W, K, stride=1, pad=0, dilation=1, bias=False, relu=False):
+        self.desc = TKConvDesc(batch, C, R1, R2, N, H, W, K, stride, pad, dilation, int(bias), int(relu))
+        self._h = c_void_p()
+        check(lib().tdc_tkconv_create(byref(self.desc), byref(self._h)))
+        self.Ho = _out_dim(H, K, stride, pad, dilation)
+        self.Wo = _out_dim(W, K, stride, pad, dilation)
+
+    def set_weights(self, first, core, last, bias=None):
+        d = self.desc
+        f, c, l, b = _host_f32(first), _host_f32(core), _host_f32(last), _host_f32(bias)
+        if tuple(f.shape) != (d.R1, d.C, 1, 1) or tuple(c.shape) != (d.R2, d.R1, d.K, d.K) \
+                or tuple(l.shape) != (d.N, d.R2, 1, 1):
+            raise ValueError("factor/core kernel shapes do not match the descriptor")
+        check(lib().tdc_tkconv_set_weights(self._h, c_void_p(f.data_ptr()), c_void_p(c.data_ptr()),
+                                           c_void_p(l.data_ptr()),
+                                           c_void_p(b.data_ptr()) if b is not None else None))
+        return self
+
+    def forward(self, x, residual=None, out=None):
+        d = self.desc
+        _dev_check(x, (d.batch, d.C, d.H, d.W), "input")
+        oshape = (d.batch, d.N, self.Ho, self.Wo)
+        if out is None:
+            out = torch.empty(oshape, device=x.device, dtype=torch.float32)
+        else:
+            _dev_check(out, oshape, "out")
+        rp = None
+        if residual is not None:
+            _dev_check(residual, oshape, "residual")
+            rp = c_void_p(residual.data_ptr())
+        check(lib().tdc_tkconv_forward(self._h, c_void_p(x.data_ptr()), rp, c_void_p(out.data_ptr()), _stream_ptr()))
+        return out
+
+    def forward_features(self, x):
+        d = self.desc
+        _dev_check(x, (d.batch, d.C, d.H, d.W), "input")
+        f1 = torch.empty((d.batch, d.R1, d.H, d.W), device=x.device, dtype=torch.float32)
+        f2 = torch.empty((d.batch, d.R2, self.Ho, self.Wo), device=x.device, dtype=torch.float32)
+        out = torch.empty((d.batch, d.N, self.Ho, self.Wo), device=x.device, dtype=torch.float32)
+        check(lib().tdc_tkconv_forward_features(self._h, c_void_p(x.data_ptr()), c_void_p(f1.data_ptr()),
+                                                c_void_p(f2.data_ptr()), c_void_p(out.data_ptr()), _stream_ptr()))
+        return out, [f1, f2, out]
+
+    def core_forward(self, x, out=None):
+        d = self.desc
+        _dev_check(x, (d.batch, d.R1, d.H, d.W), "core input")
+        if out is None:
+            out = torch.empty((d.batch, d.R2, self.Ho, self.Wo), device=x.device, dtype=torch.float32)
+        check(lib().tdc_tkconv_core_forward(self._h, c_void_p(x.data_ptr()), c_void_p(out.data_ptr()), _stream_ptr()))
+        return out
+
+    def query(self, which):
+        info = TileInfo()
+        check(lib().tdc_tkconv_query(self._h, which, byref(info)))
+        return info
+
+    def close(self):
+        if self._h:
+            lib().tdc_tkconv_destroy(self._h)
+            self._h = c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

@@ -1,0 +1,167 @@
+"""GPU parity of the single-convolution entry points (tdc_conv_*) against the CPU oracle."""
+import math
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import tdc_amd
+from oracle import ref
+from util import assert_close, seeded
+
+pytestmark = pytest.mark.gpu
+
+
+def run_conv(x, w, bias=None, resid=None, stride=1, pad=0, dil=1, relu=False, tile=None):
+    B, C, H, W = x.shape
+    N, _, KH, KW = w.shape
+    plan = tdc_amd.Conv2dPlan(B, C, N, H, W, KH, KW, stride, pad, dil, bias is not None, relu, tile=tile)
+    plan.set_weights(w, bias)
+    out = torch.full((B, N, plan.Ho, plan.Wo), float("nan"), device="cuda")  # never pre-zeroed
+    plan.forward(x.cuda(), None if resid is None else resid.cuda(), out=out)
+    torch.cuda.synchronize()
+    res = out.cpu().numpy()
+    plan.close()
+    return res
+
+
+def case(seed, B, C, N, H, W, K):
+    g = seeded(seed)
+    x = torch.rand(B, C, H, W, generator=g) * 2 - 1
+    w = torch.empty(N, C, K, K).normal_(0, math.sqrt(2.0 / (C * K * K)), generator=g)
+    return x, w
+
+
+def announce(*a):
+    print(*a, flush=True)
+    sys.stdout.flush()
+
+
+def test_config1_core_conv_model_tile():
+    """Benchmark configuration 1: 1x32x56x56, 32x32x3x3, stride 1, pad 1, seed 0."""
+    x, w = ref.make_core_case(56, 32, 32, seed=0)
+    got = run_conv(x, w, pad=1)
+    assert_close(got, ref.conv2d_c(x.numpy(), w.numpy(), pad=1), "config 1 vs C oracle")
+    assert_close(got, ref.conv2d_torch(x, w, pad=1).numpy(), "config 1 vs F.conv2d")
+
+
+@pytest.mark.parametrize("hw", ref.SWEEP_HW)
+@pytest.mark.parametrize("r1,r2", ref.SWEEP_RANKS)
+def test_sweep_shapes_model_tile(hw, r1, r2):
+    """Every shape of the core-conv sweep with the model's tile, against F.conv2d (and the C oracle when small)."""
+    announce("sweep", hw, r1, r2)
+    x, w = ref.make_core_case(hw, r1, r2)
+    got = run_conv(x, w, pad=1)
+    assert_close(got, ref.conv2d_torch(x, w, pad=1).numpy(), f"sweep {hw} {r1}->{r2} vs F.conv2d")
+    if hw * hw * r1 * r2 <= 28 * 28 * 64 * 64:
+        assert_close(got, ref.conv2d_c(x.numpy(), w.numpy(), pad=1), f"sweep {hw} {r1}->{r2} vs C oracle")
+
+
+@pytest.mark.parametrize("shape", [(1, 8, 8, 5, 5), (1, 5, 3, 4, 7), (2, 3, 17, 9, 6), (1, 40, 24, 14, 14),
+                                   (1, 32, 32, 7, 7), (1, 20, 33, 13, 11)])
+def test_every_tile_3x3(shape):
+    """All launchable tiles give the oracle's answer (the reference's recorded sweeps show diff = 0 for every tile)."""
+    B, C, N, H, W = shape
+    x, w = case(1000 + C * N + H, B, C, N, H, W, 3)
+    want = ref.conv2d_c(x.numpy(), w.numpy(), pad=1)
+    tiles = tdc_amd.model_enumerate(tdc_amd.conv_desc(B, C, N, H, W, 3, 3, 1, 1))
+    assert tiles
+    for t in tiles:
+        announce("tile3x3", shape, t)
+        assert_close(run_conv(x, w, pad=1, tile=t), want, f"{shape} {t}")
+
+
+@pytest.mark.parametrize("shape", [(1, 16, 8, 5, 5), (1, 7, 5, 9, 4), (2, 64, 48, 7, 7), (1, 100, 36, 14, 14)])
+def test_every_tile_1x1(shape):
+    B, C, N, H, W = shape
+    x, w = case(2000 + C * N + H, B, C, N, H, W, 1)
+    want = ref.conv2d_c(x.numpy(), w.numpy())
+    tiles = tdc_amd.model_enumerate(tdc_amd.conv_desc(B, C, N, H, W, 1, 1, 1, 0))
+    assert tiles
+    for t in tiles:
+        announce("tile1x1", shape, t)
+        assert_close(run_conv(x, w, tile=t), want, f"{shape} {t}")
+
+
+@pytest.mark.parametrize("K,stride,pad,dil", [(3, 2, 1, 1), (3, 1, 0, 1), (3, 1, 2, 2), (5, 1, 2, 1), (7, 2, 3, 1),
+                                              (1, 2, 0, 1), (2, 1, 1, 1), (3, 3, 1, 1)])
+def test_general_filters(K, stride, pad, dil):
+    """Stride, padding, dilation and filter sizes beyond the 3x3/s1/p1 core conv."""
+    x, w = case(3000 + K * 10 + stride, 1, 6, 10, 15, 12, K)
+    want = ref.conv2d_c(x.numpy(), w.numpy(), stride=stride, pad=pad, dil=dil)
+    tiles = tdc_amd.model_enumerate(tdc_amd.conv_desc(1, 6, 10, 15, 12, K, K, stride, pad, dil))
+    for t in tiles[::3]:
+        announce("general", K, stride, pad, dil, t)
+        assert_close(run_conv(x, w, stride=stride, pad=pad, dil=dil, tile=t), want, f"K{K} s{stride} p{pad} d{dil} {t}")
+
+
+def test_stride2_resnet_core_shapes():
+    """The three stride-2 core convs of Tucker ResNet-18 (64->64 56->28, 128->128 28->14, 256->256 14->7)."""
+    for r, hw in ((64, 56), (128, 28), (256, 14)):
+        announce("stride2", r, hw)
+        x, w = case(4000 + r, 1, r, r, hw, hw, 3)
+        got = run_conv(x, w, stride=2, pad=1)
+        want = ref.conv2d_torch(x, w, stride=2, pad=1).numpy()
+        assert got.shape == (1, r, hw // 2, hw // 2)
+        assert_close(got, want, f"stride-2 {r}@{hw}")
+        # conv_s2(x) == conv_s1(x)[::2, ::2]
+        full = run_conv(x, w, stride=1, pad=1)
+        assert_close(got, full[:, :, ::2, ::2], "stride-2 subsampling identity")
+
+
+def test_epilogue_bias_residual_relu():
+    x, w = case(5000, 2, 12, 20, 9, 9, 3)
+    g = seeded(5001)
+    bias = torch.randn(20, generator=g)
+    resid = torch.randn(2, 20, 9, 9, generator=g)
+    want = ref.conv2d_c(x.numpy(), w.numpy(), bias.numpy(), resid.numpy(), pad=1, relu=True)
+    for t in tdc_amd.model_enumerate(tdc_amd.conv_desc(2, 12, 20, 9, 9, 3, 3, 1, 1))[::5]:
+        announce("epilogue", t)
+        assert_close(run_conv(x, w, bias, resid, pad=1, relu=True, tile=t), want, f"epilogue {t}")
+    assert (want == 0).any() and (want > 0).any()
+
+
+def test_reference_known_answer_integers_all_ones():
+    """The reference harness's own check: integer inputs 0..9, all-ones weights -> exact integers, diff == 0
+    (2080Ti-evaluation/TDC-LAYERS-ORACLE/template_benchmark_cudnn.template:418-428,509)."""
+    rng = np.random.default_rng(7)
+    for (C, N, H, W) in ((32, 32, 56, 56), (64, 32, 28, 28), (96, 64, 7, 7), (192, 160, 7, 7), (32, 32, 14, 14)):
+        announce("kat", C, N, H, W)
+        x = torch.from_numpy(rng.integers(0, 10, size=(1, C, H, W)).astype(np.float32))
+        w = torch.ones(N, C, 3, 3)
+        got = run_conv(x, w, pad=1)
+        # closed form: 3x3 box sum of the channel-summed image, identical for every output channel
+        s = np.pad(x.numpy().sum(axis=1)[0].astype(np.float64), 1)
+        box = sum(s[r:r + H, c:c + W] for r in range(3) for c in range(3))
+        assert np.abs(got - box[None, None]).sum() == 0.0
+
+
+def test_deterministic_bitwise():
+    x, w = ref.make_core_case(28, 64, 64)
+    a = run_conv(x, w, pad=1)
+    b = run_conv(x, w, pad=1)
+    assert np.array_equal(a, b)
+
+
+def test_linearity_full_size():
+    """Size-independent property at the largest sweep shape: conv(a*x1 + x2) == a*conv(x1) + conv(x2)."""
+    x1, w = ref.make_core_case(56, 128, 128)
+    x2, _ = ref.make_core_case(56, 128, 128, seed=99)
+    y1 = run_conv(x1, w, pad=1)
+    y2 = run_conv(x2, w, pad=1)
+    y = run_conv(0.5 * x1 + x2, w, pad=1)
+    np.testing.assert_allclose(y, 0.5 * y1 + y2, rtol=1e-4, atol=2e-5)
+
+
+def test_errors():
+    with pytest.raises(tdc_amd.TdcError):
+        tdc_amd.Conv2dPlan(1, 4, 4, 2, 2, 5, 5, 1, 0)  # filter larger than input
+    plan = tdc_amd.Conv2dPlan(1, 4, 4, 6, 6, 3, 3, 1, 1)
+    with pytest.raises(tdc_amd.TdcError):  # forward before weights
+        plan.forward(torch.zeros(1, 4, 6, 6, device="cuda"))
+    with pytest.raises(ValueError):
+        plan.set_weights(torch.zeros(4, 4, 1, 1))
+    bad = tdc_amd.Tile(32, 1, 1, 1, 1, 1, 3)  # cch not a multiple of kc
+    with pytest.raises(tdc_amd.TdcError):
+        tdc_amd.Conv2dPlan(1, 4, 4, 6, 6, 3, 3, 1, 1, tile=bad)
