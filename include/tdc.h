@@ -106,6 +106,15 @@ int tdc_conv_plan_query(const tdc_conv_plan *plan, tdc_tile_info *info_out);
 /* d_residual may be NULL.  Output need not be pre-zeroed.  Asynchronous. */
 int tdc_conv_forward(tdc_conv_plan *plan, const float *d_in, const float *d_residual,
                      float *d_out, void *stream);
+/* Measurement helper (the reference times its kernel with one cudaEvent pair
+ * around a single cold launch, template_benchmark_cudnn.template:491-496): run
+ * `iters` back-to-back forwards on a private stream between two hipEvents
+ * recorded on that stream and return the elapsed device time of the whole batch
+ * in milliseconds.  With use_graph != 0 the launches are captured into one HIP
+ * graph and the timed region is a single replay of it, which removes host launch
+ * cost from the figure.  Synchronises the device before and after. */
+int tdc_conv_time(tdc_conv_plan *plan, const float *d_in, const float *d_residual, float *d_out,
+                  int32_t iters, int32_t use_graph, float *total_ms_out);
 void tdc_conv_plan_destroy(tdc_conv_plan *plan);
 
 /* ---- TKConv operator: 1x1 C->R1, KxK R1->R2 (stride/pad/dilation), 1x1 R2->N (+bias) */

@@ -70,47 +70,58 @@ struct Mfma<16> {
 
 enum : int { TAPS_GENERIC = 0, TAPS_1x1 = 1, TAPS_3x3 = 9 };
 
+template <int VW>
+struct VecOf;
+template <>
+struct VecOf<1> { using type = float; };
+template <>
+struct VecOf<2> { using type = float2; };
+template <>
+struct VecOf<4> { using type = float4; };
+
 // Copy input channels [c0, c0+CCH) x rows [iy0, iy0+nrows) into LDS as
-// [channel][row][RS] with zeros for the halo and for channels >= C.  One wave
-// handles one channel at a time; its lanes cover as many whole rows as fit in
-// 64 lanes (narrow images) or 64-column pieces of one row (wide images).
+// [channel][row][RS] with zeros for the halo and for channels >= C.  The slab is
+// walked as a flat list of VW-wide vectors (RS, PL, W and CS are multiples of
+// VW, so a vector is either all image or all halo); every thread issues U
+// unconditional, clamped loads before it writes anything, so a wave keeps U
+// global loads in flight instead of one.
+template <int VW>
 __device__ __forceinline__ void stage_chunk(const ConvKParams &p, const float *__restrict__ in,
                                             float *__restrict__ lds, int c0, int iy0, int nrows,
-                                            int wave, int nwaves, int lane) {
-    int rpp, lrow, lcol, cpasses;
-    bool lane_on;
-    if (p.RS <= 64) {
-        rpp = 64 / p.RS;
-        lrow = lane / p.RS;
-        lcol = lane - lrow * p.RS;
-        cpasses = 1;
-        lane_on = lane < rpp * p.RS;
-    } else {
-        rpp = 1;
-        lrow = 0;
-        lcol = lane;
-        cpasses = (p.RS + 63) >> 6;
-        lane_on = true;
-    }
-    const int HW = p.H * p.W;
-    for (int cl = wave; cl < p.CCH; cl += nwaves) {
-        const int c = c0 + cl;
-        const bool cok = c < p.C;
-        const float *src = in + (long long)(cok ? c : 0) * HW;
-        float *dst = lds + cl * p.CS;
-#pragma unroll 4
-        for (int rbase = 0; rbase < nrows; rbase += rpp) {
-            const int row = rbase + lrow;
+                                            int tid, int nthreads) {
+    using vec_t = typename VecOf<VW>::type;
+    constexpr int U = 4;
+    const int rsv = p.RS / VW;
+    const int per_ch = nrows * rsv;
+    const int total = p.CCH * per_ch;
+    const int plv = p.PL / VW;
+    const int wv = p.W / VW;
+    const vec_t *__restrict__ src = reinterpret_cast<const vec_t *>(in);
+    for (int base = tid; base < total; base += nthreads * U) {
+        vec_t v[U];
+        int dst[U];
+        bool inb[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int e = base + u * nthreads;
+            const int ee = e < total ? e : 0;
+            const int cl = ee / per_ch;
+            const int rem = ee - cl * per_ch;
+            const int row = rem / rsv;
+            const int xv = rem - row * rsv;
+            const int c = c0 + cl;
             const int iy = iy0 + row;
-            const bool rok = cok && iy >= 0 && iy < p.H;
-            for (int cp = 0; cp < cpasses; ++cp) {
-                const int col = lcol + (cp << 6);
-                const int ix = col - p.PL;
-                const bool active = lane_on && row < nrows && col < p.RS;
-                float v = 0.0f;
-                if (active && rok && ix >= 0 && ix < p.W) v = src[iy * p.W + ix];
-                if (active) dst[row * p.RS + col] = v;
-            }
+            const int ixv = xv - plv;
+            inb[u] = c < p.C && iy >= 0 && iy < p.H && ixv >= 0 && ixv < wv;
+            const int sidx = inb[u] ? (c * p.H + iy) * wv + ixv : 0;
+            v[u] = src[sidx];
+            dst[u] = e < total ? cl * p.CS + row * p.RS + xv * VW : -1;
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            vec_t val = v[u];
+            if (!inb[u]) val = vec_t{};
+            if (dst[u] >= 0) *reinterpret_cast<vec_t *>(lds + dst[u]) = val;
         }
     }
 }
@@ -121,12 +132,15 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
     using acc_t = typename M::acc_t;
     constexpr int KC = M::KC;
     constexpr int NACC = M::NACC;
-    extern __shared__ float lds[];
+    // K-steps fetched per weight prefetch: one channel group of a 3x3 filter,
+    // four channel groups of a 1x1 filter, a single step otherwise.
+    constexpr int G = (TAPS == TAPS_3x3) ? 9 : (TAPS == TAPS_1x1) ? 4 : 1;
+    extern __shared__ __align__(16) float lds[];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int nwaves = blockDim.x >> 6;
+    const int nthreads = blockDim.x;
     const int wk = wave % p.WK;
     const int wn = (wave / p.WK) % p.WN;
     const int wm = wave / (p.WK * p.WN);
@@ -146,6 +160,27 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
     const int iy0 = oy0 * p.stride - p.pad;
     const int nrows = (oy1 - oy0) * p.stride + (p.KH - 1) * p.dil + 1;
 
+    // Per-lane base of this wave's A-operand stream for each of its M blocks.
+    const int taps = (TAPS == TAPS_GENERIC) ? p.KH * p.KW : TAPS;
+    const float *__restrict__ wbase[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+        const int mblk = m0 / MF + wm * MB + mb;
+        wbase[mb] = p.wpk + ((long long)mblk * p.ncg_total) * taps * 64 + lane;
+    }
+    const int ncgw = p.CPW / KC;  // channel groups this wave consumes per LDS pass
+    // The wave's K-steps of pass `chunk` start at packed K-step index kfirst(chunk);
+    // a pass holds nkw of them, consumed G at a time.
+    const int nkw = ncgw * taps;
+    auto kfirst = [&](int chunk) { return ((chunk * p.CCH + wk * p.CPW) / KC) * taps; };
+
+    // First weights are requested before the input slab, so both fetches overlap.
+    float a_nxt[G][MB];
+#pragma unroll
+    for (int t = 0; t < G; ++t)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) a_nxt[t][mb] = wbase[mb][(long long)(kfirst(0) + t) * 64];
+
     // Per-lane LDS offset (floats) of tap (0,0), channel sub-index included.
     int boff[NB];
 #pragma unroll
@@ -158,15 +193,6 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
                    M::ksub(lane) * p.CS;
     }
 
-    // Per-lane base of this wave's A-operand stream for each of its M blocks.
-    const int taps = (TAPS == TAPS_GENERIC) ? p.KH * p.KW : TAPS;
-    const float *__restrict__ wbase[MB];
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb) {
-        const int mblk = m0 / MF + wm * MB + mb;
-        wbase[mb] = p.wpk + ((long long)mblk * p.ncg_total) * taps * 64 + lane;
-    }
-
     acc_t acc[MB][NB];
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
@@ -175,36 +201,34 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
 #pragma unroll
             for (int v = 0; v < NACC; ++v) acc[mb][nb][v] = 0.0f;
 
-    const int ncgw = p.CPW / KC;  // channel groups this wave consumes per LDS pass
     const float *lbase = lds + wk * p.CPW * p.CS;
 
     for (int chunk = 0; chunk < p.nchunks; ++chunk) {
         if (chunk > 0) __syncthreads();
-        stage_chunk(p, in, lds, chunk * p.CCH, iy0, nrows, wave, nwaves, lane);
+        if (p.VW == 4) stage_chunk<4>(p, in, lds, chunk * p.CCH, iy0, nrows, tid, nthreads);
+        else if (p.VW == 2) stage_chunk<2>(p, in, lds, chunk * p.CCH, iy0, nrows, tid, nthreads);
+        else stage_chunk<1>(p, in, lds, chunk * p.CCH, iy0, nrows, tid, nthreads);
         __syncthreads();
-        const int cg0 = (chunk * p.CCH + wk * p.CPW) / KC;
+        const int k0 = kfirst(chunk);
+        const int knext_chunk = kfirst(min(chunk + 1, p.nchunks - 1));
 
-        if constexpr (TAPS == TAPS_3x3) {
-            // One channel group (9 K-steps) per iteration; the next group's
-            // weights are requested before this group's MFMAs are issued.
-            float a_nxt[9][MB];
+        for (int k = 0; k < nkw; k += G) {
+            float a_cur[G][MB];
 #pragma unroll
-            for (int t = 0; t < 9; ++t)
+            for (int t = 0; t < G; ++t)
 #pragma unroll
-                for (int mb = 0; mb < MB; ++mb) a_nxt[t][mb] = wbase[mb][((long long)cg0 * 9 + t) * 64];
-            for (int cg = 0; cg < ncgw; ++cg) {
-                float a_cur[9][MB];
+                for (int mb = 0; mb < MB; ++mb) a_cur[t][mb] = a_nxt[t][mb];
+            // Next group of this pass, else the first group of the next pass,
+            // else (very last group) a harmless re-read of the current one.
+            int kn = k0 + k + G;
+            if (k + G >= nkw) kn = (chunk + 1 < p.nchunks) ? knext_chunk : k0 + k;
 #pragma unroll
-                for (int t = 0; t < 9; ++t)
+            for (int t = 0; t < G; ++t)
 #pragma unroll
-                    for (int mb = 0; mb < MB; ++mb) a_cur[t][mb] = a_nxt[t][mb];
-                const int cgn = cg0 + min(cg + 1, ncgw - 1);
-#pragma unroll
-                for (int t = 0; t < 9; ++t)
-#pragma unroll
-                    for (int mb = 0; mb < MB; ++mb)
-                        a_nxt[t][mb] = wbase[mb][((long long)cgn * 9 + t) * 64];
-                const float *lrow = lbase + cg * KC * p.CS;
+                for (int mb = 0; mb < MB; ++mb) a_nxt[t][mb] = wbase[mb][(long long)(kn + t) * 64];
+
+            if constexpr (TAPS == TAPS_3x3) {
+                const float *lrow = lbase + (k / 9) * KC * p.CS;
 #pragma unroll
                 for (int r = 0; r < 3; ++r) {
 #pragma unroll
@@ -220,31 +244,10 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
                                 acc[mb][nb] = M::run(a_cur[r * 3 + s][mb], b[nb], acc[mb][nb]);
                     }
                 }
-            }
-        } else if constexpr (TAPS == TAPS_1x1) {
-            // Four channel groups per iteration (ncgw is a multiple of 4 by
-            // construction of the tile), same one-iteration-ahead weight fetch.
-            constexpr int G = 4;
-            float a_nxt[G][MB];
-#pragma unroll
-            for (int t = 0; t < G; ++t)
-#pragma unroll
-                for (int mb = 0; mb < MB; ++mb) a_nxt[t][mb] = wbase[mb][((long long)cg0 + t) * 64];
-            for (int cg = 0; cg < ncgw; cg += G) {
-                float a_cur[G][MB];
-#pragma unroll
-                for (int t = 0; t < G; ++t)
-#pragma unroll
-                    for (int mb = 0; mb < MB; ++mb) a_cur[t][mb] = a_nxt[t][mb];
-                const int cgn = cg0 + min(cg + G, ncgw - G);
-#pragma unroll
-                for (int t = 0; t < G; ++t)
-#pragma unroll
-                    for (int mb = 0; mb < MB; ++mb)
-                        a_nxt[t][mb] = wbase[mb][((long long)cgn + t) * 64];
+            } else if constexpr (TAPS == TAPS_1x1) {
 #pragma unroll
                 for (int t = 0; t < G; ++t) {
-                    const float *lrow = lbase + (cg + t) * KC * p.CS;
+                    const float *lrow = lbase + (k + t) * KC * p.CS;
                     float b[NB];
 #pragma unroll
                     for (int nb = 0; nb < NB; ++nb) b[nb] = lrow[boff[nb]];
@@ -254,28 +257,21 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
                         for (int nb = 0; nb < NB; ++nb)
                             acc[mb][nb] = M::run(a_cur[t][mb], b[nb], acc[mb][nb]);
                 }
-            }
-        } else {
-            // Any filter size / dilation: taps walked at run time.
-            for (int cg = 0; cg < ncgw; ++cg) {
+            } else {
+                // Any filter size / dilation: decode the tap of this K-step.
+                const int cg = k / taps;
+                const int tap = k - cg * taps;
+                const int r = tap / p.KW;
+                const int s = tap - r * p.KW;
                 const float *lrow = lbase + cg * KC * p.CS;
-                int t = 0;
-                for (int r = 0; r < p.KH; ++r) {
-                    for (int s = 0; s < p.KW; ++s, ++t) {
-                        float a[MB], b[NB];
+                float b[NB];
 #pragma unroll
-                        for (int mb = 0; mb < MB; ++mb)
-                            a[mb] = wbase[mb][((long long)(cg0 + cg) * taps + t) * 64];
+                for (int nb = 0; nb < NB; ++nb) b[nb] = lrow[boff[nb] + r * p.dil * p.RS + s * p.dil];
 #pragma unroll
-                        for (int nb = 0; nb < NB; ++nb)
-                            b[nb] = lrow[boff[nb] + r * p.dil * p.RS + s * p.dil];
+                for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-                        for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-                            for (int nb = 0; nb < NB; ++nb)
-                                acc[mb][nb] = M::run(a[mb], b[nb], acc[mb][nb]);
-                    }
-                }
+                    for (int nb = 0; nb < NB; ++nb)
+                        acc[mb][nb] = M::run(a_cur[0][mb], b[nb], acc[mb][nb]);
             }
         }
     }
@@ -320,7 +316,7 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
         }
         __syncthreads();
         const int total = MT * PT;
-        for (int idx = tid; idx < total; idx += blockDim.x) {
+        for (int idx = tid; idx < total; idx += nthreads) {
             const int ml = idx / PT;
             const int pl = idx - ml * PT;
             const int n = m0 + ml;

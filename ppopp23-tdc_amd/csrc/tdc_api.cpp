@@ -167,12 +167,61 @@ int tdc_conv_forward(tdc_conv_plan *plan, const float *d_in, const float *d_resi
     kp.WM = plan->tile.wm; kp.WN = plan->tile.wn; kp.WK = plan->tile.wk;
     kp.CCH = plan->tile.cch; kp.nchunks = g.nchunks; kp.CPW = g.cpw;
     kp.RS = g.RS; kp.CS = g.CS; kp.PL = g.PL;
+    // Vector loads need the activations aligned to the vector size; fall back to scalars otherwise.
+    kp.VW = (reinterpret_cast<uintptr_t>(d_in) % (4 * g.VW) == 0) ? g.VW : 1;
     kp.relu = d.relu;
     kp.ncg_total = g.c_pad / g.kc;
     kp.in_bstride = (long long)d.C * d.H * d.W;
     kp.out_bstride = (long long)d.N * g.P;
     int he = launch_conv(plan->kernel, g, kp, stream);
     if (he) return hip_fail("kernel launch", he);
+    return TDC_OK;
+}
+
+int tdc_conv_time(tdc_conv_plan *plan, const float *d_in, const float *d_residual, float *d_out, int32_t iters,
+                  int32_t use_graph, float *total_ms_out) {
+    if (!plan || !total_ms_out || iters < 1) return fail(TDC_ERR_INVALID, "bad argument");
+    hipStream_t s = nullptr;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    int st = TDC_OK;
+    const char *what = "hipStreamCreate";
+    hipError_t e = hipDeviceSynchronize();
+    if (e == hipSuccess) e = hipStreamCreate(&s);
+    if (e == hipSuccess) { what = "hipEventCreate"; e = hipEventCreate(&e0); }
+    if (e == hipSuccess) e = hipEventCreate(&e1);
+    if (e == hipSuccess && use_graph) {
+        what = "graph capture";
+        e = hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal);
+        if (e == hipSuccess) {
+            for (int i = 0; i < iters && st == TDC_OK; ++i) st = tdc_conv_forward(plan, d_in, d_residual, d_out, s);
+            e = hipStreamEndCapture(s, &graph);
+        }
+        if (e == hipSuccess && st == TDC_OK) e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+        // One untimed replay so that the timed one does not pay for the upload.
+        if (e == hipSuccess && st == TDC_OK) e = hipGraphLaunch(exec, s);
+        if (e == hipSuccess && st == TDC_OK) e = hipStreamSynchronize(s);
+    }
+    if (e == hipSuccess && st == TDC_OK) {
+        what = "timed region";
+        e = hipEventRecord(e0, s);
+        if (use_graph) {
+            if (e == hipSuccess) e = hipGraphLaunch(exec, s);
+        } else {
+            for (int i = 0; i < iters && st == TDC_OK; ++i) st = tdc_conv_forward(plan, d_in, d_residual, d_out, s);
+        }
+        if (e == hipSuccess) e = hipEventRecord(e1, s);
+        if (e == hipSuccess) e = hipEventSynchronize(e1);
+        if (e == hipSuccess) e = hipEventElapsedTime(total_ms_out, e0, e1);
+    }
+    if (exec) (void)hipGraphExecDestroy(exec);
+    if (graph) (void)hipGraphDestroy(graph);
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    if (s) (void)hipStreamDestroy(s);
+    if (st != TDC_OK) return st;
+    if (e != hipSuccess) return hip_fail(what, e);
     return TDC_OK;
 }
 

@@ -38,7 +38,8 @@ struct Geometry {
     int nchunks = 0;                 // LDS passes
     int c_pad = 0;                   // nchunks * cch
     int n_pad = 0;                   // grid_y * MT (rows of the packed weights)
-    int PL = 0;                      // left zero columns in an LDS row
+    int VW = 1;                      // floats per vector of the LDS fill (4 if W%4==0, 2 if W%2==0)
+    int PL = 0;                      // left zero columns in an LDS row (multiple of VW, >= pad)
     int RS = 0;                      // LDS row stride (floats)
     int nrows = 0;                   // max input rows a workgroup stages
     int CS = 0;                      // LDS channel stride (floats)
@@ -75,6 +76,7 @@ struct ConvKParams {
     int WM, WN, WK;
     int CCH, nchunks, CPW;
     int RS, CS, PL;
+    int VW;               // vector width of the LDS fill (4, 2 or 1 floats)
     int relu;
     int ncg_total;        // c_pad / kc
     long long in_bstride;   // C*H*W

@@ -88,8 +88,11 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
     g.nchunks = ceil_div(d.C, t.cch);
     g.c_pad = g.nchunks * t.cch;
     g.n_pad = g.grid_y * g.MT;
-    g.PL = d.pad;
-    g.RS = d.W + 2 * d.pad;
+    // LDS rows are filled with VW-wide vectors: the left halo and the row stride
+    // are rounded up so that every image row starts on a vector boundary.
+    g.VW = (d.W % 4 == 0) ? 4 : (d.W % 2 == 0) ? 2 : 1;
+    g.PL = round_up(d.pad, g.VW);
+    g.RS = round_up(g.PL + d.W + d.pad, g.VW);
     int nrows = 0;
     for (int bx = 0; bx < g.grid_x; ++bx) {
         const int p0 = bx * g.PT;

@@ -77,6 +77,16 @@ class Conv2dPlan:
 
     __call__ = forward
 
+    def time_us(self, x, out, residual=None, iters=100, graph=True):
+        """Device microseconds per launch: hipEvents around `iters` back-to-back launches issued from C
+        (replayed from one HIP graph when `graph`)."""
+        import ctypes
+        ms = ctypes.c_float(0.0)
+        rp = c_void_p(residual.data_ptr()) if residual is not None else None
+        check(lib().tdc_conv_time(self._h, c_void_p(x.data_ptr()), rp, c_void_p(out.data_ptr()), iters,
+                                  int(graph), byref(ms)))
+        return ms.value * 1e3 / iters
+
     def close(self):
         if self._h:
             lib().tdc_conv_plan_destroy(self._h)

@@ -13,7 +13,7 @@ def assert_close(got, ref, what=""):
     assert got.shape == ref.shape, f"{what}: shape {got.shape} vs {ref.shape}"
     err = np.abs(got - ref)
     bound = ATOL + RTOL * np.abs(ref)
-    bad = err > bound
+    bad = ~(err <= bound)  # NaN counts as a mismatch
     if bad.any():
         i = np.unravel_index(np.argmax(err - bound), err.shape)
         raise AssertionError(f"{what}: {bad.sum()} of {bad.size} outside tolerance; worst at {i}: "
