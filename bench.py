@@ -1,0 +1,142 @@
+#!/usr/bin/env python3
+"""Benchmark of the Tucker core-conv hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One step = one pass over the 28-shape core-conv sweep (batch 1, fp32 NCHW, 3x3,
+stride 1, pad 1; H=W in {7,14,28,56} x (R1,R2) in {(16,16),(32,32),(64,64),(96,96),
+(128,128),(32,64),(64,128)}), one kernel launch per layer, inputs and packed
+weights resident in HBM.  Prints ONE JSON line: the mean device time per layer
+(us/layer), a per-layer table with each layer's fraction of its fp32/HBM
+roofline, the roofline of the dominant kernel (the 128->128 @56 layer) from HIP
+events on the launch stream, and the CPU baseline (the PyTorch-CPU convolution
+the reference operator executes) timed on this host's cores.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "ppopp23-tdc_amd"))
+sys.path.insert(0, ROOT)
+
+PEAK_FP32_TFLOPS = 157.3   # MI355X dense fp32 matrix peak
+PEAK_HBM_TBPS = 8.0
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-graph", action="store_true", help="issue launches on a plain stream instead of a HIP graph")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU; --gpus %d is not supported (single-GPU hot path, "
+                 "no collectives)." % a.gpus)
+
+    import torch
+    import tdc_amd
+    from tdc_amd.conv import Conv2dPlan, time_many_ms
+    from oracle import ref   # checker + cpu_baseline leg only
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    torch.cuda.set_device(0)
+    graph = not a.no_graph
+
+    layers = []
+    for hw in ref.SWEEP_HW:
+        for r1, r2 in ref.SWEEP_RANKS:
+            x, w = ref.make_core_case(hw, r1, r2)
+            plan = Conv2dPlan(1, r1, r2, hw, hw, 3, 3, 1, 1).set_weights(w)
+            xd = x.cuda()
+            out = torch.empty(1, r2, hw, hw, device="cuda")
+            layers.append({"hw": hw, "r1": r1, "r2": r2, "plan": plan, "x": xd, "out": out, "xc": x, "wc": w})
+    plans = [l["plan"] for l in layers]
+    xs = [l["x"] for l in layers]
+    outs = [l["out"] for l in layers]
+
+    # -- parity spot check (outside every timed region) -------------------------
+    for l in (layers[1], layers[-4]):
+        l["plan"].forward(l["x"], out=l["out"])
+        torch.cuda.synchronize()
+        want = ref.conv2d_torch(l["xc"], l["wc"], pad=1)
+        if not torch.allclose(l["out"].cpu(), want, rtol=1e-4, atol=1e-5):
+            sys.exit("bench.py: parity check failed for layer %s" % ((l["hw"], l["r1"], l["r2"]),))
+
+    # -- the timed region: W warm-up steps, then exactly K steps ------------------
+    if a.warmup > 0:
+        time_many_ms(plans, xs, outs, iters=a.warmup, graph=graph)
+    torch.cuda.synchronize()
+    t_wall0 = time.perf_counter()
+    total_ms = time_many_ms(plans, xs, outs, iters=a.steps, graph=graph)   # syncs before and after
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t_wall0) * 1e3
+    ms_per_step = total_ms / a.steps
+    us_per_layer = ms_per_step * 1e3 / len(layers)
+
+    # -- per-layer device time and roofline fraction ------------------------------
+    table = []
+    for l in layers:
+        info = l["plan"].info
+        us = min(l["plan"].time_us(l["x"], l["out"], iters=100, graph=graph) for _ in range(3))
+        table.append({"H": l["hw"], "R1": l["r1"], "R2": l["r2"], "us": round(us, 3),
+                      "roof_us": round(info.roof_us, 4), "frac": round(info.roof_us / us, 4),
+                      "gflops": round(info.flops / us * 1e-3, 1), "tile": list(info.tile.astuple())})
+
+    # -- dominant kernel: the largest layer of the sweep --------------------------
+    dom = max(range(len(layers)), key=lambda i: table[i]["us"])
+    dl, dinfo = layers[dom], layers[dom]["plan"].info
+    dom_us = sum(dl["plan"].time_us(dl["x"], dl["out"], iters=200, graph=graph) for _ in range(3)) / 3
+    mfma_bound = dinfo.flops / (PEAK_FP32_TFLOPS * 1e6) >= dinfo.bytes / (PEAK_HBM_TBPS * 1e6)
+    if mfma_bound:
+        achieved = dinfo.flops / dom_us * 1e-6     # TFLOP/s
+        roofline = {"bound": "mfma", "achieved": round(achieved, 3), "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
+                    "frac": round(achieved / PEAK_FP32_TFLOPS, 4), "traffic": None}
+    else:
+        achieved = dinfo.bytes / dom_us * 1e-3     # GB/s
+        roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_TBPS * 1e3, "unit": "GB/s",
+                    "frac": round(achieved / (PEAK_HBM_TBPS * 1e3), 4), "traffic": None}
+    roofline.update({"kernel": "core conv %d->%d @%dx%d" % (dl["r1"], dl["r2"], dl["hw"], dl["hw"]),
+                     "avg_launch_us": round(dom_us, 3), "flops_per_launch": dinfo.flops,
+                     "bytes_per_launch": dinfo.bytes, "timing": "hipEvents around 200 graph-replayed launches"})
+
+    out = {
+        "metric": "core_conv_us_per_layer", "value": round(us_per_layer, 4), "unit": "us/layer",
+        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "core-conv sweep: 28 layers, batch 1, fp32 NCHW, 3x3 s1 p1, H=W in {7,14,28,56} x "
+                               "7 rank pairs; one step = one pass over all 28 layers",
+                   "launch": "HIP graph replay" if graph else "stream launches", "layers_per_step": len(layers)},
+        "roofline": roofline,
+        "geomean_frac": round(float(torch.tensor([t["frac"] for t in table]).log().mean().exp()), 4),
+        "layers": table,
+        "host_wall_ms_timed_region": round(wall_ms, 3),
+    }
+
+    # -- CPU baseline: the reference operator's CPU path (F.conv2d), same layers --
+    if not a.no_cpu_baseline:
+        torch.set_num_threads(os.cpu_count() or 1)
+        import torch.nn.functional as F
+        with torch.no_grad():
+            for l in layers:
+                F.conv2d(l["xc"], l["wc"], None, 1, 1)
+            passes, t0 = 0, time.perf_counter()
+            while time.perf_counter() - t0 < 10.0:
+                for l in layers:
+                    ref.conv2d_torch(l["xc"], l["wc"], pad=1)
+                passes += 1
+            cpu_s = time.perf_counter() - t0
+        out["cpu_baseline"] = {"value": round(cpu_s * 1e6 / (passes * len(layers)), 2), "unit": "us/layer",
+                               "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": "%d passes over the same 28 layers with torch.nn.functional.conv2d fp32 on "
+                                         "the host (the call the reference operator makes on CPU), ~10 s" % passes}
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -115,6 +115,11 @@ int tdc_conv_forward(tdc_conv_plan *plan, const float *d_in, const float *d_resi
  * cost from the figure.  Synchronises the device before and after. */
 int tdc_conv_time(tdc_conv_plan *plan, const float *d_in, const float *d_residual, float *d_out,
                   int32_t iters, int32_t use_graph, float *total_ms_out);
+/* Same for a list of plans run one after the other: one pass over the `n`
+ * plans is one step; the timed region holds `iters` steps (each step one replay of
+ * a HIP graph of the n launches when use_graph != 0). */
+int tdc_conv_time_many(tdc_conv_plan *const *plans, const float *const *d_ins, float *const *d_outs,
+                       int32_t n, int32_t iters, int32_t use_graph, float *total_ms_out);
 void tdc_conv_plan_destroy(tdc_conv_plan *plan);
 
 /* ---- TKConv operator: 1x1 C->R1, KxK R1->R2 (stride/pad/dilation), 1x1 R2->N (+bias) */

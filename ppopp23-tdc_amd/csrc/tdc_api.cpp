@@ -178,6 +178,57 @@ int tdc_conv_forward(tdc_conv_plan *plan, const float *d_in, const float *d_resi
     return TDC_OK;
 }
 
+int tdc_conv_time_many(tdc_conv_plan *const *plans, const float *const *d_ins, float *const *d_outs, int32_t n,
+                       int32_t iters, int32_t use_graph, float *total_ms_out) {
+    if (!plans || !d_ins || !d_outs || !total_ms_out || n < 1 || iters < 1) return fail(TDC_ERR_INVALID, "bad argument");
+    for (int i = 0; i < n; ++i)
+        if (!plans[i] || !d_ins[i] || !d_outs[i]) return fail(TDC_ERR_INVALID, "null plan or buffer in list");
+    hipStream_t s = nullptr;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    int st = TDC_OK;
+    auto one_pass = [&]() {
+        for (int i = 0; i < n && st == TDC_OK; ++i) st = tdc_conv_forward(plans[i], d_ins[i], nullptr, d_outs[i], s);
+    };
+    const char *what = "hipStreamCreate";
+    hipError_t e = hipDeviceSynchronize();
+    if (e == hipSuccess) e = hipStreamCreate(&s);
+    if (e == hipSuccess) { what = "hipEventCreate"; e = hipEventCreate(&e0); }
+    if (e == hipSuccess) e = hipEventCreate(&e1);
+    if (e == hipSuccess && use_graph) {
+        // One pass over the list is one graph; the timed region replays it `iters` times.
+        what = "graph capture";
+        e = hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal);
+        if (e == hipSuccess) {
+            one_pass();
+            e = hipStreamEndCapture(s, &graph);
+        }
+        if (e == hipSuccess && st == TDC_OK) e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+        if (e == hipSuccess && st == TDC_OK) e = hipGraphLaunch(exec, s);  // untimed: upload
+        if (e == hipSuccess && st == TDC_OK) e = hipStreamSynchronize(s);
+    }
+    if (e == hipSuccess && st == TDC_OK) {
+        what = "timed region";
+        e = hipEventRecord(e0, s);
+        for (int it = 0; it < iters && st == TDC_OK && e == hipSuccess; ++it) {
+            if (use_graph) e = hipGraphLaunch(exec, s);
+            else one_pass();
+        }
+        if (e == hipSuccess) e = hipEventRecord(e1, s);
+        if (e == hipSuccess) e = hipEventSynchronize(e1);
+        if (e == hipSuccess) e = hipEventElapsedTime(total_ms_out, e0, e1);
+    }
+    if (exec) (void)hipGraphExecDestroy(exec);
+    if (graph) (void)hipGraphDestroy(graph);
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    if (s) (void)hipStreamDestroy(s);
+    if (st != TDC_OK) return st;
+    if (e != hipSuccess) return hip_fail(what, e);
+    return TDC_OK;
+}
+
 int tdc_conv_time(tdc_conv_plan *plan, const float *d_in, const float *d_residual, float *d_out, int32_t iters,
                   int32_t use_graph, float *total_ms_out) {
     if (!plan || !total_ms_out || iters < 1) return fail(TDC_ERR_INVALID, "bad argument");

@@ -18,7 +18,7 @@ TDC_OK, TDC_ERR_INVALID, TDC_ERR_UNSUPPORTED, TDC_ERR_HIP, TDC_ERR_NOMEM, TDC_ER
 EXPORTS = (
     "tdc_last_error_string", "tdc_version",
     "tdc_conv_plan_create", "tdc_conv_plan_set_weights", "tdc_conv_plan_query", "tdc_conv_forward",
-    "tdc_conv_time", "tdc_conv_plan_destroy",
+    "tdc_conv_time", "tdc_conv_time_many", "tdc_conv_plan_destroy",
     "tdc_tkconv_create", "tdc_tkconv_set_weights", "tdc_tkconv_forward", "tdc_tkconv_forward_features",
     "tdc_tkconv_core_forward", "tdc_tkconv_query", "tdc_tkconv_destroy",
     "tdc_model_evaluate", "tdc_model_enumerate", "tdc_model_select",
@@ -84,6 +84,8 @@ def lib():
     L.tdc_conv_plan_query.argtypes = [c_void_p, POINTER(TileInfo)]
     L.tdc_conv_forward.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]
     L.tdc_conv_time.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, POINTER(ctypes.c_float)]
+    L.tdc_conv_time_many.argtypes = [POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p), c_int32, c_int32, c_int32,
+                                     POINTER(ctypes.c_float)]
     L.tdc_conv_plan_destroy.argtypes = [c_void_p]
     L.tdc_conv_plan_destroy.restype = None
     L.tdc_tkconv_create.argtypes = [POINTER(TKConvDesc), POINTER(c_void_p)]

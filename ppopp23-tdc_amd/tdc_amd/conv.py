@@ -99,6 +99,18 @@ class Conv2dPlan:
             pass
 
 
+def time_many_ms(plans, xs, outs, iters=1, graph=True):
+    """Device milliseconds of `iters` passes over the list of (plan, input, output), launched from C."""
+    import ctypes
+    n = len(plans)
+    P = (c_void_p * n)(*[p._h for p in plans])
+    X = (c_void_p * n)(*[c_void_p(x.data_ptr()) for x in xs])
+    O = (c_void_p * n)(*[c_void_p(o.data_ptr()) for o in outs])
+    ms = ctypes.c_float(0.0)
+    check(lib().tdc_conv_time_many(P, X, O, n, iters, int(graph), byref(ms)))
+    return ms.value
+
+
 def _out_dim(n, k, stride, pad, dil):
     return (n + 2 * pad - dil * (k - 1) - 1) // stride + 1
 
