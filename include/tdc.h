@@ -60,9 +60,10 @@ typedef struct tdc_conv_desc {
 } tdc_conv_desc;
 
 /* Tiling of one convolution on the gfx950 compute unit.  One workgroup computes
- * an (mf*mb*wm) output-channel x (mf*nb*wn) flat-pixel tile; its wm*wn*wk
+ * (mf*mb*wm) output channels of a th x tw tile of output pixels (th is derived:
+ * as many rows as fit in the workgroup's mf*nb*wn pixel lanes); its wm*wn*wk
  * wavefronts split output channels, pixels and input channels; input channels
- * are staged through LDS `cch` at a time. */
+ * are staged through LDS `cch` at a time, double-buffered. */
 typedef struct tdc_tile {
     int32_t mf;   /* MFMA block edge: 32 (v_mfma_f32_32x32x2_f32) or 16 (16x16x4) */
     int32_t mb;   /* MFMA blocks per wave along output channels (1 or 2)        */
@@ -71,6 +72,7 @@ typedef struct tdc_tile {
     int32_t wn;   /* waves along pixels                                        */
     int32_t wk;   /* waves along input channels (in-workgroup split-K)          */
     int32_t cch;  /* input channels staged in LDS per pass                      */
+    int32_t tw;   /* output tile width in pixels                               */
 } tdc_tile;
 
 typedef struct tdc_tile_info {
@@ -82,11 +84,12 @@ typedef struct tdc_tile_info {
     int32_t waves_per_simd;          /* resident, limited by VGPR/LDS/slots    */
     int32_t wg_per_cu;
     int32_t nchunks;                 /* LDS passes over input channels         */
+    int32_t th;                      /* output tile height in pixels           */
     double flops;                    /* algorithmic 2*Ho*Wo*C*N*KH*KW*batch    */
     double bytes;                    /* algorithmic: in + out + weights once   */
     double roof_us;                  /* max(bytes/8TB/s, flops/157.3TF)        */
     double pred_us;                  /* analytic model's predicted device time */
-    double pred_hbm_bytes;           /* modelled L2->CU traffic (re-reads incl.) */
+    double pred_l2_bytes;            /* modelled L2->LDS copy traffic (halo and re-reads included) */
 } tdc_tile_info;
 
 typedef struct tdc_conv_plan tdc_conv_plan;

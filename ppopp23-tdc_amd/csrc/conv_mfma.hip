@@ -1,28 +1,37 @@
 // Direct convolution as an implicit GEMM on the gfx950 fp32 matrix cores.
 //
-//   out[n][p] = sum_{c,r,s} w[n][c][r][s] * in[c][iy(p,r)][ix(p,s)]
+//   out[n][oy][ox] = sum_{c,r,s} w[n][c][r][s] * in[c][oy*stride-pad+r*dil][ox*stride-pad+s*dil]
 //
-// is computed as  D[M = out channels][N = flat output pixels] += A[M][K] * B[K][N]
-// with K running over (input channel, filter tap).  A (weights) is pre-packed on
-// the host in exactly the per-lane order the MFMA instruction wants and is
-// streamed from L2 with one coalesced 256-byte load per wave per K-step.  B
-// (input) is staged once per workgroup into LDS as raw rows with a zero halo
-// ([channel][row][col], the same slab-plus-halo idea as the reference's
-// load_input_2_shared_memory, 2080Ti-evaluation/TDC-LAYERS-ORACLE/
-// template_benchmark_cudnn.template:340-363,377-389), and each K-step reads it
-// with one conflict-free ds_read_b32: the 32 (or 16) pixel lanes of an MFMA
-// column block read consecutive words of one row, shifted by the tap.
+// is computed as  D[M = out channels][N = output pixels] += A[M][K] * B[K][N]
+// with K running over (input channel, filter tap).
+//
+// One workgroup owns a TH x TW tile of output pixels and MT output channels.
+// Input channels are consumed CCH at a time.  For every such pass the
+// workgroup needs (a) the input window of its tile, [CCH][rows][cols] with a
+// zero halo — the slab-plus-halo idea of the reference's
+// load_input_2_shared_memory (2080Ti-evaluation/TDC-LAYERS-ORACLE/
+// template_benchmark_cudnn.template:340-363,377-389) — and (b) the weights of
+// its MT output channels for those CCH channels, pre-packed on the host in the
+// per-lane order the MFMA A operand wants.  Both are copied global -> LDS by
+// the buffer unit itself (`buffer_load_dwordx4 ... lds`): no register is
+// involved, every wave fires all its copies of a pass at once, and lanes that
+// fall on halo or padding present an out-of-range offset, which the hardware
+// answers with zeros.  Two LDS stages alternate: while the MFMAs of pass i run
+// out of one stage, the copies of pass i+1 land in the other.
+//
+// Each K-step is then two conflict-free ds_read_b32 (A: 64 consecutive words,
+// B: the pixel lanes of a tile row read consecutive words, shifted by the tap)
+// and MB*NB MFMAs.
 //
 // Differences from the reference kernel (template_benchmark_cudnn.template:365-402):
-//   * lanes index PIXELS (coalesced stores, conflict-free LDS), output channels
-//     live in the MFMA accumulator rows; the reference maps lane -> channel and
-//     broadcasts one LDS word to the whole warp;
+//   * lanes index PIXELS, output channels live in the MFMA accumulator rows; the
+//     reference maps lane -> channel and broadcasts one LDS word to the warp;
 //   * the split over input-channel slabs (the reference's TC / atomicAdd into a
 //     pre-zeroed output) happens across the wavefronts of ONE workgroup and is
 //     reduced through LDS in a fixed order: no atomics, no pre-zeroing,
 //     bit-reproducible;
-//   * pixels are tiled as a flat index over Ho*Wo, so ragged edges cost at most
-//     one partial MFMA block per layer instead of one per row;
+//   * tiles are two-dimensional (TH x TW), so the halo is paid on a short
+//     perimeter instead of on whole image rows;
 //   * bias, residual add and ReLU are fused into the store.
 #include <hip/hip_runtime.h>
 
@@ -32,6 +41,7 @@ namespace tdc {
 
 typedef float f4_t __attribute__((ext_vector_type(4)));
 typedef float f16_t __attribute__((ext_vector_type(16)));
+typedef __attribute__((address_space(3))) void *lds_ptr_t;
 
 template <int MF>
 struct Mfma;
@@ -70,59 +80,52 @@ struct Mfma<16> {
 
 enum : int { TAPS_GENERIC = 0, TAPS_1x1 = 1, TAPS_3x3 = 9 };
 
-template <int VW>
-struct VecOf;
-template <>
-struct VecOf<1> { using type = float; };
-template <>
-struct VecOf<2> { using type = float2; };
-template <>
-struct VecOf<4> { using type = float4; };
+constexpr int OOB_OFFSET = 0x7ffffff0;  // beyond any buffer: the load returns zero
 
-// Copy input channels [c0, c0+CCH) x rows [iy0, iy0+nrows) into LDS as
-// [channel][row][RS] with zeros for the halo and for channels >= C.  The slab is
-// walked as a flat list of VW-wide vectors (RS, PL, W and CS are multiples of
-// VW, so a vector is either all image or all halo); every thread issues U
-// unconditional, clamped loads before it writes anything, so a wave keeps U
-// global loads in flight instead of one.
-template <int VW>
-__device__ __forceinline__ void stage_chunk(const ConvKParams &p, const float *__restrict__ in,
-                                            float *__restrict__ lds, int c0, int iy0, int nrows,
-                                            int tid, int nthreads) {
-    using vec_t = typename VecOf<VW>::type;
-    constexpr int U = 4;
-    const int rsv = p.RS / VW;
-    const int per_ch = nrows * rsv;
-    const int total = p.CCH * per_ch;
-    const int plv = p.PL / VW;
-    const int wv = p.W / VW;
-    const vec_t *__restrict__ src = reinterpret_cast<const vec_t *>(in);
-    for (int base = tid; base < total; base += nthreads * U) {
-        vec_t v[U];
-        int dst[U];
-        bool inb[U];
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const int e = base + u * nthreads;
-            const int ee = e < total ? e : 0;
-            const int cl = ee / per_ch;
-            const int rem = ee - cl * per_ch;
-            const int row = rem / rsv;
-            const int xv = rem - row * rsv;
-            const int c = c0 + cl;
-            const int iy = iy0 + row;
-            const int ixv = xv - plv;
-            inb[u] = c < p.C && iy >= 0 && iy < p.H && ixv >= 0 && ixv < wv;
-            const int sidx = inb[u] ? (c * p.H + iy) * wv + ixv : 0;
-            v[u] = src[sidx];
-            dst[u] = e < total ? cl * p.CS + row * p.RS + xv * VW : -1;
+// Start the copies of one pass (input channels [c0, c0+CCH) and their weights)
+// into the LDS stage at `stage`.  Nothing is waited for here.
+//
+// Input: the stage holds [CCH][CS] floats, a channel slot being [nrows][RS]
+// (+ tail).  The slot is walked in E-byte elements; element e of the stage goes
+// to LDS position e, lane l of a copy instruction supplying element blk*64+l.
+// Weights: a linear copy of `wslab_floats` floats.
+template <int E>
+__device__ __forceinline__ void issue_pass(const ConvKParams &p, __amdgpu_buffer_rsrc_t in_rsrc,
+                                           __amdgpu_buffer_rsrc_t w_rsrc, float *__restrict__ stage,
+                                           int c0, int iy0, int ix0a, unsigned w_byte0, int wave,
+                                           int nwaves, int lane) {
+    constexpr int VW = E / 4;
+    const int rsv = p.RS / VW;  // elements per LDS row
+    const int csv = p.CS / VW;  // elements per LDS channel slot
+    const int total = p.CCH * csv;
+    const int nblk = (total + 63) >> 6;
+    for (int blk = wave; blk < nblk; blk += nwaves) {
+        const int e = (blk << 6) + lane;
+        const int cl = e / csv;
+        const int rem = e - cl * csv;
+        const int row = rem / rsv;
+        const int xv = rem - row * rsv;
+        const int c = c0 + cl;
+        const int iy = iy0 + row;
+        const int ix = ix0a + xv * VW;
+        const bool inb = c < p.C && row < p.nrows && iy >= 0 && iy < p.H && ix >= 0 && ix < p.W;
+        const int voff = inb ? ((c * p.H + iy) * p.W + ix) * 4 : OOB_OFFSET;
+        if (e < total) {
+            if constexpr (E == 16)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(in_rsrc, (lds_ptr_t)(stage + (blk << 6) * VW), 16, voff, 0, 0, 0);
+            else
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(in_rsrc, (lds_ptr_t)(stage + (blk << 6) * VW), 4, voff, 0, 0, 0);
         }
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            vec_t val = v[u];
-            if (!inb[u]) val = vec_t{};
-            if (dst[u] >= 0) *reinterpret_cast<vec_t *>(lds + dst[u]) = val;
-        }
+    }
+    // Weights: 16-byte elements, 1 KiB per instruction.
+    float *wdst = stage + p.in_stage_floats;
+    const int wtotal = p.wslab_floats >> 2;
+    const int wnblk = (wtotal + 63) >> 6;
+    for (int blk = wave; blk < wnblk; blk += nwaves) {
+        const int e = (blk << 6) + lane;
+        if (e < wtotal)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(w_rsrc, (lds_ptr_t)(wdst + (blk << 8)), 16,
+                                                     (int)(w_byte0 + (unsigned)e * 16u), 0, 0, 0);
     }
 }
 
@@ -132,65 +135,62 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
     using acc_t = typename M::acc_t;
     constexpr int KC = M::KC;
     constexpr int NACC = M::NACC;
-    // K-steps fetched per weight prefetch: one channel group of a 3x3 filter,
-    // four channel groups of a 1x1 filter, a single step otherwise.
-    constexpr int G = (TAPS == TAPS_3x3) ? 9 : (TAPS == TAPS_1x1) ? 4 : 1;
     extern __shared__ __align__(16) float lds[];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int nthreads = blockDim.x;
+    const int nwaves = nthreads >> 6;
     const int wk = wave % p.WK;
     const int wn = (wave / p.WK) % p.WN;
     const int wm = wave / (p.WK * p.WN);
 
-    const int PT = MF * NB * p.WN;
+    const int PT = MF * NB * p.WN;  // pixel lanes of the workgroup (>= TH*TW)
     const int MT = MF * MB * p.WM;
-    const int p0 = blockIdx.x * PT;
+    const int tile_y = blockIdx.x / p.ntx;
+    const int tile_x = blockIdx.x - tile_y * p.ntx;
+    const int oy0 = tile_y * p.TH;
+    const int ox0 = tile_x * p.TW;
     const int m0 = blockIdx.y * MT;
     const float *__restrict__ in = p.in + (long long)blockIdx.z * p.in_bstride;
     float *__restrict__ out = p.out + (long long)blockIdx.z * p.out_bstride;
     const float *__restrict__ resid =
         p.resid ? p.resid + (long long)blockIdx.z * p.out_bstride : nullptr;
+    // Raw buffers: byte offsets at or beyond num_records read as zero.
+    const __amdgpu_buffer_rsrc_t in_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(in), (short)0, (int)(p.in_bstride * 4), 0x00020000);
+    const __amdgpu_buffer_rsrc_t w_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.wpk), (short)0, (int)p.wpk_bytes, 0x00020000);
 
-    const int plast = min(p0 + PT, p.P) - 1;
-    const int oy0 = p0 / p.Wo;
-    const int oy1 = plast / p.Wo;
     const int iy0 = oy0 * p.stride - p.pad;
-    const int nrows = (oy1 - oy0) * p.stride + (p.KH - 1) * p.dil + 1;
+    const int ix0 = ox0 * p.stride - p.pad;
+    // With 16-byte elements the window starts on a 4-float boundary of the image row.
+    const int ix0a = (p.VW == 4) ? ((ix0 >> 2) << 2) : ix0;
+    // Packed weights: [channel tile][pass][...]; one pass of this channel tile is contiguous.
+    const unsigned w_pass_bytes = (unsigned)p.wslab_floats * 4u;
+    const unsigned w_byte_base = (unsigned)blockIdx.y * (unsigned)p.nchunks * w_pass_bytes;
 
-    // Per-lane base of this wave's A-operand stream for each of its M blocks.
-    const int taps = (TAPS == TAPS_GENERIC) ? p.KH * p.KW : TAPS;
-    const float *__restrict__ wbase[MB];
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb) {
-        const int mblk = m0 / MF + wm * MB + mb;
-        wbase[mb] = p.wpk + ((long long)mblk * p.ncg_total) * taps * 64 + lane;
-    }
-    const int ncgw = p.CPW / KC;  // channel groups this wave consumes per LDS pass
-    // The wave's K-steps of pass `chunk` start at packed K-step index kfirst(chunk);
-    // a pass holds nkw of them, consumed G at a time.
-    const int nkw = ncgw * taps;
-    auto kfirst = [&](int chunk) { return ((chunk * p.CCH + wk * p.CPW) / KC) * taps; };
+    auto issue = [&](int chunk) {
+        float *stage = lds + (chunk & (p.nstage - 1)) * p.stage_floats;
+        if (p.VW == 4)
+            issue_pass<16>(p, in_rsrc, w_rsrc, stage, chunk * p.CCH, iy0, ix0a, w_byte_base + chunk * w_pass_bytes,
+                           wave, nwaves, lane);
+        else
+            issue_pass<4>(p, in_rsrc, w_rsrc, stage, chunk * p.CCH, iy0, ix0a, w_byte_base + chunk * w_pass_bytes,
+                          wave, nwaves, lane);
+    };
+    issue(0);
 
-    // First weights are requested before the input slab, so both fetches overlap.
-    float a_nxt[G][MB];
-#pragma unroll
-    for (int t = 0; t < G; ++t)
-#pragma unroll
-        for (int mb = 0; mb < MB; ++mb) a_nxt[t][mb] = wbase[mb][(long long)(kfirst(0) + t) * 64];
-
-    // Per-lane LDS offset (floats) of tap (0,0), channel sub-index included.
+    // Per-lane LDS offset (floats) of tap (0,0) for each pixel block, channel sub-index included.
     int boff[NB];
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
-        int pp = p0 + (wn * NB + nb) * MF + M::col(lane);
-        pp = min(pp, p.P - 1);
-        const int oy = pp / p.Wo;
-        const int ox = pp - oy * p.Wo;
-        boff[nb] = (oy - oy0) * p.stride * p.RS + ox * p.stride + (p.PL - p.pad) +
-                   M::ksub(lane) * p.CS;
+        const int j = (wn * NB + nb) * MF + M::col(lane);
+        int jy = j / p.TW;
+        const int jx = j - jy * p.TW;
+        jy = min(jy, p.TH - 1);  // lanes past the tile re-read its last row; they are never stored
+        boff[nb] = jy * p.stride * p.RS + jx * p.stride + (ix0 - ix0a) + M::ksub(lane) * p.CS;
     }
 
     acc_t acc[MB][NB];
@@ -201,93 +201,101 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
 #pragma unroll
             for (int v = 0; v < NACC; ++v) acc[mb][nb][v] = 0.0f;
 
-    const float *lbase = lds + wk * p.CPW * p.CS;
+    const int taps = (TAPS == TAPS_GENERIC) ? p.KH * p.KW : TAPS;
+    const int ncg_pass = p.CCH / KC;  // channel groups per pass
+    const int ncgw = p.CPW / KC;      // ... of which this wave takes [wk*ncgw, (wk+1)*ncgw)
 
     for (int chunk = 0; chunk < p.nchunks; ++chunk) {
-        if (chunk > 0) __syncthreads();
-        if (p.VW == 4) stage_chunk<4>(p, in, lds, chunk * p.CCH, iy0, nrows, tid, nthreads);
-        else if (p.VW == 2) stage_chunk<2>(p, in, lds, chunk * p.CCH, iy0, nrows, tid, nthreads);
-        else stage_chunk<1>(p, in, lds, chunk * p.CCH, iy0, nrows, tid, nthreads);
+        // My copies of this pass have landed; after the barrier everybody's have, and
+        // everybody is done reading the stage the next pass is about to overwrite.
+        __builtin_amdgcn_s_waitcnt(0);
         __syncthreads();
-        const int k0 = kfirst(chunk);
-        const int knext_chunk = kfirst(min(chunk + 1, p.nchunks - 1));
+        if (chunk + 1 < p.nchunks) issue(chunk + 1);
 
-        for (int k = 0; k < nkw; k += G) {
-            float a_cur[G][MB];
+        const float *stage = lds + (chunk & (p.nstage - 1)) * p.stage_floats;
+        const float *sin = stage + wk * p.CPW * p.CS;
+        const float *sw[MB];
 #pragma unroll
-            for (int t = 0; t < G; ++t)
-#pragma unroll
-                for (int mb = 0; mb < MB; ++mb) a_cur[t][mb] = a_nxt[t][mb];
-            // Next group of this pass, else the first group of the next pass,
-            // else (very last group) a harmless re-read of the current one.
-            int kn = k0 + k + G;
-            if (k + G >= nkw) kn = (chunk + 1 < p.nchunks) ? knext_chunk : k0 + k;
-#pragma unroll
-            for (int t = 0; t < G; ++t)
-#pragma unroll
-                for (int mb = 0; mb < MB; ++mb) a_nxt[t][mb] = wbase[mb][(long long)(kn + t) * 64];
+        for (int mb = 0; mb < MB; ++mb)
+            sw[mb] = stage + p.in_stage_floats + (((wm * MB + mb) * ncg_pass + wk * ncgw) * taps) * 64 + lane;
 
-            if constexpr (TAPS == TAPS_3x3) {
-                const float *lrow = lbase + (k / 9) * KC * p.CS;
+        if constexpr (TAPS == TAPS_3x3) {
+            // dilation 1: the column tap is an immediate offset of the LDS read,
+            // the row tap one of three per-lane row addresses.
+#pragma unroll 2
+            for (int g = 0; g < ncgw; ++g) {
+                const float *lgrp = sin + g * KC * p.CS;
 #pragma unroll
                 for (int r = 0; r < 3; ++r) {
+                    const float *lrow[NB];
+#pragma unroll
+                    for (int nb = 0; nb < NB; ++nb) lrow[nb] = lgrp + boff[nb] + r * p.RS;
 #pragma unroll
                     for (int s = 0; s < 3; ++s) {
-                        float b[NB];
+                        float a[MB], b[NB];
 #pragma unroll
-                        for (int nb = 0; nb < NB; ++nb)
-                            b[nb] = lrow[boff[nb] + r * p.dil * p.RS + s * p.dil];
+                        for (int mb = 0; mb < MB; ++mb) a[mb] = sw[mb][(g * 9 + r * 3 + s) * 64];
+#pragma unroll
+                        for (int nb = 0; nb < NB; ++nb) b[nb] = lrow[nb][s];
 #pragma unroll
                         for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-                            for (int nb = 0; nb < NB; ++nb)
-                                acc[mb][nb] = M::run(a_cur[r * 3 + s][mb], b[nb], acc[mb][nb]);
+                            for (int nb = 0; nb < NB; ++nb) acc[mb][nb] = M::run(a[mb], b[nb], acc[mb][nb]);
                     }
                 }
-            } else if constexpr (TAPS == TAPS_1x1) {
+            }
+        } else if constexpr (TAPS == TAPS_1x1) {
+#pragma unroll 4
+            for (int g = 0; g < ncgw; ++g) {
+                float a[MB], b[NB];
 #pragma unroll
-                for (int t = 0; t < G; ++t) {
-                    const float *lrow = lbase + (k + t) * KC * p.CS;
-                    float b[NB];
+                for (int mb = 0; mb < MB; ++mb) a[mb] = sw[mb][g * 64];
 #pragma unroll
-                    for (int nb = 0; nb < NB; ++nb) b[nb] = lrow[boff[nb]];
-#pragma unroll
-                    for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-                        for (int nb = 0; nb < NB; ++nb)
-                            acc[mb][nb] = M::run(a_cur[t][mb], b[nb], acc[mb][nb]);
-                }
-            } else {
-                // Any filter size / dilation: decode the tap of this K-step.
-                const int cg = k / taps;
-                const int tap = k - cg * taps;
-                const int r = tap / p.KW;
-                const int s = tap - r * p.KW;
-                const float *lrow = lbase + cg * KC * p.CS;
-                float b[NB];
-#pragma unroll
-                for (int nb = 0; nb < NB; ++nb) b[nb] = lrow[boff[nb] + r * p.dil * p.RS + s * p.dil];
+                for (int nb = 0; nb < NB; ++nb) b[nb] = sin[g * KC * p.CS + boff[nb]];
 #pragma unroll
                 for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-                    for (int nb = 0; nb < NB; ++nb)
-                        acc[mb][nb] = M::run(a_cur[0][mb], b[nb], acc[mb][nb]);
+                    for (int nb = 0; nb < NB; ++nb) acc[mb][nb] = M::run(a[mb], b[nb], acc[mb][nb]);
+            }
+        } else {
+            // Any filter size / dilation: taps walked at run time.
+            for (int g = 0; g < ncgw; ++g) {
+                const float *lgrp = sin + g * KC * p.CS;
+                int t = 0;
+                for (int r = 0; r < p.KH; ++r) {
+                    for (int s = 0; s < p.KW; ++s, ++t) {
+                        float a[MB], b[NB];
+#pragma unroll
+                        for (int mb = 0; mb < MB; ++mb) a[mb] = sw[mb][(g * taps + t) * 64];
+#pragma unroll
+                        for (int nb = 0; nb < NB; ++nb) b[nb] = lgrp[boff[nb] + r * p.dil * p.RS + s * p.dil];
+#pragma unroll
+                        for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                            for (int nb = 0; nb < NB; ++nb) acc[mb][nb] = M::run(a[mb], b[nb], acc[mb][nb]);
+                    }
+                }
             }
         }
     }
 
     if (p.WK == 1) {
         // Straight from the accumulators: each store instruction writes runs of
-        // MF consecutive pixels of one output channel.
+        // consecutive pixels of one output channel.
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb) {
+        for (int nb = 0; nb < NB; ++nb) {
+            const int j = (wn * NB + nb) * MF + M::col(lane);
+            const int jy = j / p.TW;
+            const int jx = j - jy * p.TW;
+            const int oy = oy0 + jy, ox = ox0 + jx;
+            const bool pix_ok = jy < p.TH && oy < p.Ho && ox < p.Wo;
+            const int pp = oy * p.Wo + ox;
 #pragma unroll
-            for (int nb = 0; nb < NB; ++nb) {
-                const int pp = p0 + (wn * NB + nb) * MF + M::col(lane);
+            for (int mb = 0; mb < MB; ++mb) {
 #pragma unroll
                 for (int v = 0; v < NACC; ++v) {
                     const int n = m0 + (wm * MB + mb) * MF + M::row(v, lane);
-                    if (n < p.N && pp < p.P) {
+                    if (n < p.N && pix_ok) {
                         float val = acc[mb][nb][v];
                         if (p.bias) val += p.bias[n];
                         const long long o = (long long)n * p.P + pp;
@@ -300,7 +308,7 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
         }
     } else {
         // Split-K across waves: park every wave's partial tile in LDS
-        // ([wk][channel][pixel]) and add the WK slices in index order.
+        // ([wk][channel][pixel lane]) and add the WK slices in index order.
         __syncthreads();
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) {
@@ -318,14 +326,16 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
         const int total = MT * PT;
         for (int idx = tid; idx < total; idx += nthreads) {
             const int ml = idx / PT;
-            const int pl = idx - ml * PT;
+            const int j = idx - ml * PT;
+            const int jy = j / p.TW;
+            const int jx = j - jy * p.TW;
             const int n = m0 + ml;
-            const int pp = p0 + pl;
-            if (n < p.N && pp < p.P) {
+            const int oy = oy0 + jy, ox = ox0 + jx;
+            if (n < p.N && jy < p.TH && oy < p.Ho && ox < p.Wo) {
                 float val = lds[idx];
                 for (int k = 1; k < p.WK; ++k) val += lds[k * total + idx];
                 if (p.bias) val += p.bias[n];
-                const long long o = (long long)n * p.P + pp;
+                const long long o = (long long)n * p.P + oy * p.Wo + ox;
                 if (resid) val += resid[o];
                 if (p.relu) val = fmaxf(val, 0.0f);
                 out[o] = val;
@@ -335,9 +345,8 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
 }
 
 // ---------------------------------------------------------------------------
-// Instantiation table.  Tiles with a 2x2 block grid per wave need up to 64
-// accumulator registers plus two weight buffers, so they are built for at most
-// 8 waves per workgroup (256 registers per lane); the others for 16 waves.
+// Instantiation table.  A 2x2 block grid of MFMAs per wave is built for at
+// most 8 waves per workgroup (256 registers per lane); everything else for 16.
 // ---------------------------------------------------------------------------
 typedef void (*kernel_fn)(const ConvKParams);
 
@@ -357,25 +366,20 @@ static kernel_fn pick_mf(int mf, int mb, int nb) {
     return nullptr;
 }
 
-static int taps_mode(const ConvKParams &kp) {
-    if (kp.KH == 3 && kp.KW == 3) return TAPS_3x3;
-    if (kp.KH == 1 && kp.KW == 1) return TAPS_1x1;
+static int taps_mode(int KH, int KW, int dil) {
+    if (KH == 3 && KW == 3 && dil == 1) return TAPS_3x3;
+    if (KH == 1 && KW == 1) return TAPS_1x1;
     return TAPS_GENERIC;
 }
 
-static kernel_fn pick_kernel(const tdc_tile &t, int mode) {
-    switch (mode) {
-        case TAPS_3x3: return pick_mf<TAPS_3x3>(t.mf, t.mb, t.nb);
-        case TAPS_1x1: return pick_mf<TAPS_1x1>(t.mf, t.mb, t.nb);
-        default: return pick_mf<TAPS_GENERIC>(t.mf, t.mb, t.nb);
+const void *conv_kernel_for(const tdc_tile &t, int KH, int KW, int dilation) {
+    kernel_fn fn = nullptr;
+    switch (taps_mode(KH, KW, dilation)) {
+        case TAPS_3x3: fn = pick_mf<TAPS_3x3>(t.mf, t.mb, t.nb); break;
+        case TAPS_1x1: fn = pick_mf<TAPS_1x1>(t.mf, t.mb, t.nb); break;
+        default: fn = pick_mf<TAPS_GENERIC>(t.mf, t.mb, t.nb); break;
     }
-}
-
-const void *conv_kernel_for(const tdc_tile &t, int KH, int KW) {
-    ConvKParams kp{};
-    kp.KH = KH;
-    kp.KW = KW;
-    return reinterpret_cast<const void *>(pick_kernel(t, taps_mode(kp)));
+    return reinterpret_cast<const void *>(fn);
 }
 
 int prepare_conv_kernel(const void *fn, const Geometry &g) {

@@ -104,11 +104,11 @@ int tdc_conv_plan_create(const tdc_conv_desc *desc, const tdc_tile *forced_tile,
     }
     p->tile = p->info.tile;
     if (!make_geometry(*desc, p->tile, p->geo, &why)) return fail(TDC_ERR_INVALID, why);
-    p->kernel = conv_kernel_for(p->tile, desc->KH, desc->KW);
+    p->kernel = conv_kernel_for(p->tile, desc->KH, desc->KW, desc->dilation);
     if (!p->kernel) return fail(TDC_ERR_UNSUPPORTED, "no kernel instantiated for this tile");
     int he = prepare_conv_kernel(p->kernel, p->geo);
     if (he) return hip_fail("hipFuncSetAttribute(MaxDynamicSharedMemorySize)", he);
-    const size_t wfloats = packed_weight_floats(p->geo, p->tile.mf);
+    const size_t wfloats = packed_weight_floats(p->geo);
     e = hipMalloc((void **)&p->d_wpk, wfloats * sizeof(float));
     if (e != hipSuccess) return hip_fail("hipMalloc(packed weights)", e);
     if (desc->has_bias) {
@@ -126,14 +126,14 @@ int tdc_conv_plan_set_weights(tdc_conv_plan *plan, const float *w_oihw, const fl
     if (!plan || !w_oihw) return fail(TDC_ERR_INVALID, "null argument");
     if ((plan->desc.has_bias != 0) != (bias != nullptr))
         return fail(TDC_ERR_INVALID, "bias pointer does not match desc.has_bias");
-    const size_t wfloats = packed_weight_floats(plan->geo, plan->tile.mf);
+    const size_t wfloats = packed_weight_floats(plan->geo);
     std::vector<float> packed;
     try {
         packed.resize(wfloats);
     } catch (const std::bad_alloc &) {
         return fail(TDC_ERR_NOMEM, "out of host memory packing weights");
     }
-    pack_weights(plan->desc, plan->geo, plan->tile.mf, w_oihw, packed.data());
+    pack_weights(plan->desc, plan->tile, plan->geo, w_oihw, packed.data());
     hipError_t e = hipMemcpy(plan->d_wpk, packed.data(), wfloats * sizeof(float), hipMemcpyHostToDevice);
     if (e != hipSuccess) return hip_fail("hipMemcpy(packed weights)", e);
     if (bias) {
@@ -161,16 +161,19 @@ int tdc_conv_forward(tdc_conv_plan *plan, const float *d_in, const float *d_resi
     kp.bias = plan->d_bias;
     kp.resid = d_residual;
     kp.out = d_out;
-    kp.C = d.C; kp.H = d.H; kp.W = d.W; kp.N = d.N;
+    kp.C = d.C; kp.H = g.He; kp.W = g.We; kp.N = d.N;
     kp.Ho = g.Ho; kp.Wo = g.Wo; kp.P = g.P;
     kp.KH = d.KH; kp.KW = d.KW; kp.stride = d.stride; kp.pad = d.pad; kp.dil = d.dilation;
+    kp.TW = g.TW; kp.TH = g.TH; kp.ntx = g.ntx;
     kp.WM = plan->tile.wm; kp.WN = plan->tile.wn; kp.WK = plan->tile.wk;
     kp.CCH = plan->tile.cch; kp.nchunks = g.nchunks; kp.CPW = g.cpw;
-    kp.RS = g.RS; kp.CS = g.CS; kp.PL = g.PL;
-    // Vector loads need the activations aligned to the vector size; fall back to scalars otherwise.
+    kp.RS = g.RS; kp.CS = g.CS; kp.nrows = g.nrows;
+    // 16-byte copy elements need 16-byte aligned activations; otherwise fall back to 4-byte elements.
     kp.VW = (reinterpret_cast<uintptr_t>(d_in) % (4 * g.VW) == 0) ? g.VW : 1;
+    kp.in_stage_floats = g.in_stage_floats; kp.wslab_floats = g.wslab_floats;
+    kp.stage_floats = g.stage_floats; kp.nstage = g.nstage;
     kp.relu = d.relu;
-    kp.ncg_total = g.c_pad / g.kc;
+    kp.wpk_bytes = (unsigned)(packed_weight_floats(g) * sizeof(float));
     kp.in_bstride = (long long)d.C * d.H * d.W;
     kp.out_bstride = (long long)d.N * g.P;
     int he = launch_conv(plan->kernel, g, kp, stream);

@@ -28,21 +28,28 @@ const Machine &machine();
 
 // ---- launch geometry derived from (desc, tile) ----------------------------
 struct Geometry {
-    int Ho = 0, Wo = 0, P = 0;       // output height/width, Ho*Wo
+    // The kernel's view of the input: a 1x1 / stride 1 / pad 0 convolution is
+    // run on the image flattened to one row of H*W pixels.
+    int He = 0, We = 0;
+    int Ho = 0, Wo = 0, P = 0;       // output height/width (of the kernel's view), Ho*Wo
     int kc = 0;                      // input channels consumed per MFMA (2 or 4)
     int taps = 0;                    // KH*KW
-    int PT = 0, MT = 0;              // pixels / output channels per workgroup
+    int PT = 0, MT = 0;              // pixel lanes / output channels per workgroup
+    int TW = 0, TH = 0;              // output tile
+    int ntx = 0, nty = 0;            // tiles across / down
     int grid_x = 0, grid_y = 0, grid_z = 0;
     int waves = 0, threads = 0;
     int cpw = 0;                     // channels per wave per LDS pass (cch / wk)
     int nchunks = 0;                 // LDS passes
     int c_pad = 0;                   // nchunks * cch
-    int n_pad = 0;                   // grid_y * MT (rows of the packed weights)
-    int VW = 1;                      // floats per vector of the LDS fill (4 if W%4==0, 2 if W%2==0)
-    int PL = 0;                      // left zero columns in an LDS row (multiple of VW, >= pad)
+    int VW = 1;                      // floats per element of the LDS fill (4 if We%4==0, else 1)
+    int nrows = 0, ncols = 0;        // input window of one tile
     int RS = 0;                      // LDS row stride (floats)
-    int nrows = 0;                   // max input rows a workgroup stages
     int CS = 0;                      // LDS channel stride (floats)
+    int in_stage_floats = 0;         // cch * CS, rounded up to 4
+    int wslab_floats = 0;            // weights of one pass of one channel tile
+    int stage_floats = 0;
+    int nstage = 1;
     int lds_bytes = 0;
     int max_waves_kernel = 0;        // launch bound of the instantiated kernel
 };
@@ -51,18 +58,16 @@ struct Geometry {
 bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::string *why);
 bool check_desc(const tdc_conv_desc &d, std::string *why);
 
-// Model: fills everything in `info` except nothing device-specific.
 bool model_evaluate(const tdc_conv_desc &d, const tdc_tile &t, tdc_tile_info &info, std::string *why);
 std::vector<tdc_tile> model_enumerate(const tdc_conv_desc &d);
 bool model_select(const tdc_conv_desc &d, tdc_tile_info &info, std::string *why);
 
 // ---- weight packing --------------------------------------------------------
-// OIHW [N,C,KH,KW] -> MFMA A-operand order [n_pad/mf][c_pad/kc][taps][64 lanes]:
-// lane l of entry (mblk, cg, tap) holds w[mblk*mf + l%mf][cg*kc + l/mf][tap],
-// zero outside N x C.
-size_t packed_weight_floats(const Geometry &g, int mf);
-void pack_weights(const tdc_conv_desc &d, const Geometry &g, int mf, const float *w_oihw,
-                  float *packed);
+// OIHW [N,C,KH,KW] -> [channel tile][pass][M block in tile][channel group in pass][tap][64 lanes]
+// in MFMA A-operand order: lane l of an entry holds
+// w[tile*MT + mblk*mf + l%mf][pass*cch + cg*kc + l/mf][tap], zero outside N x C.
+size_t packed_weight_floats(const Geometry &g);
+void pack_weights(const tdc_conv_desc &d, const tdc_tile &t, const Geometry &g, const float *w_oihw, float *packed);
 
 // ---- kernel arguments ------------------------------------------------------
 struct ConvKParams {
@@ -73,18 +78,19 @@ struct ConvKParams {
     float *out;
     int C, H, W, N, Ho, Wo, P;
     int KH, KW, stride, pad, dil;
+    int TW, TH, ntx;
     int WM, WN, WK;
     int CCH, nchunks, CPW;
-    int RS, CS, PL;
-    int VW;               // vector width of the LDS fill (4, 2 or 1 floats)
+    int RS, CS, VW, nrows;
+    int in_stage_floats, wslab_floats, stage_floats, nstage;
     int relu;
-    int ncg_total;        // c_pad / kc
+    unsigned wpk_bytes;
     long long in_bstride;   // C*H*W
     long long out_bstride;  // N*P
 };
 
 // The instantiated kernel for a tile and filter size (nullptr if none).
-const void *conv_kernel_for(const tdc_tile &t, int KH, int KW);
+const void *conv_kernel_for(const tdc_tile &t, int KH, int KW, int dilation);
 // One-time per-plan attribute setup (dynamic LDS above 64 KiB).  hipError_t as int.
 int prepare_conv_kernel(const void *fn, const Geometry &g);
 // Enqueue the kernel.  Returns a hipError_t as int.

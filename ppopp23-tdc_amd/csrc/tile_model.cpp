@@ -1,4 +1,4 @@
-// Launch geometry and the closed-form gfx950 tile model.
+// Launch geometry, weight packing and the closed-form gfx950 tile model.
 //
 // The reference chooses (TH, TW, TC) per layer either from a measured sweep
 // (2080Ti-evaluation/TDC-LAYERS-ORACLE/gen_from_occupancy.py:51-66) or from an
@@ -7,8 +7,8 @@
 // 2080Ti-evaluation/Gen-occupancy/template.cu:277-284).  This file is the
 // self-contained counterpart for one MI355X: occupancy comes from the register
 // and LDS footprint of the tile, latency from MFMA issue cycles per SIMD, the
-// L1 fill rate for the staged input and streamed weights, and wave quantisation
-// over 256 compute units.  Host-only code: it runs without a GPU.
+// copy volume of the staged input window and weights, and wave quantisation over
+// 256 compute units.  Host-only code: it runs without a GPU.
 #include <algorithm>
 #include <cmath>
 #include <cstdlib>
@@ -39,19 +39,25 @@ bool check_desc(const tdc_conv_desc &d, std::string *why) {
     const long long eh = (long long)d.H + 2LL * d.pad - (long long)d.dilation * (d.KH - 1) - 1;
     const long long ew = (long long)d.W + 2LL * d.pad - (long long)d.dilation * (d.KW - 1) - 1;
     if (eh < 0 || ew < 0) return fail("filter (with dilation) larger than padded input");
-    if ((long long)d.C * d.H * d.W >= (1LL << 31) || (long long)d.N * d.H * d.W >= (1LL << 31))
-        return fail("per-image tensor exceeds 2^31 elements");
+    // One image is addressed through a 32-bit buffer descriptor (byte offsets below 2^31).
+    if ((long long)d.C * d.H * d.W >= (1LL << 29) || (long long)d.N * d.H * d.W >= (1LL << 29))
+        return fail("per-image tensor exceeds 2^29 elements");
+    if ((long long)d.N * d.C * d.KH * d.KW >= (1LL << 28)) return fail("weight tensor exceeds 2^28 elements");
     return true;
 }
 
 // LDS channel stride: the lanes of one ds_read that belong to different input
-// channels of an MFMA K-step must fall into different banks.  With 4-byte banks
-// a stride of 32 (mod 64) separates the two halves of a 32x32x2 step and a
-// stride of 16 (mod 64) separates the four quarters of a 16x16x4 step.
-static int pad_channel_stride(int raw, int mf) {
+// channels of an MFMA K-step should fall into different banks.  With 4-byte
+// banks a stride of 32 (mod 64) separates the two halves of a 32x32x2 step and
+// a stride of 16 (mod 32) the quarters of a 16x16x4 step.  Small windows are
+// not inflated by more than a quarter for this.
+static int pad_channel_stride(int raw, int mf, int vw) {
+    const int mod = (mf == 32) ? 64 : 32;
     const int want = (mf == 32) ? 32 : 16;
-    int cs = raw;
-    while (cs % 64 != want) ++cs;
+    int cs = round_up(raw, vw);
+    int padded = cs;
+    while (padded % mod != want) padded += vw;
+    if (padded - raw <= raw / 4) cs = padded;
     return cs;
 }
 
@@ -66,70 +72,84 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
     if (t.wm < 1 || t.wn < 1 || t.wk < 1) return fail("tile.wm / wn / wk must be >= 1");
     g = Geometry();
     g.max_waves_kernel = (t.mb == 2 && t.nb == 2) ? 8 : 16;
+    if ((long long)t.wm * t.wn * t.wk > g.max_waves_kernel) return fail("too many waves per workgroup for this tile");
     g.waves = t.wm * t.wn * t.wk;
-    if (g.waves > g.max_waves_kernel) return fail("too many waves per workgroup for this tile");
     g.threads = g.waves * 64;
-    g.Ho = (d.H + 2 * d.pad - d.dilation * (d.KH - 1) - 1) / d.stride + 1;
-    g.Wo = (d.W + 2 * d.pad - d.dilation * (d.KW - 1) - 1) / d.stride + 1;
+    const bool flat = (d.KH == 1 && d.KW == 1 && d.stride == 1 && d.pad == 0);
+    g.He = flat ? 1 : d.H;
+    g.We = flat ? d.H * d.W : d.W;
+    g.Ho = (g.He + 2 * d.pad - d.dilation * (d.KH - 1) - 1) / d.stride + 1;
+    g.Wo = (g.We + 2 * d.pad - d.dilation * (d.KW - 1) - 1) / d.stride + 1;
     g.P = g.Ho * g.Wo;
     g.kc = (t.mf == 32) ? 2 : 4;
     g.taps = d.KH * d.KW;
     g.PT = t.mf * t.nb * t.wn;
     g.MT = t.mf * t.mb * t.wm;
-    g.grid_x = ceil_div(g.P, g.PT);
+    if (t.tw < 1 || t.tw > g.PT || t.tw > g.Wo) return fail("tile.tw must be in [1, min(Wo, pixel lanes)]");
+    g.TW = t.tw;
+    g.TH = std::min(g.PT / t.tw, g.Ho);
+    g.ntx = ceil_div(g.Wo, g.TW);
+    g.nty = ceil_div(g.Ho, g.TH);
+    if ((long long)g.ntx * g.nty > (1LL << 30)) return fail("grid too large");
+    g.grid_x = g.ntx * g.nty;
     g.grid_y = ceil_div(d.N, g.MT);
     g.grid_z = d.batch;
     if (g.grid_y > 65535 || g.grid_z > 65535) return fail("grid too large");
-    const bool one_by_one = (d.KH == 1 && d.KW == 1);
-    const int granule = g.kc * t.wk * (one_by_one ? 4 : 1);
-    if (t.cch < granule || t.cch % granule != 0)
-        return fail("tile.cch must be a positive multiple of kc*wk (x4 for 1x1 filters)");
+    const int granule = g.kc * t.wk;
+    if (t.cch < granule || t.cch % granule != 0) return fail("tile.cch must be a positive multiple of kc*wk");
+    if (t.cch > round_up(d.C, granule)) return fail("tile.cch exceeds the (padded) channel count");
     g.cpw = t.cch / t.wk;
     g.nchunks = ceil_div(d.C, t.cch);
     g.c_pad = g.nchunks * t.cch;
-    g.n_pad = g.grid_y * g.MT;
-    // LDS rows are filled with VW-wide vectors: the left halo and the row stride
-    // are rounded up so that every image row starts on a vector boundary.
-    g.VW = (d.W % 4 == 0) ? 4 : (d.W % 2 == 0) ? 2 : 1;
-    g.PL = round_up(d.pad, g.VW);
-    g.RS = round_up(g.PL + d.W + d.pad, g.VW);
-    int nrows = 0;
-    for (int bx = 0; bx < g.grid_x; ++bx) {
-        const int p0 = bx * g.PT;
-        const int pl = std::min(p0 + g.PT, g.P) - 1;
-        const int span = pl / g.Wo - p0 / g.Wo;
-        nrows = std::max(nrows, span * d.stride + (d.KH - 1) * d.dilation + 1);
+    g.nrows = (g.TH - 1) * d.stride + (d.KH - 1) * d.dilation + 1;
+    g.ncols = (g.TW - 1) * d.stride + (d.KW - 1) * d.dilation + 1;
+    // LDS rows are filled with 16-byte elements when image rows are a multiple of
+    // 4 floats: the window then starts at the 4-float boundary at or left of its
+    // first column, which can cost up to 3 extra columns.
+    g.VW = (g.We % 4 == 0) ? 4 : 1;
+    if (g.VW == 4) {
+        int shift = 0;
+        for (int tx = 0; tx < std::min(g.ntx, 4); ++tx) {
+            const int ix0 = tx * g.TW * d.stride - d.pad;
+            shift = std::max(shift, ((ix0 % 4) + 4) % 4);
+        }
+        g.RS = round_up(g.ncols + shift, 4);
+    } else {
+        g.RS = g.ncols;
     }
-    g.nrows = nrows;
-    g.CS = pad_channel_stride(nrows * g.RS, t.mf);
-    const long long in_bytes = (long long)t.cch * g.CS * 4;
+    g.CS = pad_channel_stride(g.nrows * g.RS, t.mf, g.VW);
+    g.in_stage_floats = round_up(t.cch * g.CS, 4);
+    g.wslab_floats = (t.wm * t.mb) * (t.cch / g.kc) * g.taps * 64;
+    g.stage_floats = g.in_stage_floats + g.wslab_floats;
+    g.nstage = g.nchunks > 1 ? 2 : 1;
+    const long long stage_bytes = (long long)g.nstage * g.stage_floats * 4;
     const long long red_bytes = t.wk > 1 ? (long long)t.wk * g.MT * g.PT * 4 : 0;
-    const long long lds = std::max(in_bytes, red_bytes);
+    const long long lds = std::max(stage_bytes, red_bytes);
     if (lds > machine().lds_bytes_per_cu) return fail("tile needs more than 160 KiB of LDS");
     g.lds_bytes = (int)lds;
+    if ((long long)g.grid_y * g.nchunks * g.wslab_floats * 4 >= (1LL << 31)) return fail("packed weights exceed 2 GiB");
     return true;
 }
 
-size_t packed_weight_floats(const Geometry &g, int mf) {
-    return (size_t)(g.n_pad / mf) * (size_t)(g.c_pad / g.kc) * (size_t)g.taps * 64;
+size_t packed_weight_floats(const Geometry &g) {
+    return (size_t)g.grid_y * (size_t)g.nchunks * (size_t)g.wslab_floats;
 }
 
-void pack_weights(const tdc_conv_desc &d, const Geometry &g, int mf, const float *w, float *packed) {
-    const int nmblk = g.n_pad / mf;
-    const int ncg = g.c_pad / g.kc;
+void pack_weights(const tdc_conv_desc &d, const tdc_tile &t, const Geometry &g, const float *w, float *packed) {
+    const int mbw = t.wm * t.mb;
+    const int ncg = t.cch / g.kc;
     const int taps = g.taps;
-    for (int mblk = 0; mblk < nmblk; ++mblk) {
-        for (int cg = 0; cg < ncg; ++cg) {
-            for (int tap = 0; tap < taps; ++tap) {
-                float *dst = packed + (((size_t)mblk * ncg + cg) * taps + tap) * 64;
-                for (int l = 0; l < 64; ++l) {
-                    const int n = mblk * mf + l % mf;
-                    const int c = cg * g.kc + l / mf;
-                    dst[l] = (n < d.N && c < d.C) ? w[((size_t)n * d.C + c) * taps + tap] : 0.0f;
-                }
-            }
-        }
-    }
+    float *dst = packed;
+    for (int by = 0; by < g.grid_y; ++by)
+        for (int chunk = 0; chunk < g.nchunks; ++chunk)
+            for (int mbl = 0; mbl < mbw; ++mbl)
+                for (int cg = 0; cg < ncg; ++cg)
+                    for (int tap = 0; tap < taps; ++tap)
+                        for (int l = 0; l < 64; ++l) {
+                            const int n = by * g.MT + mbl * t.mf + l % t.mf;
+                            const int c = chunk * t.cch + cg * g.kc + l / t.mf;
+                            *dst++ = (n < d.N && c < d.C) ? w[((size_t)n * d.C + c) * taps + tap] : 0.0f;
+                        }
 }
 
 // ---------------------------------------------------------------------------
@@ -138,21 +158,22 @@ void pack_weights(const tdc_conv_desc &d, const Geometry &g, int mf, const float
 namespace {
 
 struct ModelConst {
-    double launch_us = 1.6;        // empty-kernel device time incl. dispatch ramp
-    double l1_bytes_per_clk = 64;  // per-CU vector memory fill rate
-    double mem_latency_clk = 1800; // first-byte latency of a dependent fetch (L2/MALL)
+    double launch_us = 1.7;           // device time of an empty kernel in a back-to-back stream
+    double setup_clk = 900;           // kernel arguments, index arithmetic before the first copy is issued
+    double copy_latency_clk = 2200;   // first byte of a global->LDS copy (L2 / memory-side cache)
+    double copy_bytes_per_clk = 48;   // sustained global->LDS rate of one CU
+    double l2_bytes_per_clk = 3600;   // whole-chip L2->CU rate when every CU copies at once
     double lds_bytes_per_clk = 128;
-    double sync_clk = 200;
+    double sync_clk = 120;
+    double store_bytes_per_clk = 32;  // per CU, short runs per channel
 };
 const ModelConst MC;
 
-int estimate_vgprs(const tdc_tile &t, int taps) {
+// Registers per lane of the instantiated kernels, rounded up to the allocation granule of 8.
+int kernel_vgprs(const tdc_tile &t, int taps_mode) {
     const int nacc = (t.mf == 32) ? 16 : 4;
-    int regs = nacc * t.mb * t.nb;             // accumulators
-    if (taps == 9) regs += 2 * 9 * t.mb + 9 * t.nb;   // two weight buffers + row of B
-    else if (taps == 1) regs += 2 * 4 * t.mb + 4 * t.nb;
-    else regs += t.mb + t.nb;
-    regs += 28;                                 // addresses, indices, staging temporaries
+    int regs = nacc * t.mb * t.nb + 6 * (t.mb + t.nb) + 24;
+    if (taps_mode == 9) regs += 6 * t.nb;
     return round_up(regs, 8);
 }
 
@@ -170,71 +191,78 @@ bool model_evaluate(const tdc_conv_desc &d, const tdc_tile &t, tdc_tile_info &in
     info.block_threads = g.threads;
     info.lds_bytes = g.lds_bytes;
     info.nchunks = g.nchunks;
-    info.vgpr_estimate = estimate_vgprs(t, g.taps);
+    info.th = g.TH;
+    const int mode = (d.KH == 3 && d.KW == 3 && d.dilation == 1) ? 9 : (d.KH == 1 && d.KW == 1) ? 1 : 0;
+    info.vgpr_estimate = kernel_vgprs(t, mode);
 
     // --- occupancy (replaces cudaOccupancyMaxActiveBlocksPerMultiprocessor) ---
     const int waves_simd_vgpr = std::min(m.max_waves_per_simd, m.vgprs_per_simd_lane / info.vgpr_estimate);
     const int wg_waves_per_simd = ceil_div(g.waves, m.simds_per_cu);
     const int wg_by_vgpr = waves_simd_vgpr / wg_waves_per_simd;
     const int wg_by_lds = m.lds_bytes_per_cu / std::max(g.lds_bytes, 1);
-    int wg_per_cu = std::min(wg_by_vgpr, wg_by_lds);
+    int wg_per_cu = std::min(std::min(wg_by_vgpr, wg_by_lds), 8);
     if (wg_per_cu < 1) {
         if (why) *why = "tile does not fit one compute unit";
         return false;
     }
-    wg_per_cu = std::min(wg_per_cu, 8);
     info.wg_per_cu = wg_per_cu;
     info.waves_per_simd = wg_per_cu * wg_waves_per_simd;
 
     // --- algorithmic work and roofline ---------------------------------------
-    const double P = g.P;
+    const double P = (double)g.P;
     info.flops = 2.0 * P * d.C * d.N * g.taps * d.batch;
     info.bytes = 4.0 * ((double)d.batch * ((double)d.C * d.H * d.W + (double)d.N * P) +
                         (double)g.taps * d.C * d.N);
     info.roof_us = std::max(info.bytes / (m.hbm_tbps * 1e6), info.flops / (m.fp32_tflops * 1e6));
 
     // --- per-workgroup costs (clock cycles of one CU) ------------------------
+    const long long n_wg = (long long)g.grid_x * g.grid_y * g.grid_z;
     const double mfma_clk = (t.mf == 32) ? 64.0 : 32.0;
-    const double ksteps_wave = (double)g.nchunks * (g.cpw / g.kc) * g.taps;
-    const double mfma_wave = ksteps_wave * t.mb * t.nb * mfma_clk;       // one wave's matrix-core time
-    const double stage_bytes = (double)g.c_pad * g.nrows * g.RS * 4.0;   // input slab of one WG
-    const double weight_bytes = ksteps_wave * t.mb * 256.0 * g.waves;    // streamed by all waves of one WG
+    const double ksteps_pass = (double)(g.cpw / g.kc) * g.taps;
+    // One wave's matrix-core time per pass; the LDS reads of a K-step (one A and
+    // one B word per lane per block row/column) must fit under it.
+    const double mfma_pass = ksteps_pass * t.mb * t.nb * mfma_clk;
+    const double ldsrd_pass = ksteps_pass * (t.mb + t.nb) * 256.0 / MC.lds_bytes_per_clk;
+    const double copy_bytes_pass = (double)g.stage_floats * 4.0;
     const double red_bytes = t.wk > 1 ? (double)t.wk * g.MT * g.PT * 4.0 * 2.0 : 0.0;
     const double out_bytes = (double)g.MT * g.PT * 4.0;
 
-    const long long n_wg = (long long)g.grid_x * g.grid_y * g.grid_z;
-    auto round_clk = [&](int r) {
-        // r workgroups share one CU: matrix time adds up per SIMD, fills share the L1 port.
-        const double mfma = mfma_wave * wg_waves_per_simd * r;
-        const double wfill = weight_bytes * r / MC.l1_bytes_per_clk;
-        const double sfill = stage_bytes * r / MC.l1_bytes_per_clk;
-        // Staging of one workgroup overlaps other workgroups' MFMAs only when r > 1.
-        const double stage = MC.mem_latency_clk * g.nchunks + (r > 1 ? 0.5 : 1.0) * sfill +
-                             2.0 * MC.sync_clk * g.nchunks;
-        const double epi = red_bytes * r / MC.lds_bytes_per_clk + out_bytes * r / MC.l1_bytes_per_clk +
-                           (t.wk > 1 ? 2.0 * MC.sync_clk : 0.0) + 300.0;
-        return stage + std::max(mfma + MC.mem_latency_clk * 0.25, wfill + MC.mem_latency_clk) + epi;
+    auto wg_time = [&](int r, long long concurrent_wgs) {
+        // r workgroups share one CU: matrix time adds up per SIMD, LDS reads over the CU, copies share
+        // the CU's fill rate and, chip-wide, the L2.
+        const double compute =
+            std::max(mfma_pass * wg_waves_per_simd * r, ldsrd_pass * g.waves * r) + 2 * MC.sync_clk;
+        const double chip_share =
+            MC.l2_bytes_per_clk / std::max<double>(1.0, (double)std::min<long long>(concurrent_wgs, m.cus));
+        const double rate = std::min(MC.copy_bytes_per_clk, chip_share);
+        const double copy = copy_bytes_pass * r / rate;
+        // First pass is exposed; afterwards the copy of pass i+1 runs under the MFMAs of pass i.
+        double clk = MC.setup_clk + MC.copy_latency_clk + copy;
+        clk += compute;  // last pass: nothing left to hide
+        if (g.nchunks > 1) clk += (g.nchunks - 1) * std::max(compute, copy + 0.35 * MC.copy_latency_clk);
+        clk += red_bytes * r / MC.lds_bytes_per_clk + out_bytes * r / MC.store_bytes_per_clk +
+               (t.wk > 1 ? 2.0 * MC.sync_clk : 0.0) + 400.0;
+        return clk;
     };
     const long long slots = (long long)m.cus * wg_per_cu;
     const long long full = n_wg / slots;
     const long long rem = n_wg % slots;
-    double clk = (double)full * round_clk(wg_per_cu);
-    if (rem) clk += round_clk((int)ceil_div((int)rem, m.cus));
+    double clk = (double)full * wg_time(wg_per_cu, slots);
+    if (rem) clk += wg_time((int)((rem + m.cus - 1) / m.cus), rem);
     info.pred_us = MC.launch_us + clk / (m.clock_ghz * 1e3);
-    info.pred_hbm_bytes = (double)n_wg * (stage_bytes + weight_bytes) + (double)d.batch * d.N * P * 4.0;
+    info.pred_l2_bytes = (double)n_wg * g.nchunks * copy_bytes_pass;
     return true;
 }
 
 std::vector<tdc_tile> model_enumerate(const tdc_conv_desc &d) {
     std::vector<tdc_tile> out;
-    std::string why;
-    if (!check_desc(d, &why)) return out;
-    const Machine &m = machine();
-    const int Ho = (d.H + 2 * d.pad - d.dilation * (d.KH - 1) - 1) / d.stride + 1;
-    const int Wo = (d.W + 2 * d.pad - d.dilation * (d.KW - 1) - 1) / d.stride + 1;
+    if (!check_desc(d, nullptr)) return out;
+    const bool flat = (d.KH == 1 && d.KW == 1 && d.stride == 1 && d.pad == 0);
+    const int He = flat ? 1 : d.H, We = flat ? d.H * d.W : d.W;
+    const int Ho = (He + 2 * d.pad - d.dilation * (d.KH - 1) - 1) / d.stride + 1;
+    const int Wo = (We + 2 * d.pad - d.dilation * (d.KW - 1) - 1) / d.stride + 1;
     const int P = Ho * Wo;
-    const bool one_by_one = (d.KH == 1 && d.KW == 1);
-    static const int mfs[] = {32, 16};
+    static const int mfs[] = {16, 32};
     static const int wks[] = {1, 2, 4, 8, 16};
     static const int wms[] = {1, 2, 4};
     static const int wns[] = {1, 2, 4};
@@ -247,41 +275,38 @@ std::vector<tdc_tile> model_enumerate(const tdc_conv_desc &d) {
                         for (int wk : wks) {
                             const int maxw = (mb == 2 && nb == 2) ? 8 : 16;
                             if (wm * wn * wk > maxw) continue;
-                            // Do not tile past the problem.
-                            if (mf * mb * wm > round_up(d.N, mf)) continue;
-                            if (mf * nb * wn > round_up(P, mf)) continue;
-                            const int granule = kc * wk * (one_by_one ? 4 : 1);
-                            const int c_full = round_up(d.C, granule);
-                            // Candidate LDS pass sizes: everything at once, or the largest
-                            // slab that leaves room for 1, 2 or 4 workgroups per CU.
-                            int last = -1;
-                            for (int share = 0; share <= 3; ++share) {
-                                int cch;
-                                if (share == 0) {
-                                    cch = c_full;
-                                } else {
-                                    const int budget = m.lds_bytes_per_cu / (1 << (share - 1));
-                                    tdc_tile probe{mf, mb, nb, wm, wn, wk, granule};
-                                    Geometry gp;
-                                    if (!make_geometry(d, probe, gp, nullptr)) continue;
-                                    const int fit = budget / (gp.CS * 4);
-                                    cch = std::min(c_full, (fit / granule) * granule);
-                                    if (cch < granule) continue;
-                                    // Prefer an even split of the channels over a ragged last pass.
-                                    const int passes = ceil_div(d.C, cch);
-                                    cch = round_up(ceil_div(d.C, passes), granule);
-                                }
-                                if (cch == last) continue;
-                                tdc_tile t{mf, mb, nb, wm, wn, wk, cch};
-                                Geometry g;
-                                if (!make_geometry(d, t, g, nullptr)) continue;
-                                bool dup = false;
-                                for (const tdc_tile &o : out)
-                                    if (!std::memcmp(&o, &t, sizeof(t))) { dup = true; break; }
-                                if (dup) continue;
-                                out.push_back(t);
-                                last = cch;
+                            if (mf * mb * wm > round_up(d.N, mf)) continue;  // do not tile past the problem
+                            const int PT = mf * nb * wn;
+                            if (PT > round_up(P, mf)) continue;
+                            // Tile widths: the whole row, and power-of-two or exact-divisor widths
+                            // that keep at least 70 % of the pixel lanes on real pixels.
+                            std::vector<int> tws;
+                            for (int tw = 1; tw <= std::min(Wo, PT); ++tw) {
+                                const bool pow2 = (tw & (tw - 1)) == 0;
+                                const bool widest = (tw == std::min(Wo, PT));
+                                if (!(widest || (pow2 && tw >= 4) || (Wo % tw == 0 && tw >= 4))) continue;
+                                const int th = std::min(PT / tw, Ho);
+                                const double util = (double)P / ((double)ceil_div(Wo, tw) * ceil_div(Ho, th) * PT);
+                                if (util < 0.7 && !widest) continue;
+                                tws.push_back(tw);
                             }
+                            const int granule = kc * wk;
+                            const int c_full = round_up(d.C, granule);
+                            std::vector<int> cchs;
+                            for (int div : {1, 2, 4, 8}) {
+                                const int cch = round_up(ceil_div(d.C, div), granule);
+                                if (std::find(cchs.begin(), cchs.end(), cch) == cchs.end()) cchs.push_back(cch);
+                            }
+                            for (int fixed : {16, 32})
+                                if (fixed % granule == 0 && fixed < c_full &&
+                                    std::find(cchs.begin(), cchs.end(), fixed) == cchs.end())
+                                    cchs.push_back(fixed);
+                            for (int tw : tws)
+                                for (int cch : cchs) {
+                                    tdc_tile t{mf, mb, nb, wm, wn, wk, cch, tw};
+                                    Geometry g;
+                                    if (make_geometry(d, t, g, nullptr)) out.push_back(t);
+                                }
                         }
     }
     return out;

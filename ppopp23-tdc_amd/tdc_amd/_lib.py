@@ -37,20 +37,20 @@ class ConvDesc(Structure):
 
 
 class Tile(Structure):
-    _fields_ = [(n, c_int32) for n in ("mf", "mb", "nb", "wm", "wn", "wk", "cch")]
+    _fields_ = [(n, c_int32) for n in ("mf", "mb", "nb", "wm", "wn", "wk", "cch", "tw")]
 
     def astuple(self):
-        return (self.mf, self.mb, self.nb, self.wm, self.wn, self.wk, self.cch)
+        return (self.mf, self.mb, self.nb, self.wm, self.wn, self.wk, self.cch, self.tw)
 
     def __repr__(self):
-        return "Tile(mf=%d, mb=%d, nb=%d, wm=%d, wn=%d, wk=%d, cch=%d)" % self.astuple()
+        return "Tile(mf=%d, mb=%d, nb=%d, wm=%d, wn=%d, wk=%d, cch=%d, tw=%d)" % self.astuple()
 
 
 class TileInfo(Structure):
     _fields_ = [("tile", Tile)] + [(n, c_int32) for n in (
         "grid_x", "grid_y", "grid_z", "block_threads", "lds_bytes", "vgpr_estimate", "waves_per_simd",
-        "wg_per_cu", "nchunks")] + [(n, c_double) for n in ("flops", "bytes", "roof_us", "pred_us",
-                                                           "pred_hbm_bytes")]
+        "wg_per_cu", "nchunks", "th")] + [(n, c_double) for n in ("flops", "bytes", "roof_us", "pred_us",
+                                                                 "pred_l2_bytes")]
 
     def asdict(self):
         d = {n: getattr(self, n) for n, _ in self._fields_ if n != "tile"}
