@@ -82,51 +82,72 @@ enum : int { TAPS_GENERIC = 0, TAPS_1x1 = 1, TAPS_3x3 = 9 };
 
 constexpr int OOB_OFFSET = 0x7ffffff0;  // beyond any buffer: the load returns zero
 
-// Start the copies of one pass (input channels [c0, c0+CCH) and their weights)
-// into the LDS stage at `stage`.  Nothing is waited for here.
-//
-// Input: the stage holds [CCH][CS] floats, a channel slot being [nrows][RS]
-// (+ tail).  The slot is walked in E-byte elements; element e of the stage goes
-// to LDS position e, lane l of a copy instruction supplying element blk*64+l.
-// Weights: a linear copy of `wslab_floats` floats.
+__device__ __forceinline__ int fdiv(int n, const FastDiv &f) {
+    return f.d == 1 ? n : (int)__umulhi((unsigned)n, f.m);
+}
+
+// Copy planning.  A pass moves the input window of CCH channels and the weight
+// slab of those channels into one LDS stage.  The stage is cut into blocks of
+// 64 elements (E = 16 or 4 bytes each); one `buffer_load ... lds` instruction
+// fills one block, lane l supplying element l.  Blocks are dealt round-robin to
+// the waves.  Which input element belongs at a given LDS position does not
+// depend on the pass except for a constant byte offset (CCH channels further
+// on), so each lane works out the offsets of its first MAXPRE blocks once and
+// keeps them in registers; halo, padding and positions past the slab get an
+// out-of-range offset, which the buffer unit answers with zeros (channels past
+// C fall off the end of the image buffer the same way).
+constexpr int MAXPRE = 6;
+
+template <int E>
+__device__ __forceinline__ int input_copy_offset(const ConvKParams &p, int e, int iy0, int ix0a) {
+    constexpr int VW = E / 4;
+    const int rsv = p.fd_rsv.d;  // elements per LDS row
+    const int csv = p.fd_csv.d;  // elements per LDS channel slot
+    const int cl = fdiv(e, p.fd_csv);
+    const int rem = e - cl * csv;
+    const int row = fdiv(rem, p.fd_rsv);
+    const int xv = rem - row * rsv;
+    const int iy = iy0 + row;
+    const int ix = ix0a + xv * VW;
+    const bool inb = cl < p.CCH && row < p.nrows && iy >= 0 && iy < p.H && ix >= 0 && ix < p.W;
+    return inb ? ((cl * p.H + iy) * p.W + ix) * 4 : OOB_OFFSET;
+}
+
+template <int E>
+__device__ __forceinline__ void copy_block(__amdgpu_buffer_rsrc_t rsrc, float *dst, int voff, int soff) {
+    if constexpr (E == 16)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_ptr_t)dst, 16, voff, soff, 0, 0);
+    else
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_ptr_t)dst, 4, voff, soff, 0, 0);
+}
+
+// Start the copies of pass `chunk` into the LDS stage at `stage`.  Nothing is
+// waited for here.  Everything that does not depend on the lane is kept in
+// scalar registers: vector ALU instructions issued next to MFMAs are not free.
 template <int E>
 __device__ __forceinline__ void issue_pass(const ConvKParams &p, __amdgpu_buffer_rsrc_t in_rsrc,
                                            __amdgpu_buffer_rsrc_t w_rsrc, float *__restrict__ stage,
-                                           int c0, int iy0, int ix0a, unsigned w_byte0, int wave,
-                                           int nwaves, int lane) {
+                                           const int (&pre)[MAXPRE], int lane16, int chunk, int iy0, int ix0a,
+                                           int w_byte0, int wave, int nwaves, int lane) {
     constexpr int VW = E / 4;
-    const int rsv = p.RS / VW;  // elements per LDS row
-    const int csv = p.CS / VW;  // elements per LDS channel slot
-    const int total = p.CCH * csv;
-    const int nblk = (total + 63) >> 6;
-    for (int blk = wave; blk < nblk; blk += nwaves) {
-        const int e = (blk << 6) + lane;
-        const int cl = e / csv;
-        const int rem = e - cl * csv;
-        const int row = rem / rsv;
-        const int xv = rem - row * rsv;
-        const int c = c0 + cl;
-        const int iy = iy0 + row;
-        const int ix = ix0a + xv * VW;
-        const bool inb = c < p.C && row < p.nrows && iy >= 0 && iy < p.H && ix >= 0 && ix < p.W;
-        const int voff = inb ? ((c * p.H + iy) * p.W + ix) * 4 : OOB_OFFSET;
-        if (e < total) {
-            if constexpr (E == 16)
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(in_rsrc, (lds_ptr_t)(stage + (blk << 6) * VW), 16, voff, 0, 0, 0);
-            else
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(in_rsrc, (lds_ptr_t)(stage + (blk << 6) * VW), 4, voff, 0, 0, 0);
-        }
+    const int nblk = p.in_stage_floats / (64 * VW);
+    // This pass starts chunk*CCH channels further on.  The shift goes through the vector offset on
+    // purpose: only that one is range-checked, and channels past C must read as zero.
+    const int pass_bytes = chunk * p.CCH * p.H * p.W * 4;
+#pragma unroll
+    for (int i = 0; i < MAXPRE; ++i) {
+        const int blk = wave + i * nwaves;
+        if (blk < nblk) copy_block<E>(in_rsrc, stage + blk * 64 * VW, pre[i] + pass_bytes, 0);
     }
-    // Weights: 16-byte elements, 1 KiB per instruction.
+    for (int blk = wave + MAXPRE * nwaves; blk < nblk; blk += nwaves)
+        copy_block<E>(in_rsrc, stage + blk * 64 * VW,
+                      input_copy_offset<E>(p, (blk << 6) + lane, iy0, ix0a) + pass_bytes, 0);
+    // Weights: a linear copy in 16-byte elements, 1 KiB per instruction; always inside the packed buffer
+    // (or past its end, which reads as zero into the slack), so the block offset can ride in the scalar operand.
     float *wdst = stage + p.in_stage_floats;
-    const int wtotal = p.wslab_floats >> 2;
-    const int wnblk = (wtotal + 63) >> 6;
-    for (int blk = wave; blk < wnblk; blk += nwaves) {
-        const int e = (blk << 6) + lane;
-        if (e < wtotal)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(w_rsrc, (lds_ptr_t)(wdst + (blk << 8)), 16,
-                                                     (int)(w_byte0 + (unsigned)e * 16u), 0, 0, 0);
-    }
+    const int wnblk = (p.wslab_floats + 255) >> 8;
+    for (int blk = wave; blk < wnblk; blk += nwaves)
+        copy_block<16>(w_rsrc, wdst + (blk << 8), lane16, w_byte0 + (blk << 10));
 }
 
 template <int MF, int MB, int NB, int TAPS, int MAXW>
@@ -142,13 +163,14 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int nthreads = blockDim.x;
     const int nwaves = nthreads >> 6;
-    const int wk = wave % p.WK;
-    const int wn = (wave / p.WK) % p.WN;
-    const int wm = wave / (p.WK * p.WN);
+    const int wave_nk = fdiv(wave, p.fd_wk);  // wave = (wm * WN + wn) * WK + wk
+    const int wk = wave - wave_nk * p.WK;
+    const int wm = fdiv(wave_nk, p.fd_wn);
+    const int wn = wave_nk - wm * p.WN;
 
     const int PT = MF * NB * p.WN;  // pixel lanes of the workgroup (>= TH*TW)
     const int MT = MF * MB * p.WM;
-    const int tile_y = blockIdx.x / p.ntx;
+    const int tile_y = fdiv(blockIdx.x, p.fd_ntx);
     const int tile_x = blockIdx.x - tile_y * p.ntx;
     const int oy0 = tile_y * p.TH;
     const int ox0 = tile_x * p.TW;
@@ -171,14 +193,23 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
     const unsigned w_pass_bytes = (unsigned)p.wslab_floats * 4u;
     const unsigned w_byte_base = (unsigned)blockIdx.y * (unsigned)p.nchunks * w_pass_bytes;
 
+    // Offsets of this lane's elements in its wave's first MAXPRE input blocks (pass 0).
+    int pre[MAXPRE];
+#pragma unroll
+    for (int i = 0; i < MAXPRE; ++i) {
+        const int e = ((wave + i * nwaves) << 6) + lane;
+        pre[i] = OOB_OFFSET;
+        if (e < p.in_stage_floats)  // (in elements this bound is only tighter)
+            pre[i] = (p.VW == 4) ? input_copy_offset<16>(p, e, iy0, ix0a) : input_copy_offset<4>(p, e, iy0, ix0a);
+    }
+    const int lane16 = lane * 16;
     auto issue = [&](int chunk) {
         float *stage = lds + (chunk & (p.nstage - 1)) * p.stage_floats;
+        const int w_byte0 = (int)(w_byte_base + (unsigned)chunk * w_pass_bytes);
         if (p.VW == 4)
-            issue_pass<16>(p, in_rsrc, w_rsrc, stage, chunk * p.CCH, iy0, ix0a, w_byte_base + chunk * w_pass_bytes,
-                           wave, nwaves, lane);
+            issue_pass<16>(p, in_rsrc, w_rsrc, stage, pre, lane16, chunk, iy0, ix0a, w_byte0, wave, nwaves, lane);
         else
-            issue_pass<4>(p, in_rsrc, w_rsrc, stage, chunk * p.CCH, iy0, ix0a, w_byte_base + chunk * w_pass_bytes,
-                          wave, nwaves, lane);
+            issue_pass<4>(p, in_rsrc, w_rsrc, stage, pre, lane16, chunk, iy0, ix0a, w_byte0, wave, nwaves, lane);
     };
     issue(0);
 
@@ -187,7 +218,7 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
         const int j = (wn * NB + nb) * MF + M::col(lane);
-        int jy = j / p.TW;
+        int jy = fdiv(j, p.fd_tw);
         const int jx = j - jy * p.TW;
         jy = min(jy, p.TH - 1);  // lanes past the tile re-read its last row; they are never stored
         boff[nb] = jy * p.stride * p.RS + jx * p.stride + (ix0 - ix0a) + M::ksub(lane) * p.CS;
@@ -285,7 +316,7 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
             const int j = (wn * NB + nb) * MF + M::col(lane);
-            const int jy = j / p.TW;
+            const int jy = fdiv(j, p.fd_tw);
             const int jx = j - jy * p.TW;
             const int oy = oy0 + jy, ox = ox0 + jx;
             const bool pix_ok = jy < p.TH && oy < p.Ho && ox < p.Wo;
@@ -325,9 +356,9 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
         __syncthreads();
         const int total = MT * PT;
         for (int idx = tid; idx < total; idx += nthreads) {
-            const int ml = idx / PT;
+            const int ml = fdiv(idx, p.fd_pt);
             const int j = idx - ml * PT;
-            const int jy = j / p.TW;
+            const int jy = fdiv(j, p.fd_tw);
             const int jx = j - jy * p.TW;
             const int n = m0 + ml;
             const int oy = oy0 + jy, ox = ox0 + jx;

@@ -173,6 +173,13 @@ int tdc_conv_forward(tdc_conv_plan *plan, const float *d_in, const float *d_resi
     kp.in_stage_floats = g.in_stage_floats; kp.wslab_floats = g.wslab_floats;
     kp.stage_floats = g.stage_floats; kp.nstage = g.nstage;
     kp.relu = d.relu;
+    kp.fd_csv = make_fastdiv(g.CS / kp.VW);
+    kp.fd_rsv = make_fastdiv(g.RS / kp.VW);
+    kp.fd_tw = make_fastdiv(g.TW);
+    kp.fd_ntx = make_fastdiv(g.ntx);
+    kp.fd_pt = make_fastdiv(g.PT);
+    kp.fd_wk = make_fastdiv(plan->tile.wk);
+    kp.fd_wn = make_fastdiv(plan->tile.wn);
     kp.wpk_bytes = (unsigned)(packed_weight_floats(g) * sizeof(float));
     kp.in_bstride = (long long)d.C * d.H * d.W;
     kp.out_bstride = (long long)d.N * g.P;

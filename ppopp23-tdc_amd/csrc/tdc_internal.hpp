@@ -69,6 +69,20 @@ bool model_select(const tdc_conv_desc &d, tdc_tile_info &info, std::string *why)
 size_t packed_weight_floats(const Geometry &g);
 void pack_weights(const tdc_conv_desc &d, const tdc_tile &t, const Geometry &g, const float *w_oihw, float *packed);
 
+// Division of a small non-negative integer by a run-time constant as one
+// multiply-high: q = (n * m) >> 32 with m = floor(2^32 / d) + 1, exact whenever
+// n * d < 2^32.  d == 1 is passed through.
+struct FastDiv {
+    unsigned m;
+    int d;
+};
+inline FastDiv make_fastdiv(int d) {
+    FastDiv f;
+    f.d = d;
+    f.m = d > 1 ? (unsigned)((1ULL << 32) / (unsigned)d + 1ULL) : 0u;
+    return f;
+}
+
 // ---- kernel arguments ------------------------------------------------------
 struct ConvKParams {
     const float *in;
@@ -84,6 +98,9 @@ struct ConvKParams {
     int RS, CS, VW, nrows;
     int in_stage_floats, wslab_floats, stage_floats, nstage;
     int relu;
+    FastDiv fd_csv, fd_rsv;      // LDS channel slot / row, in copy elements
+    FastDiv fd_tw, fd_ntx, fd_pt;
+    FastDiv fd_wk, fd_wn;
     unsigned wpk_bytes;
     long long in_bstride;   // C*H*W
     long long out_bstride;  // N*P

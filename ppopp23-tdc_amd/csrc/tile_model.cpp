@@ -90,7 +90,9 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
     g.TH = std::min(g.PT / t.tw, g.Ho);
     g.ntx = ceil_div(g.Wo, g.TW);
     g.nty = ceil_div(g.Ho, g.TH);
-    if ((long long)g.ntx * g.nty > (1LL << 30)) return fail("grid too large");
+    // (the kernel divides the tile index by ntx with a 32-bit multiply-high)
+    if ((long long)g.ntx * g.nty > 65535 * 16) return fail("grid too large");
+    if ((long long)g.ntx * g.nty * g.ntx >= (1LL << 32)) return fail("grid too large");
     g.grid_x = g.ntx * g.nty;
     g.grid_y = ceil_div(d.N, g.MT);
     g.grid_z = d.batch;
@@ -118,15 +120,18 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
         g.RS = g.ncols;
     }
     g.CS = pad_channel_stride(g.nrows * g.RS, t.mf, g.VW);
-    g.in_stage_floats = round_up(t.cch * g.CS, 4);
+    // Copies are issued in whole blocks of 64 elements (1 KiB with 16-byte elements): both parts of
+    // a stage are rounded up to that, the slack receiving zeros.
+    g.in_stage_floats = round_up(t.cch * g.CS, 256);
     g.wslab_floats = (t.wm * t.mb) * (t.cch / g.kc) * g.taps * 64;
-    g.stage_floats = g.in_stage_floats + g.wslab_floats;
+    g.stage_floats = g.in_stage_floats + round_up(g.wslab_floats, 256);
     g.nstage = g.nchunks > 1 ? 2 : 1;
     const long long stage_bytes = (long long)g.nstage * g.stage_floats * 4;
     const long long red_bytes = t.wk > 1 ? (long long)t.wk * g.MT * g.PT * 4 : 0;
     const long long lds = std::max(stage_bytes, red_bytes);
     if (lds > machine().lds_bytes_per_cu) return fail("tile needs more than 160 KiB of LDS");
     g.lds_bytes = (int)lds;
+    if (const char *e = std::getenv("TDC_EXPERIMENT_MIN_LDS")) g.lds_bytes = std::max(g.lds_bytes, std::atoi(e));
     if ((long long)g.grid_y * g.nchunks * g.wslab_floats * 4 >= (1LL << 31)) return fail("packed weights exceed 2 GiB");
     return true;
 }
