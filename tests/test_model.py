@@ -1,0 +1,86 @@
+"""Host-side checks of the launch geometry and the analytic gfx950 tile model (no GPU needed)."""
+import math
+
+import pytest
+
+import tdc_amd
+from oracle import ref
+
+LDS_BYTES = 160 * 1024
+
+
+def conv3(c, n, hw, stride=1):
+    return tdc_amd.conv_desc(1, c, n, hw, hw, 3, 3, stride, 1)
+
+
+@pytest.mark.parametrize("hw", ref.SWEEP_HW)
+@pytest.mark.parametrize("r1,r2", ref.SWEEP_RANKS)
+def test_every_candidate_is_launchable_and_covers_the_output(hw, r1, r2):
+    d = conv3(r1, r2, hw)
+    tiles = tdc_amd.model_enumerate(d)
+    assert tiles, "no tile for a sweep shape"
+    for t in tiles[:: max(1, len(tiles) // 60)]:
+        i = tdc_amd.model_evaluate(d, t)
+        lanes = t.mf * t.nb * t.wn
+        assert 1 <= i.th and i.th * t.tw <= lanes
+        ntx, nty = math.ceil(hw / t.tw), math.ceil(hw / i.th)
+        assert i.grid_x == ntx * nty and ntx * t.tw >= hw and nty * i.th >= hw      # tiles cover the image
+        assert i.grid_y * t.mf * t.mb * t.wm >= r2                                   # ... and all channels
+        assert i.nchunks * t.cch >= r1 and t.cch % ((2 if t.mf == 32 else 4) * t.wk) == 0
+        assert i.block_threads == 64 * t.wm * t.wn * t.wk <= 1024
+        assert 0 < i.lds_bytes <= LDS_BYTES
+        assert i.wg_per_cu >= 1 and i.pred_us > 0
+
+
+def test_algorithmic_work_and_roofline_of_config1():
+    i = tdc_amd.model_select(conv3(32, 32, 56))
+    assert i.flops == 2 * 56 * 56 * 32 * 32 * 9 == 57802752
+    assert i.bytes == 4 * (32 * 56 * 56 + 32 * 56 * 56 + 9 * 32 * 32) == 839680
+    assert abs(i.roof_us - 57802752 / 157.3e6) < 1e-9          # fp32-bound: 0.367 us
+    big = tdc_amd.model_select(conv3(128, 128, 56))
+    assert abs(big.roof_us - 5.8795) < 1e-3
+    tiny = tdc_amd.model_select(conv3(16, 16, 7))
+    assert abs(tiny.roof_us - 15488 / 8e6) < 1e-9               # HBM-bound: 0.0019 us
+
+
+def test_select_is_argmin_of_the_enumeration():
+    d = conv3(64, 64, 28)
+    best = tdc_amd.model_select(d)
+    preds = [tdc_amd.model_evaluate(d, t).pred_us for t in tdc_amd.model_enumerate(d)]
+    assert best.pred_us == min(preds)
+
+
+def test_model_prefers_split_k_waves_for_tiny_layers_and_more_tiles_for_big_ones():
+    small = tdc_amd.model_select(conv3(128, 128, 7))
+    big = tdc_amd.model_select(conv3(128, 128, 56))
+    assert small.tile.wk >= 2                       # few pixels: parallelism has to come from input channels
+    assert big.grid_x * big.grid_y >= 128           # enough workgroups to spread over the 256 CUs
+    assert big.pred_us > small.pred_us
+
+
+def test_one_by_one_convolutions_run_on_the_flattened_image():
+    d = tdc_amd.conv_desc(1, 256, 64, 56, 56, 1, 1, 1, 0)
+    i = tdc_amd.model_select(d)
+    assert i.th == 1 and i.tile.tw == i.tile.mf * i.tile.nb * i.tile.wn     # a tile is a run of consecutive pixels
+    assert i.flops == 2 * 56 * 56 * 256 * 64
+
+
+def test_invalid_tiles_are_rejected():
+    d = conv3(32, 32, 14)
+    for t in [tdc_amd.Tile(8, 1, 1, 1, 1, 1, 32, 4),      # mf
+              tdc_amd.Tile(16, 3, 1, 1, 1, 1, 32, 4),     # mb
+              tdc_amd.Tile(16, 1, 1, 4, 4, 4, 32, 4),     # 64 waves
+              tdc_amd.Tile(16, 1, 1, 1, 1, 1, 30, 4),     # cch not a multiple of 4
+              tdc_amd.Tile(16, 1, 1, 1, 1, 1, 32, 15),    # tw wider than the image
+              tdc_amd.Tile(16, 1, 1, 1, 1, 1, 32, 0)]:
+        with pytest.raises(tdc_amd.TdcError):
+            tdc_amd.model_evaluate(d, t)
+    with pytest.raises(tdc_amd.TdcError):                  # LDS overflow
+        tdc_amd.model_evaluate(conv3(2048, 256, 56), tdc_amd.Tile(32, 2, 2, 2, 2, 1, 2048, 56))
+
+
+def test_stride2_and_stem_shapes_have_tiles():
+    for d in (conv3(64, 64, 56, 2), conv3(256, 256, 14, 2), tdc_amd.conv_desc(1, 3, 64, 224, 224, 7, 7, 2, 3),
+              tdc_amd.conv_desc(8, 64, 16, 56, 56, 3, 3, 1, 1)):
+        i = tdc_amd.model_select(d)
+        assert i.grid_x > 0 and i.lds_bytes <= LDS_BYTES
