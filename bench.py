@@ -24,6 +24,21 @@ sys.path.insert(0, ROOT)
 
 PEAK_FP32_TFLOPS = 157.3   # MI355X dense fp32 matrix peak
 PEAK_HBM_TBPS = 8.0
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "core_conv_128x128_56_hbm_traffic.txt")
+
+
+def measured_traffic(tile):
+    """HBM bytes per launch of the dominant kernel from the committed rocprofv3 --pmc summary
+    (FETCH_SIZE + WRITE_SIZE, scaled by a copy kernel of known size); None if it was taken with another tile."""
+    try:
+        for line in open(TRAFFIC_FILE):
+            if line.startswith("traffic_bytes_per_launch:"):
+                parts = line.split()
+                if [int(v) for v in parts[3].split(",")] == list(tile):
+                    return int(parts[1])
+    except (OSError, ValueError, IndexError):
+        pass
+    return None
 
 
 def main():
@@ -33,6 +48,11 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="issue launches on a plain stream instead of a HIP graph")
+    ap.add_argument("--only-dominant", action="store_true",
+                    help="profiling aid: launch only the dominant layer (128->128 @56), `steps` times, and exit")
+    ap.add_argument("--calibrate-copy", type=int, default=0, metavar="BYTES",
+                    help="profiling aid: run a plain device copy of BYTES bytes a few times (reference reading for "
+                         "the FETCH_SIZE / WRITE_SIZE counters) before anything else")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU; --gpus %d is not supported (single-GPU hot path, "
@@ -47,6 +67,23 @@ def main():
         sys.exit("bench.py needs a GPU")
     torch.cuda.set_device(0)
     graph = not a.no_graph
+
+    if a.calibrate_copy:
+        src = torch.empty(a.calibrate_copy // 4, device="cuda").normal_()
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+
+    if a.only_dominant:
+        x, w = ref.make_core_case(56, 128, 128)
+        plan = Conv2dPlan(1, 128, 128, 56, 56, 3, 3, 1, 1).set_weights(w)
+        xd, out = x.cuda(), torch.empty(1, 128, 56, 56, device="cuda")
+        for _ in range(a.steps):
+            plan.forward(xd, out=out)
+        torch.cuda.synchronize()
+        print(json.dumps({"only_dominant": True, "launches": a.steps, "tile": list(plan.info.tile.astuple())}))
+        return
 
     layers = []
     for hw in ref.SWEEP_HW:
@@ -101,6 +138,7 @@ def main():
         achieved = dinfo.bytes / dom_us * 1e-3     # GB/s
         roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_TBPS * 1e3, "unit": "GB/s",
                     "frac": round(achieved / (PEAK_HBM_TBPS * 1e3), 4), "traffic": None}
+    roofline["traffic"] = measured_traffic(dinfo.tile.astuple())
     roofline.update({"kernel": "core conv %d->%d @%dx%d" % (dl["r1"], dl["r2"], dl["hw"], dl["hw"]),
                      "avg_launch_us": round(dom_us, 3), "flops_per_launch": dinfo.flops,
                      "bytes_per_launch": dinfo.bytes, "timing": "hipEvents around 200 graph-replayed launches"})

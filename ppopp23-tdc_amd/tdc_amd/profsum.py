@@ -1,0 +1,92 @@
+"""Summarise rocprofv3 CSV output per (kernel, launch geometry).
+
+rocprofv3's own ``--stats`` table aggregates by kernel NAME, and one template
+instantiation of the convolution kernel serves many layer shapes; the launch
+geometry (grid, workgroup, LDS) is what tells the layers apart.
+
+    python -m tdc_amd.profsum kernel <dir-with-*_kernel_trace.csv>
+    python -m tdc_amd.profsum pmc    <dir-with-*_counter_collection.csv> [--copy-bytes N]
+
+``kernel``: count / mean / min / max duration in microseconds per (kernel, grid, workgroup, LDS).
+``pmc``: mean counter value per (kernel, grid, workgroup); with ``--copy-bytes N`` the FETCH_SIZE /
+WRITE_SIZE readings (KiB) of every kernel are also shown scaled by the reading of the largest
+copy kernel in the same run, which is known to read and write N bytes.
+"""
+from __future__ import annotations
+
+import argparse
+import collections
+import csv
+import glob
+import os
+import sys
+
+
+def _short(name):
+    name = name.replace("void tdc::", "").replace("(tdc::ConvKParams)", "")
+    return name if len(name) <= 60 else name[:57] + "..."
+
+
+def kernel_summary(path, out=sys.stdout):
+    files = sorted(glob.glob(os.path.join(path, "**", "*kernel_trace.csv"), recursive=True))
+    if not files:
+        raise SystemExit(f"no *kernel_trace.csv under {path}")
+    acc = collections.defaultdict(list)
+    for f in files:
+        for r in csv.DictReader(open(f)):
+            key = (_short(r["Kernel_Name"]), int(r["Grid_Size_X"]), int(r["Grid_Size_Y"]), int(r["Workgroup_Size_X"]),
+                   int(r.get("LDS_Block_Size", 0) or 0))
+            acc[key].append((int(r["End_Timestamp"]) - int(r["Start_Timestamp"])) * 1e-3)
+    rows = sorted(acc.items(), key=lambda kv: -sum(kv[1]))
+    out.write("%-60s %9s %6s %5s %7s %7s %9s %9s %9s\n" % ("kernel", "grid_x", "grid_y", "wg", "lds", "calls", "mean_us",
+                                                       "min_us", "max_us"))
+    for (name, gx, gy, wg, lds), v in rows:
+        out.write("%-60s %9d %6d %5d %7d %7d %9.3f %9.3f %9.3f\n" % (name, gx, gy, wg, lds, len(v), sum(v) / len(v), min(v),
+                                                                   max(v)))
+    return rows
+
+
+def pmc_summary(path, copy_bytes=None, out=sys.stdout):
+    files = sorted(glob.glob(os.path.join(path, "**", "*counter_collection.csv"), recursive=True))
+    if not files:
+        raise SystemExit(f"no *counter_collection.csv under {path}")
+    acc = collections.defaultdict(lambda: collections.defaultdict(list))
+    for f in files:
+        for r in csv.DictReader(open(f)):
+            key = (_short(r["Kernel_Name"]), int(r["Grid_Size"]), int(r["Workgroup_Size"]))
+            acc[key][r["Counter_Name"]].append(float(r["Counter_Value"]))
+    scale = {}
+    if copy_bytes:
+        # the biggest copy-like kernel of the run is the calibration copy
+        for cname in ("FETCH_SIZE", "WRITE_SIZE"):
+            best = 0.0
+            for (name, _, _), ctrs in acc.items():
+                if cname in ctrs and ("copy" in name.lower() or "elementwise" in name.lower()):
+                    best = max(best, max(ctrs[cname]))
+            if best > 0:
+                scale[cname] = copy_bytes / (best * 1024.0)
+                out.write("# %s of the %d-byte copy kernel: %.1f KiB -> 1 counted KiB = %.4f KiB moved\n" % (
+                    cname, copy_bytes, best, scale[cname]))
+    for (name, grid, wg), ctrs in sorted(acc.items(), key=lambda kv: -kv[0][1]):
+        for cname, v in sorted(ctrs.items()):
+            mean = sum(v) / len(v)
+            line = "%-60s grid %9d wg %5d  %-28s n=%5d mean=%16.2f" % (name, grid, wg, cname, len(v), mean)
+            if cname in scale:
+                line += "   scaled bytes/launch = %.0f" % (mean * 1024.0 * scale[cname])
+            out.write(line + "\n")
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser()
+    ap.add_argument("mode", choices=["kernel", "pmc"])
+    ap.add_argument("path")
+    ap.add_argument("--copy-bytes", type=int, default=None)
+    a = ap.parse_args(argv)
+    if a.mode == "kernel":
+        kernel_summary(a.path)
+    else:
+        pmc_summary(a.path, a.copy_bytes)
+
+
+if __name__ == "__main__":
+    main()
