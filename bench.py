@@ -47,6 +47,7 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end Tucker ResNet-18 forward")
     ap.add_argument("--no-graph", action="store_true", help="issue launches on a plain stream instead of a HIP graph")
     ap.add_argument("--only-dominant", action="store_true",
                     help="profiling aid: launch only the dominant layer (128->128 @56), `steps` times, and exit")
@@ -156,6 +157,28 @@ def main():
         "host_wall_ms_timed_region": round(wall_ms, 3),
     }
 
+    # -- end-to-end Tucker ResNet-18, batch 1, 3x224x224 (one HIP-graph launch per forward) ---------
+    e2e_params = e2e_x = None
+    if not a.no_e2e:
+        from tdc_amd import nets
+        from oracle import nets_ref
+        e2e_params = nets.resnet18_params(seed=18)
+        e2e_x = torch.randn(1, 3, 224, 224, generator=torch.Generator().manual_seed(18))
+        net = nets.build_tucker_resnet18(e2e_params, batch=1)
+        logits = net(e2e_x.cuda()).cpu().reshape(1, -1)
+        want = nets_ref.tucker_resnet18_forward(e2e_params, e2e_x)
+        err = float((logits - want).abs().max())
+        if not err <= 1e-5 + 1e-4 * float(want.abs().max()):
+            sys.exit("bench.py: end-to-end parity check failed (max err %g)" % err)
+        net.time_ms(iters=20)
+        e2e_ms = min(net.time_ms(iters=100) for _ in range(3))
+        out["tucker_resnet18_b1"] = {"ms": round(e2e_ms, 4), "kernels_per_forward": net.num_kernels,
+                                     "ms_eager_launches": round(net.time_ms(iters=50, graph=False), 4),
+                                     "max_abs_err_vs_cpu": err, "launch": "one HIP graph replay per forward",
+                                     "config": "ResNet-18 [2,2,2,2], every 3x3 conv = TKConv with R1=R2=planes/2, "
+                                               "BN folded, batch 1, fp32 3x224x224, random init seed 18"}
+        net.close()
+
     # -- CPU baseline: the reference operator's CPU path (F.conv2d), same layers --
     if not a.no_cpu_baseline:
         torch.set_num_threads(os.cpu_count() or 1)
@@ -173,6 +196,16 @@ def main():
                                "cores": torch.get_num_threads(), "kind": "port",
                                "sample": "%d passes over the same 28 layers with torch.nn.functional.conv2d fp32 on "
                                          "the host (the call the reference operator makes on CPU), ~10 s" % passes}
+        if e2e_params is not None:
+            from oracle import nets_ref
+            for _ in range(3):
+                nets_ref.tucker_resnet18_forward(e2e_params, e2e_x)
+            n, t0 = 0, time.perf_counter()
+            while time.perf_counter() - t0 < 5.0:
+                nets_ref.tucker_resnet18_forward(e2e_params, e2e_x)
+                n += 1
+            out["tucker_resnet18_b1"]["cpu_ms"] = round((time.perf_counter() - t0) * 1e3 / n, 3)
+            out["tucker_resnet18_b1"]["cpu_cores"] = torch.get_num_threads()
     print(json.dumps(out))
 
 

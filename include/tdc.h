@@ -20,6 +20,8 @@
  *   tdc_tkconv_*    TkConv::initialize / TkConv::forward (common.h:158-166,
  *                   src/BasicBlock.cu:14-31) and TKConv2dC.forward /
  *                   forward_features (inference/TKConv.py:90-106)
+ *   tdc_net_*       the E2E drivers and BasicBlock/Pool/Add/Concate layer objects
+ *                   (2080Ti-evaluation/EndToEnd/resnet18-tk/src/main.cu:19-156, inc/common.h:70-197)
  *   tdc_model_*     compute_latency / compute_*_vol / modeling
  *                   (2080Ti-evaluation/TDC-LAYERS-MODELING/model.py:136-156,209-235)
  *                   and the occupancy probe (2080Ti-evaluation/Gen-occupancy/template.cu:277-284)
@@ -155,6 +157,42 @@ int tdc_tkconv_core_forward(tdc_tkconv *op, const float *d_in, float *d_out, voi
 /* which: 0 = first 1x1, 1 = core, 2 = last 1x1 */
 int tdc_tkconv_query(const tdc_tkconv *op, int which, tdc_tile_info *info_out);
 void tdc_tkconv_destroy(tdc_tkconv *op);
+
+/* ---- whole-network forward graphs ----------------------------------------------
+ * A net is a list of operators over net-owned device tensors (tensor 0 is the
+ * input), captured into one HIP graph by tdc_net_finalize and replayed by
+ * tdc_net_forward.  Counterpart of the reference's native E2E drivers and layer
+ * objects (2080Ti-evaluation/EndToEnd/resnet18-tk/src/main.cu:19-156,
+ * src/BasicBlock.cu:14-50, inc/common.h:70-197): BatchNorm is expected folded into
+ * the weights/bias handed over, ReLU and the residual add ride in the
+ * convolution epilogues.  Weight pointers are HOST pointers; ids are tensor ids. */
+typedef struct tdc_net tdc_net;
+
+int tdc_net_create(int32_t batch, int32_t C, int32_t H, int32_t W, tdc_net **net_out);
+/* Dense convolution (also the classifier: a 1x1 convolution on a [C,1,1] tensor).  residual = -1 for none. */
+int tdc_net_conv(tdc_net *net, int32_t in, int32_t N, int32_t KH, int32_t KW, int32_t stride, int32_t pad,
+                 const float *w_oihw, const float *bias, int32_t residual, int32_t relu, int32_t *out);
+/* Tucker convolution 1x1 C->R1, KxK R1->R2 (stride, pad), 1x1 R2->N, then +bias, +residual, ReLU. */
+int tdc_net_tkconv(tdc_net *net, int32_t in, int32_t R1, int32_t R2, int32_t N, int32_t K, int32_t stride,
+                   int32_t pad, const float *first, const float *core, const float *last, const float *bias,
+                   int32_t residual, int32_t relu, int32_t *out);
+/* mode 0 = max, 1 = average (window count includes padding). */
+int tdc_net_pool(tdc_net *net, int32_t in, int32_t mode, int32_t k, int32_t stride, int32_t pad, int32_t *out);
+int tdc_net_global_avgpool(tdc_net *net, int32_t in, int32_t *out);
+/* Channel concatenation of n tensors of equal height/width. */
+int tdc_net_concat(tdc_net *net, const int32_t *ins, int32_t n, int32_t *out);
+int tdc_net_tensor_shape(const tdc_net *net, int32_t id, int32_t *C, int32_t *H, int32_t *W);
+int tdc_net_num_kernels(const tdc_net *net);
+/* Runs the net once eagerly, then captures it; `output_id` is what tdc_net_forward returns. */
+int tdc_net_finalize(tdc_net *net, int32_t output_id);
+/* d_in / d_out: device buffers copied to / from the net's own input / output tensors on `stream`
+ * (NULL = leave the net's tensors as they are).  Asynchronous. */
+int tdc_net_forward(tdc_net *net, const float *d_in, float *d_out, void *stream);
+/* hipEvents around `iters` forwards (graph replays, or eager launches when use_graph == 0); blocks. */
+int tdc_net_time(tdc_net *net, int32_t iters, int32_t use_graph, float *total_ms_out);
+/* Copy any tensor of the net to the host (synchronises the device). */
+int tdc_net_read_tensor(tdc_net *net, int32_t id, float *host_out);
+void tdc_net_destroy(tdc_net *net);
 
 /* ---- analytic gfx950 tile model (host only; works without a GPU) ---------- */
 

@@ -22,6 +22,11 @@ static int fail(tdc_status st, const std::string &msg) {
     return (int)st;
 }
 
+int api_fail(int status, const std::string &msg) {
+    set_error(msg);
+    return status;
+}
+
 static int hip_fail(const char *what, int err) {
     return fail(TDC_ERR_HIP, std::string(what) + ": " + hipGetErrorString((hipError_t)err));
 }

@@ -113,6 +113,13 @@ int prepare_conv_kernel(const void *fn, const Geometry &g);
 // Enqueue the kernel.  Returns a hipError_t as int.
 int launch_conv(const void *fn, const Geometry &g, const ConvKParams &kp, void *stream);
 
+// Pooling / concatenation kernels of the whole-network graphs (hipError_t as int).
+int launch_pool2d(const float *in, float *out, int planes, int H, int W, int Ho, int Wo, int k, int stride, int pad,
+                  int mode, void *stream);
+int launch_global_avgpool(const float *in, float *out, int planes, int HW, void *stream);
+int launch_copy_channels(const float *in, float *out, int B, int C, int HW, int Ctot, int c0, void *stream);
+
 void set_error(const std::string &msg);
+int api_fail(int status, const std::string &msg);   // records the message, returns status
 
 }  // namespace tdc

@@ -22,6 +22,9 @@ EXPORTS = (
     "tdc_tkconv_create", "tdc_tkconv_set_weights", "tdc_tkconv_forward", "tdc_tkconv_forward_features",
     "tdc_tkconv_core_forward", "tdc_tkconv_query", "tdc_tkconv_destroy",
     "tdc_model_evaluate", "tdc_model_enumerate", "tdc_model_select",
+    "tdc_net_create", "tdc_net_conv", "tdc_net_tkconv", "tdc_net_pool", "tdc_net_global_avgpool", "tdc_net_concat",
+    "tdc_net_tensor_shape", "tdc_net_num_kernels", "tdc_net_finalize", "tdc_net_forward", "tdc_net_time",
+    "tdc_net_read_tensor", "tdc_net_destroy",
 )
 
 
@@ -99,6 +102,21 @@ def lib():
     L.tdc_model_evaluate.argtypes = [POINTER(ConvDesc), POINTER(Tile), POINTER(TileInfo)]
     L.tdc_model_enumerate.argtypes = [POINTER(ConvDesc), POINTER(Tile), c_int32, POINTER(c_int32)]
     L.tdc_model_select.argtypes = [POINTER(ConvDesc), POINTER(TileInfo)]
+    i32, i32p, fpv = c_int32, POINTER(c_int32), c_void_p
+    L.tdc_net_create.argtypes = [i32, i32, i32, i32, POINTER(c_void_p)]
+    L.tdc_net_conv.argtypes = [c_void_p, i32, i32, i32, i32, i32, i32, fpv, fpv, i32, i32, i32p]
+    L.tdc_net_tkconv.argtypes = [c_void_p, i32, i32, i32, i32, i32, i32, i32, fpv, fpv, fpv, fpv, i32, i32, i32p]
+    L.tdc_net_pool.argtypes = [c_void_p, i32, i32, i32, i32, i32, i32p]
+    L.tdc_net_global_avgpool.argtypes = [c_void_p, i32, i32p]
+    L.tdc_net_concat.argtypes = [c_void_p, i32p, i32, i32p]
+    L.tdc_net_tensor_shape.argtypes = [c_void_p, i32, i32p, i32p, i32p]
+    L.tdc_net_num_kernels.argtypes = [c_void_p]
+    L.tdc_net_finalize.argtypes = [c_void_p, i32]
+    L.tdc_net_forward.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p]
+    L.tdc_net_time.argtypes = [c_void_p, i32, i32, POINTER(ctypes.c_float)]
+    L.tdc_net_read_tensor.argtypes = [c_void_p, i32, c_void_p]
+    L.tdc_net_destroy.argtypes = [c_void_p]
+    L.tdc_net_destroy.restype = None
     for name in EXPORTS:
         fn = getattr(L, name)
         if fn.restype is c_int:  # default restype: status code

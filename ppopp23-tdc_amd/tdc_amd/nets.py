@@ -1,0 +1,194 @@
+"""Whole-network forward graphs on the native library (tdc_net_*).
+
+``Net`` wraps the C handle.  ``build_tucker_resnet18`` lays out the reference's
+Tucker-compressed ResNet-18 (inference/resnet_inet_tt.py:53-117 ``TTBasicBlock``,
+:287-394 ``TTResNet`` with ``[2,2,2,2]`` blocks; every 3x3 convolution a
+``TKConv2dC``) from a state-dict-style parameter dictionary whose keys are the
+reference's (``layer1.0.conv1.first_kernel`` ...).  BatchNorm (inference mode) is
+folded into the weights and bias of the convolution in front of it at build time;
+ReLU and the residual add run in the convolution epilogues; the whole forward is
+one HIP-graph launch.
+"""
+from __future__ import annotations
+
+import ctypes
+import math
+from ctypes import byref, c_int32, c_void_p
+
+import torch
+
+from ._lib import check, lib
+
+BN_EPS = 1e-5
+
+
+def _h(t):
+    return None if t is None else t.detach().to(device="cpu", dtype=torch.float32).contiguous()
+
+
+def _p(t):
+    return None if t is None else c_void_p(t.data_ptr())
+
+
+class Net:
+    def __init__(self, batch, C, H, W):
+        self._h = c_void_p()
+        check(lib().tdc_net_create(batch, C, H, W, byref(self._h)))
+        self.batch = batch
+        self.input_id = 0
+        self.output_id = None
+        self._keep = []
+
+    def conv(self, x, weight, bias=None, stride=1, pad=0, residual=-1, relu=False):
+        w, b = _h(weight), _h(bias)
+        out = c_int32()
+        check(lib().tdc_net_conv(self._h, x, w.shape[0], w.shape[2], w.shape[3], stride, pad, _p(w), _p(b), residual,
+                                 int(relu), byref(out)))
+        return out.value
+
+    def tkconv(self, x, first, core, last, bias=None, stride=1, pad=0, residual=-1, relu=False):
+        f, c, l, b = _h(first), _h(core), _h(last), _h(bias)
+        out = c_int32()
+        check(lib().tdc_net_tkconv(self._h, x, f.shape[0], c.shape[0], l.shape[0], c.shape[2], stride, pad, _p(f), _p(c),
+                                   _p(l), _p(b), residual, int(relu), byref(out)))
+        return out.value
+
+    def pool(self, x, mode, k, stride, pad=0):
+        out = c_int32()
+        check(lib().tdc_net_pool(self._h, x, {"max": 0, "avg": 1}[mode], k, stride, pad, byref(out)))
+        return out.value
+
+    def global_avgpool(self, x):
+        out = c_int32()
+        check(lib().tdc_net_global_avgpool(self._h, x, byref(out)))
+        return out.value
+
+    def concat(self, ids):
+        arr = (c_int32 * len(ids))(*ids)
+        out = c_int32()
+        check(lib().tdc_net_concat(self._h, arr, len(ids), byref(out)))
+        return out.value
+
+    def shape(self, tid):
+        c, h, w = c_int32(), c_int32(), c_int32()
+        check(lib().tdc_net_tensor_shape(self._h, tid, byref(c), byref(h), byref(w)))
+        return (self.batch, c.value, h.value, w.value)
+
+    def finalize(self, output_id):
+        check(lib().tdc_net_finalize(self._h, output_id))
+        self.output_id = output_id
+        return self
+
+    @property
+    def num_kernels(self):
+        return lib().tdc_net_num_kernels(self._h)
+
+    def forward(self, x):
+        """x: device tensor [B,C,H,W]; returns a new device tensor with the output."""
+        if not x.is_cuda or x.dtype != torch.float32 or tuple(x.shape) != self.shape(0) or not x.is_contiguous():
+            raise ValueError(f"input must be a contiguous float32 device tensor of shape {self.shape(0)}")
+        out = torch.empty(self.shape(self.output_id), device=x.device, dtype=torch.float32)
+        s = c_void_p(torch.cuda.current_stream().cuda_stream)
+        check(lib().tdc_net_forward(self._h, c_void_p(x.data_ptr()), c_void_p(out.data_ptr()), s))
+        return out
+
+    __call__ = forward
+
+    def time_ms(self, iters=100, graph=True):
+        ms = ctypes.c_float(0.0)
+        check(lib().tdc_net_time(self._h, iters, int(graph), byref(ms)))
+        return ms.value / iters
+
+    def read(self, tid):
+        out = torch.empty(self.shape(tid), dtype=torch.float32)
+        check(lib().tdc_net_read_tensor(self._h, tid, c_void_p(out.data_ptr())))
+        return out
+
+    def close(self):
+        if self._h:
+            lib().tdc_net_destroy(self._h)
+            self._h = c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+# ---------------------------------------------------------------------------------------------------
+def bn_scale_shift(p, prefix):
+    """Inference-mode BatchNorm as y = x*scale + shift."""
+    scale = p[prefix + ".weight"] / torch.sqrt(p[prefix + ".running_var"] + BN_EPS)
+    shift = p[prefix + ".bias"] - p[prefix + ".running_mean"] * scale
+    return scale, shift
+
+
+def fold_dense(weight, scale):
+    return weight * scale.reshape(-1, 1, 1, 1)
+
+
+RESNET18_STAGES = ((64, 1), (128, 2), (256, 2), (512, 2))   # (planes, stride of the first block)
+
+
+def resnet18_params(seed=18, num_classes=1000, rank_ratio=0.5):
+    """Random-init Tucker ResNet-18 with the reference's state-dict key names: Kaiming-normal convolutions,
+    non-trivial BatchNorm statistics (so that the folding is exercised), ranks R1 = R2 = planes * rank_ratio."""
+    g = torch.Generator().manual_seed(seed)
+
+    def kaiming(*shape):
+        fan_in = shape[1] * shape[2] * shape[3]
+        return torch.empty(*shape).normal_(0, math.sqrt(2.0 / fan_in), generator=g)
+
+    def bn(prefix, n, p):
+        p[prefix + ".weight"] = torch.rand(n, generator=g) * 0.5 + 0.75
+        p[prefix + ".bias"] = torch.randn(n, generator=g) * 0.1
+        p[prefix + ".running_mean"] = torch.randn(n, generator=g) * 0.1
+        p[prefix + ".running_var"] = torch.rand(n, generator=g) * 0.5 + 0.75
+
+    p = {"conv1.weight": kaiming(64, 3, 7, 7)}
+    bn("bn1", 64, p)
+    inplanes = 64
+    for s, (planes, stride) in enumerate(RESNET18_STAGES, start=1):
+        r = int(planes * rank_ratio)
+        for b in range(2):
+            cin = inplanes if b == 0 else planes
+            for k, c in (("conv1", cin), ("conv2", planes)):
+                pre = f"layer{s}.{b}.{k}"
+                p[pre + ".first_kernel"] = kaiming(r, c, 1, 1)
+                p[pre + ".core_kernel"] = kaiming(r, r, 3, 3)
+                p[pre + ".last_kernel"] = kaiming(planes, r, 1, 1)
+                bn(f"layer{s}.{b}.bn{k[-1]}", planes, p)
+            if b == 0 and (stride != 1 or inplanes != planes):
+                p[f"layer{s}.0.downsample.0.weight"] = kaiming(planes, inplanes, 1, 1)
+                bn(f"layer{s}.0.downsample.1", planes, p)
+        inplanes = planes
+    p["fc.weight"] = torch.empty(num_classes, 512).normal_(0, 0.01, generator=g)
+    p["fc.bias"] = torch.randn(num_classes, generator=g) * 0.01
+    return p
+
+
+def build_tucker_resnet18(params, batch=1, H=224, W=224):
+    """Returns a finalized Net computing the logits [batch, num_classes, 1, 1]."""
+    p = params
+    net = Net(batch, 3, H, W)
+    s, t = bn_scale_shift(p, "bn1")
+    x = net.conv(0, fold_dense(p["conv1.weight"], s), t, stride=2, pad=3, relu=True)      # conv1 + bn1 + relu
+    x = net.pool(x, "max", 3, 2, 1)
+    for st, (planes, stride) in enumerate(RESNET18_STAGES, start=1):
+        for b in range(2):
+            pre = f"layer{st}.{b}"
+            blk_stride = stride if b == 0 else 1
+            identity = x
+            if pre + ".downsample.0.weight" in p:
+                ds, dt = bn_scale_shift(p, pre + ".downsample.1")
+                identity = net.conv(x, fold_dense(p[pre + ".downsample.0.weight"], ds), dt, stride=blk_stride)
+            s1, t1 = bn_scale_shift(p, pre + ".bn1")
+            y = net.tkconv(x, p[pre + ".conv1.first_kernel"], p[pre + ".conv1.core_kernel"],
+                           fold_dense(p[pre + ".conv1.last_kernel"], s1), t1, stride=blk_stride, pad=1, relu=True)
+            s2, t2 = bn_scale_shift(p, pre + ".bn2")
+            x = net.tkconv(y, p[pre + ".conv2.first_kernel"], p[pre + ".conv2.core_kernel"],
+                           fold_dense(p[pre + ".conv2.last_kernel"], s2), t2, stride=1, pad=1, residual=identity, relu=True)
+    x = net.global_avgpool(x)
+    x = net.conv(x, p["fc.weight"].reshape(p["fc.weight"].shape[0], -1, 1, 1), p["fc.bias"])
+    return net.finalize(x)

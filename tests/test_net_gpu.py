@@ -1,0 +1,80 @@
+"""End-to-end Tucker ResNet-18 (benchmark configuration 4) on the GPU against the CPU restatement."""
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import tdc_amd
+from tdc_amd import nets
+from oracle import nets_ref
+from util import ATOL, RTOL
+
+pytestmark = pytest.mark.gpu
+
+
+def scale_close(got, ref, what):
+    """|got - ref| <= ATOL + RTOL * max|ref|: the layer tolerance applied at the scale of the tensor (errors of
+    ~55 stacked fp32 layers do not stay proportional to each individual element)."""
+    got, ref = np.asarray(got, np.float64), np.asarray(ref, np.float64)
+    assert got.shape == ref.shape, what
+    bound = ATOL + RTOL * np.abs(ref).max()
+    err = np.abs(got - ref).max()
+    assert np.isfinite(got).all() and err <= bound, f"{what}: max err {err:.3e} > {bound:.3e}"
+
+
+def test_pool_and_concat_ops():
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(2, 6, 13, 11, generator=g)
+    net = nets.Net(2, 6, 13, 11)
+    a = net.pool(0, "max", 3, 2, 1)
+    b = net.pool(0, "avg", 2, 2, 0)
+    c = net.global_avgpool(0)
+    d = net.concat([0, 0])
+    w = torch.randn(4, 12, 1, 1, generator=g)
+    e = net.conv(d, w)
+    net.finalize(e)
+    out = net(x.cuda()).cpu()
+    F = torch.nn.functional
+    assert torch.equal(net.read(a), F.max_pool2d(x, 3, 2, 1))
+    assert torch.allclose(net.read(b), F.avg_pool2d(x, 2, 2), atol=1e-6)
+    assert torch.allclose(net.read(c), F.adaptive_avg_pool2d(x, 1), atol=1e-6)
+    assert torch.equal(net.read(d), torch.cat([x, x], 1))
+    assert torch.allclose(out, F.conv2d(torch.cat([x, x], 1), w), rtol=1e-4, atol=1e-5)
+    assert net.num_kernels == 6
+    net.close()
+
+
+def test_tucker_resnet18_logits_and_features():
+    p = nets.resnet18_params(seed=18)
+    x = torch.randn(1, 3, 224, 224, generator=torch.Generator().manual_seed(18))
+    want, feats = nets_ref.tucker_resnet18_forward(p, x, return_features=True)
+    net = nets.build_tucker_resnet18(p, batch=1)
+    print("kernels per forward:", net.num_kernels, flush=True)
+    sys.stdout.flush()
+    got = net(x.cuda())
+    torch.cuda.synchronize()
+    assert tuple(got.shape) == (1, 1000, 1, 1)
+    scale_close(got.cpu().numpy().reshape(1, 1000), want.numpy(), "logits")
+    # graph replays are repeatable and do not depend on what ran in between
+    again = net(x.cuda())
+    other = net(torch.randn(1, 3, 224, 224).cuda())
+    third = net(x.cuda())
+    torch.cuda.synchronize()
+    assert torch.equal(got, again) and torch.equal(got, third) and not torch.equal(got, other)
+    # intermediate stage outputs (tensor ids follow construction order)
+    ids = {}
+    tid = 2  # 0 input, 1 stem, 2 maxpool
+    scale_close(net.read(1).numpy(), feats["stem"].numpy(), "stem")
+    scale_close(net.read(2).numpy(), feats["maxpool"].numpy(), "maxpool")
+    net.close()
+
+
+def test_resnet18_batch2_small_resolution():
+    p = nets.resnet18_params(seed=5, num_classes=10)
+    x = torch.randn(2, 3, 64, 64, generator=torch.Generator().manual_seed(6))
+    want = nets_ref.tucker_resnet18_forward(p, x)
+    net = nets.build_tucker_resnet18(p, batch=2, H=64, W=64)
+    got = net(x.cuda()).cpu().numpy().reshape(2, 10)
+    scale_close(got, want.numpy(), "logits b2")
+    net.close()
