@@ -98,9 +98,8 @@ __device__ __forceinline__ int fdiv(int n, const FastDiv &f) {
 // C fall off the end of the image buffer the same way).
 constexpr int MAXPRE = 6;
 
-template <int E>
 __device__ __forceinline__ int input_copy_offset(const ConvKParams &p, int e, int iy0, int ix0a) {
-    constexpr int VW = E / 4;
+    const int VW = p.VW;
     const int rsv = p.fd_rsv.d;  // elements per LDS row
     const int csv = p.fd_csv.d;  // elements per LDS channel slot
     const int cl = fdiv(e, p.fd_csv);
@@ -109,13 +108,15 @@ __device__ __forceinline__ int input_copy_offset(const ConvKParams &p, int e, in
     const int xv = rem - row * rsv;
     const int iy = iy0 + row;
     const int ix = ix0a + xv * VW;
-    const bool inb = cl < p.CCH && row < p.nrows && iy >= 0 && iy < p.H && ix >= 0 && ix < p.W;
-    return inb ? ((cl * p.H + iy) * p.W + ix) * 4 : OOB_OFFSET;
+    // Branch-free: unsigned compares fold the lower bounds in.
+    const bool inb = (cl < p.CCH) & (row < p.nrows) & ((unsigned)iy < (unsigned)p.H) & ((unsigned)ix < (unsigned)p.W);
+    const int off = ((cl * p.H + iy) * p.W + ix) * 4;
+    return inb ? off : OOB_OFFSET;
 }
 
-template <int E>
-__device__ __forceinline__ void copy_block(__amdgpu_buffer_rsrc_t rsrc, float *dst, int voff, int soff) {
-    if constexpr (E == 16)
+// One `buffer_load ... lds`: 64 elements of `vw` floats each from rsrc[voff + soff] to dst.
+__device__ __forceinline__ void copy_block(int vw, __amdgpu_buffer_rsrc_t rsrc, float *dst, int voff, int soff) {
+    if (vw == 4)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_ptr_t)dst, 16, voff, soff, 0, 0);
     else
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_ptr_t)dst, 4, voff, soff, 0, 0);
@@ -124,30 +125,28 @@ __device__ __forceinline__ void copy_block(__amdgpu_buffer_rsrc_t rsrc, float *d
 // Start the copies of pass `chunk` into the LDS stage at `stage`.  Nothing is
 // waited for here.  Everything that does not depend on the lane is kept in
 // scalar registers: vector ALU instructions issued next to MFMAs are not free.
-template <int E>
 __device__ __forceinline__ void issue_pass(const ConvKParams &p, __amdgpu_buffer_rsrc_t in_rsrc,
                                            __amdgpu_buffer_rsrc_t w_rsrc, float *__restrict__ stage,
                                            const int (&pre)[MAXPRE], int lane16, int chunk, int iy0, int ix0a,
                                            int w_byte0, int wave, int nwaves, int lane) {
-    constexpr int VW = E / 4;
-    const int nblk = p.in_stage_floats / (64 * VW);
+    const int VW = p.VW;
+    const int blk_floats = 64 * VW;
+    const int nblk = p.in_stage_floats / blk_floats;
     // This pass starts chunk*CCH channels further on.  The shift goes through the vector offset on
     // purpose: only that one is range-checked, and channels past C must read as zero.
     const int pass_bytes = chunk * p.CCH * p.H * p.W * 4;
 #pragma unroll
     for (int i = 0; i < MAXPRE; ++i) {
         const int blk = wave + i * nwaves;
-        if (blk < nblk) copy_block<E>(in_rsrc, stage + blk * 64 * VW, pre[i] + pass_bytes, 0);
+        if (blk < nblk) copy_block(VW, in_rsrc, stage + blk * blk_floats, pre[i] + pass_bytes, 0);
     }
     for (int blk = wave + MAXPRE * nwaves; blk < nblk; blk += nwaves)
-        copy_block<E>(in_rsrc, stage + blk * 64 * VW,
-                      input_copy_offset<E>(p, (blk << 6) + lane, iy0, ix0a) + pass_bytes, 0);
+        copy_block(VW, in_rsrc, stage + blk * blk_floats, input_copy_offset(p, (blk << 6) + lane, iy0, ix0a) + pass_bytes, 0);
     // Weights: a linear copy in 16-byte elements, 1 KiB per instruction; always inside the packed buffer
     // (or past its end, which reads as zero into the slack), so the block offset can ride in the scalar operand.
     float *wdst = stage + p.in_stage_floats;
     const int wnblk = (p.wslab_floats + 255) >> 8;
-    for (int blk = wave; blk < wnblk; blk += nwaves)
-        copy_block<16>(w_rsrc, wdst + (blk << 8), lane16, w_byte0 + (blk << 10));
+    for (int blk = wave; blk < wnblk; blk += nwaves) copy_block(4, w_rsrc, wdst + (blk << 8), lane16, w_byte0 + (blk << 10));
 }
 
 template <int MF, int MB, int NB, int TAPS, int MAXW>
@@ -158,6 +157,13 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
     constexpr int NACC = M::NACC;
     extern __shared__ __align__(16) float lds[];
 
+    // Fetch every kernel argument the prologue needs in one go: left alone, the compiler loads them in
+    // several dependent batches, each costing a scalar-cache round trip before the first copy can start.
+    asm volatile("" ::"s"(p.in), "s"(p.wpk), "s"(p.H), "s"(p.W), "s"(p.CCH), "s"(p.nrows), "s"(p.TW), "s"(p.TH),
+                 "s"(p.ntx), "s"(p.stride), "s"(p.pad), "s"(p.VW), "s"(p.in_stage_floats), "s"(p.wslab_floats),
+                 "s"(p.stage_floats), "s"(p.nstage), "s"(p.nchunks), "s"(p.fd_csv.m), "s"(p.fd_csv.d),
+                 "s"(p.fd_rsv.m), "s"(p.fd_rsv.d), "s"(p.fd_ntx.m), "s"(p.fd_wk.m), "s"(p.fd_wn.m), "s"(p.WK),
+                 "s"(p.WN), "s"(p.in_bstride), "s"(p.wpk_bytes));
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -200,16 +206,13 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
         const int e = ((wave + i * nwaves) << 6) + lane;
         pre[i] = OOB_OFFSET;
         if (e < p.in_stage_floats)  // (in elements this bound is only tighter)
-            pre[i] = (p.VW == 4) ? input_copy_offset<16>(p, e, iy0, ix0a) : input_copy_offset<4>(p, e, iy0, ix0a);
+            pre[i] = input_copy_offset(p, e, iy0, ix0a);
     }
     const int lane16 = lane * 16;
     auto issue = [&](int chunk) {
         float *stage = lds + (chunk & (p.nstage - 1)) * p.stage_floats;
         const int w_byte0 = (int)(w_byte_base + (unsigned)chunk * w_pass_bytes);
-        if (p.VW == 4)
-            issue_pass<16>(p, in_rsrc, w_rsrc, stage, pre, lane16, chunk, iy0, ix0a, w_byte0, wave, nwaves, lane);
-        else
-            issue_pass<4>(p, in_rsrc, w_rsrc, stage, pre, lane16, chunk, iy0, ix0a, w_byte0, wave, nwaves, lane);
+        issue_pass(p, in_rsrc, w_rsrc, stage, pre, lane16, chunk, iy0, ix0a, w_byte0, wave, nwaves, lane);
     };
     issue(0);
 
@@ -251,42 +254,82 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
             sw[mb] = stage + p.in_stage_floats + (((wm * MB + mb) * ncg_pass + wk * ncgw) * taps) * 64 + lane;
 
         if constexpr (TAPS == TAPS_3x3) {
-            // dilation 1: the column tap is an immediate offset of the LDS read,
-            // the row tap one of three per-lane row addresses.
-#pragma unroll 2
-            for (int g = 0; g < ncgw; ++g) {
+            // dilation 1: the column tap is an immediate offset of the LDS read, the row tap one of
+            // three per-lane row addresses.  Two register sets ping-pong: the operands of channel
+            // group g+1 are read from LDS before the MFMAs of group g are issued, so the matrix pipe
+            // does not wait for LDS latency (one group is 9*MB*NB MFMAs deep).  The scheduling
+            // barriers keep the compiler from sinking the reads back to their first use.
+            float a0[9][MB], b0[9][NB], a1[9][MB], b1[9][NB];
+            auto load_group = [&](int g, float(&a)[9][MB], float(&b)[9][NB]) {
                 const float *lgrp = sin + g * KC * p.CS;
 #pragma unroll
                 for (int r = 0; r < 3; ++r) {
-                    const float *lrow[NB];
 #pragma unroll
-                    for (int nb = 0; nb < NB; ++nb) lrow[nb] = lgrp + boff[nb] + r * p.RS;
+                    for (int nb = 0; nb < NB; ++nb) {
+                        const float *lrow = lgrp + boff[nb] + r * p.RS;
 #pragma unroll
-                    for (int s = 0; s < 3; ++s) {
-                        float a[MB], b[NB];
+                        for (int s = 0; s < 3; ++s) b[r * 3 + s][nb] = lrow[s];
+                    }
+                }
 #pragma unroll
-                        for (int mb = 0; mb < MB; ++mb) a[mb] = sw[mb][(g * 9 + r * 3 + s) * 64];
+                for (int t = 0; t < 9; ++t)
 #pragma unroll
-                        for (int nb = 0; nb < NB; ++nb) b[nb] = lrow[nb][s];
+                    for (int mb = 0; mb < MB; ++mb) a[t][mb] = sw[mb][(g * 9 + t) * 64];
+            };
+            auto mfma_group = [&](const float(&a)[9][MB], const float(&b)[9][NB]) {
+#pragma unroll
+                for (int t = 0; t < 9; ++t)
+#pragma unroll
+                    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                        for (int nb = 0; nb < NB; ++nb) acc[mb][nb] = M::run(a[t][mb], b[t][nb], acc[mb][nb]);
+            };
+            load_group(0, a0, b0);
+            for (int g = 0; g < ncgw; g += 2) {
+                load_group(min(g + 1, ncgw - 1), a1, b1);
+                __builtin_amdgcn_sched_barrier(0);
+                mfma_group(a0, b0);
+                __builtin_amdgcn_sched_barrier(0);
+                load_group(min(g + 2, ncgw - 1), a0, b0);
+                __builtin_amdgcn_sched_barrier(0);
+                if (g + 1 < ncgw) mfma_group(a1, b1);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        } else if constexpr (TAPS == TAPS_1x1) {
+            // Same ping-pong, a group being four K-steps (channel groups).
+            constexpr int G = 4;
+            float a0[G][MB], b0[G][NB], a1[G][MB], b1[G][NB];
+            auto load_group = [&](int g0, float(&a)[G][MB], float(&b)[G][NB]) {
+#pragma unroll
+                for (int t = 0; t < G; ++t) {
+                    const int g = min(g0 + t, ncgw - 1);
+#pragma unroll
+                    for (int mb = 0; mb < MB; ++mb) a[t][mb] = sw[mb][g * 64];
+#pragma unroll
+                    for (int nb = 0; nb < NB; ++nb) b[t][nb] = sin[g * KC * p.CS + boff[nb]];
+                }
+            };
+            auto mfma_group = [&](int g0, const float(&a)[G][MB], const float(&b)[G][NB]) {
+#pragma unroll
+                for (int t = 0; t < G; ++t) {
+                    if (g0 + t < ncgw) {
 #pragma unroll
                         for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-                            for (int nb = 0; nb < NB; ++nb) acc[mb][nb] = M::run(a[mb], b[nb], acc[mb][nb]);
+                            for (int nb = 0; nb < NB; ++nb) acc[mb][nb] = M::run(a[t][mb], b[t][nb], acc[mb][nb]);
                     }
                 }
-            }
-        } else if constexpr (TAPS == TAPS_1x1) {
-#pragma unroll 4
-            for (int g = 0; g < ncgw; ++g) {
-                float a[MB], b[NB];
-#pragma unroll
-                for (int mb = 0; mb < MB; ++mb) a[mb] = sw[mb][g * 64];
-#pragma unroll
-                for (int nb = 0; nb < NB; ++nb) b[nb] = sin[g * KC * p.CS + boff[nb]];
-#pragma unroll
-                for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-                    for (int nb = 0; nb < NB; ++nb) acc[mb][nb] = M::run(a[mb], b[nb], acc[mb][nb]);
+            };
+            load_group(0, a0, b0);
+            for (int g0 = 0; g0 < ncgw; g0 += 2 * G) {
+                load_group(min(g0 + G, ncgw - 1), a1, b1);
+                __builtin_amdgcn_sched_barrier(0);
+                mfma_group(g0, a0, b0);
+                __builtin_amdgcn_sched_barrier(0);
+                load_group(min(g0 + 2 * G, ncgw - 1), a0, b0);
+                __builtin_amdgcn_sched_barrier(0);
+                mfma_group(g0 + G, a1, b1);
+                __builtin_amdgcn_sched_barrier(0);
             }
         } else {
             // Any filter size / dilation: taps walked at run time.
