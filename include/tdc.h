@@ -205,6 +205,12 @@ int tdc_model_enumerate(const tdc_conv_desc *desc, tdc_tile *tiles_out, int32_t 
                         int32_t *count_out);
 /* The model's pick = argmin pred_us over tdc_model_enumerate. */
 int tdc_model_select(const tdc_conv_desc *desc, tdc_tile_info *info_out);
+/* Calibration constants of the latency model (launch floor, copy latency and rate, barrier cost, ...;
+ * the counterpart of num_sm / num_threads / a,b,c / ratio in the reference's model.py:265-266,278).
+ * get: writes up to `cap` values, *count_out = how many there are.  set: all of them, all > 0;
+ * process-wide, not thread-safe against concurrent model calls. */
+int tdc_model_get_constants(double *values_out, int32_t cap, int32_t *count_out);
+int tdc_model_set_constants(const double *values, int32_t count);
 
 #ifdef __cplusplus
 }

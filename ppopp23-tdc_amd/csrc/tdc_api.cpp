@@ -90,6 +90,18 @@ int tdc_model_select(const tdc_conv_desc *desc, tdc_tile_info *info_out) {
     return TDC_OK;
 }
 
+int tdc_model_get_constants(double *out, int32_t cap, int32_t *count_out) {
+    if (!count_out || (cap > 0 && !out)) return fail(TDC_ERR_INVALID, "null argument");
+    *count_out = model_constants(out, cap);
+    return TDC_OK;
+}
+
+int tdc_model_set_constants(const double *values, int32_t count) {
+    if (!values) return fail(TDC_ERR_INVALID, "null argument");
+    if (!model_set_constants(values, count)) return fail(TDC_ERR_INVALID, "wrong number of constants, or a non-positive one");
+    return TDC_OK;
+}
+
 int tdc_conv_plan_create(const tdc_conv_desc *desc, const tdc_tile *forced_tile, tdc_conv_plan **plan_out) {
     if (!desc || !plan_out) return fail(TDC_ERR_INVALID, "null argument");
     *plan_out = nullptr;

@@ -61,6 +61,8 @@ bool check_desc(const tdc_conv_desc &d, std::string *why);
 bool model_evaluate(const tdc_conv_desc &d, const tdc_tile &t, tdc_tile_info &info, std::string *why);
 std::vector<tdc_tile> model_enumerate(const tdc_conv_desc &d);
 bool model_select(const tdc_conv_desc &d, tdc_tile_info &info, std::string *why);
+int model_constants(double *out, int cap);            // returns the number of constants
+bool model_set_constants(const double *in, int n);
 
 // ---- weight packing --------------------------------------------------------
 // OIHW [N,C,KH,KW] -> [channel tile][pass][M block in tile][channel group in pass][tap][64 lanes]

@@ -162,17 +162,43 @@ void pack_weights(const tdc_conv_desc &d, const tdc_tile &t, const Geometry &g, 
 // ---------------------------------------------------------------------------
 namespace {
 
+// Calibration constants of the latency model.  The defaults were fitted to a measured sweep of every
+// launchable tile of the 28 benchmark layers on one MI355X (python -m tdc_amd.fit_model); they can be
+// replaced at run time through tdc_model_set_constants, e.g. for another CDNA part.  They play the role
+// of num_sm / num_threads / the (a, b, c) weights / the keep-ratio in the reference's model
+// (2080Ti-evaluation/TDC-LAYERS-MODELING/model.py:265-266,278).
 struct ModelConst {
     double launch_us = 1.7;           // device time of an empty kernel in a back-to-back stream
-    double setup_clk = 900;           // kernel arguments, index arithmetic before the first copy is issued
-    double copy_latency_clk = 2200;   // first byte of a global->LDS copy (L2 / memory-side cache)
-    double copy_bytes_per_clk = 48;   // sustained global->LDS rate of one CU
-    double l2_bytes_per_clk = 3600;   // whole-chip L2->CU rate when every CU copies at once
-    double lds_bytes_per_clk = 128;
-    double sync_clk = 120;
-    double store_bytes_per_clk = 32;  // per CU, short runs per channel
+    double setup_clk = 1530;          // kernel arguments and index arithmetic before the first copy is issued
+    double copy_latency_clk = 1734;   // first byte of a global->LDS copy (L2 / memory-side cache)
+    double copy_bytes_per_clk = 30.2;   // sustained global->LDS rate of one CU
+    double l2_bytes_per_clk = 8640;   // whole-chip L2->CU rate when every CU copies at once
+    double lds_bytes_per_clk = 38.8;   // LDS traffic of the split-K reduction
+    double sync_clk = 127.5;            // one workgroup barrier
+    double store_bytes_per_clk = 5.2;  // per CU, short runs per channel
+    double kstep_issue_clk = 4.35;       // vector-ALU / LDS-issue cycles per operand read, not hidden under MFMAs
+    double pass_overhead_clk = 424;   // per wave and pass: copy issue, pointer set-up, pipeline fill
+    double wave_setup_clk = 2.2;      // prologue cycles added per extra wave sharing a SIMD
 };
-const ModelConst MC;
+ModelConst MC;
+constexpr int kNumModelConst = 11;
+
+double *mc_field(int i) {
+    switch (i) {
+        case 0: return &MC.launch_us;
+        case 1: return &MC.setup_clk;
+        case 2: return &MC.copy_latency_clk;
+        case 3: return &MC.copy_bytes_per_clk;
+        case 4: return &MC.l2_bytes_per_clk;
+        case 5: return &MC.lds_bytes_per_clk;
+        case 6: return &MC.sync_clk;
+        case 7: return &MC.store_bytes_per_clk;
+        case 8: return &MC.kstep_issue_clk;
+        case 9: return &MC.pass_overhead_clk;
+        case 10: return &MC.wave_setup_clk;
+        default: return nullptr;
+    }
+}
 
 // Registers per lane of the instantiated kernels, rounded up to the allocation granule of 8.
 int kernel_vgprs(const tdc_tile &t, int taps_mode) {
@@ -227,26 +253,26 @@ bool model_evaluate(const tdc_conv_desc &d, const tdc_tile &t, tdc_tile_info &in
     // One wave's matrix-core time per pass; the LDS reads of a K-step (one A and
     // one B word per lane per block row/column) must fit under it.
     const double mfma_pass = ksteps_pass * t.mb * t.nb * mfma_clk;
-    const double ldsrd_pass = ksteps_pass * (t.mb + t.nb) * 256.0 / MC.lds_bytes_per_clk;
     const double copy_bytes_pass = (double)g.stage_floats * 4.0;
     const double red_bytes = t.wk > 1 ? (double)t.wk * g.MT * g.PT * 4.0 * 2.0 : 0.0;
     const double out_bytes = (double)g.MT * g.PT * 4.0;
 
     auto wg_time = [&](int r, long long concurrent_wgs) {
-        // r workgroups share one CU: matrix time adds up per SIMD, LDS reads over the CU, copies share
-        // the CU's fill rate and, chip-wide, the L2.
-        const double compute =
-            std::max(mfma_pass * wg_waves_per_simd * r, ldsrd_pass * g.waves * r) + 2 * MC.sync_clk;
+        // r workgroups share one CU: matrix time and the issue cycles of the operand reads add up per
+        // SIMD; copies share the CU's fill rate and, chip-wide, the L2.
+        const double waves_simd = (double)wg_waves_per_simd * r;
+        const double per_wave = mfma_pass + ksteps_pass * (t.mb + t.nb) * MC.kstep_issue_clk + MC.pass_overhead_clk;
+        const double compute = per_wave * waves_simd + MC.sync_clk;
         const double chip_share =
             MC.l2_bytes_per_clk / std::max<double>(1.0, (double)std::min<long long>(concurrent_wgs, m.cus));
         const double rate = std::min(MC.copy_bytes_per_clk, chip_share);
         const double copy = copy_bytes_pass * r / rate;
         // First pass is exposed; afterwards the copy of pass i+1 runs under the MFMAs of pass i.
-        double clk = MC.setup_clk + MC.copy_latency_clk + copy;
+        double clk = MC.setup_clk + MC.wave_setup_clk * (waves_simd - 1.0) + MC.copy_latency_clk + copy;
         clk += compute;  // last pass: nothing left to hide
-        if (g.nchunks > 1) clk += (g.nchunks - 1) * std::max(compute, copy + 0.35 * MC.copy_latency_clk);
+        if (g.nchunks > 1) clk += (g.nchunks - 1) * std::max(compute, copy + MC.copy_latency_clk);
         clk += red_bytes * r / MC.lds_bytes_per_clk + out_bytes * r / MC.store_bytes_per_clk +
-               (t.wk > 1 ? 2.0 * MC.sync_clk : 0.0) + 400.0;
+               (t.wk > 1 ? 2.0 * MC.sync_clk : 0.0);
         return clk;
     };
     const long long slots = (long long)m.cus * wg_per_cu;
@@ -289,6 +315,7 @@ std::vector<tdc_tile> model_enumerate(const tdc_conv_desc &d) {
                             for (int tw = 1; tw <= std::min(Wo, PT); ++tw) {
                                 const bool pow2 = (tw & (tw - 1)) == 0;
                                 const bool widest = (tw == std::min(Wo, PT));
+                                if (flat && !widest) continue;  // one row of pixels: nothing to gain from narrower runs
                                 if (!(widest || (pow2 && tw >= 4) || (Wo % tw == 0 && tw >= 4))) continue;
                                 const int th = std::min(PT / tw, Ho);
                                 const double util = (double)P / ((double)ceil_div(Wo, tw) * ceil_div(Ho, th) * PT);
@@ -315,6 +342,19 @@ std::vector<tdc_tile> model_enumerate(const tdc_conv_desc &d) {
                         }
     }
     return out;
+}
+
+int model_constants(double *out, int cap) {
+    for (int i = 0; i < kNumModelConst && i < cap; ++i) out[i] = *mc_field(i);
+    return kNumModelConst;
+}
+
+bool model_set_constants(const double *in, int n) {
+    if (n != kNumModelConst) return false;
+    for (int i = 0; i < n; ++i)
+        if (!(in[i] > 0.0)) return false;
+    for (int i = 0; i < n; ++i) *mc_field(i) = in[i];
+    return true;
 }
 
 bool model_select(const tdc_conv_desc &d, tdc_tile_info &best, std::string *why) {

@@ -21,7 +21,8 @@ EXPORTS = (
     "tdc_conv_time", "tdc_conv_time_many", "tdc_conv_plan_destroy",
     "tdc_tkconv_create", "tdc_tkconv_set_weights", "tdc_tkconv_forward", "tdc_tkconv_forward_features",
     "tdc_tkconv_core_forward", "tdc_tkconv_query", "tdc_tkconv_destroy",
-    "tdc_model_evaluate", "tdc_model_enumerate", "tdc_model_select",
+    "tdc_model_evaluate", "tdc_model_enumerate", "tdc_model_select", "tdc_model_get_constants",
+    "tdc_model_set_constants",
     "tdc_net_create", "tdc_net_conv", "tdc_net_tkconv", "tdc_net_pool", "tdc_net_global_avgpool", "tdc_net_concat",
     "tdc_net_tensor_shape", "tdc_net_num_kernels", "tdc_net_finalize", "tdc_net_forward", "tdc_net_time",
     "tdc_net_read_tensor", "tdc_net_destroy",
@@ -102,6 +103,8 @@ def lib():
     L.tdc_model_evaluate.argtypes = [POINTER(ConvDesc), POINTER(Tile), POINTER(TileInfo)]
     L.tdc_model_enumerate.argtypes = [POINTER(ConvDesc), POINTER(Tile), c_int32, POINTER(c_int32)]
     L.tdc_model_select.argtypes = [POINTER(ConvDesc), POINTER(TileInfo)]
+    L.tdc_model_get_constants.argtypes = [POINTER(c_double), c_int32, POINTER(c_int32)]
+    L.tdc_model_set_constants.argtypes = [POINTER(c_double), c_int32]
     i32, i32p, fpv = c_int32, POINTER(c_int32), c_void_p
     L.tdc_net_create.argtypes = [i32, i32, i32, i32, POINTER(c_void_p)]
     L.tdc_net_conv.argtypes = [c_void_p, i32, i32, i32, i32, i32, i32, fpv, fpv, i32, i32, i32p]
@@ -145,6 +148,23 @@ def model_evaluate(desc: ConvDesc, tile: Tile) -> TileInfo:
     info = TileInfo()
     check(lib().tdc_model_evaluate(byref(desc), byref(tile), byref(info)))
     return info
+
+
+MODEL_CONSTANT_NAMES = ("launch_us", "setup_clk", "copy_latency_clk", "copy_bytes_per_clk", "l2_bytes_per_clk",
+                        "lds_bytes_per_clk", "sync_clk", "store_bytes_per_clk", "kstep_issue_clk", "pass_overhead_clk",
+                        "wave_setup_clk")
+
+
+def model_get_constants():
+    n = c_int32(0)
+    buf = (c_double * 64)()
+    check(lib().tdc_model_get_constants(buf, 64, byref(n)))
+    return [buf[i] for i in range(n.value)]
+
+
+def model_set_constants(values):
+    arr = (c_double * len(values))(*values)
+    check(lib().tdc_model_set_constants(arr, len(values)))
 
 
 def model_enumerate(desc: ConvDesc, cap: int = 8192):
