@@ -47,10 +47,13 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-miopen", action="store_true", help="skip timing the same layers with MIOpen (through torch)")
     ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end Tucker ResNet-18 forward")
     ap.add_argument("--no-graph", action="store_true", help="issue launches on a plain stream instead of a HIP graph")
     ap.add_argument("--only-dominant", action="store_true",
                     help="profiling aid: launch only the dominant layer (128->128 @56), `steps` times, and exit")
+    ap.add_argument("--only-e2e", action="store_true",
+                    help="profiling aid: run only the end-to-end Tucker ResNet-18 forward, `steps` times, and exit")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="BYTES",
                     help="profiling aid: run a plain device copy of BYTES bytes a few times (reference reading for "
                          "the FETCH_SIZE / WRITE_SIZE counters) before anything else")
@@ -75,6 +78,13 @@ def main():
         for _ in range(5):
             dst.copy_(src)
         torch.cuda.synchronize()
+
+    if a.only_e2e:
+        from tdc_amd import nets
+        net = nets.build_tucker_resnet18(nets.resnet18_params(seed=18), batch=1)
+        ms = net.time_ms(iters=a.steps, graph=graph)
+        print(json.dumps({"only_e2e": True, "forwards": a.steps, "ms": ms, "kernels": net.num_kernels}))
+        return
 
     if a.only_dominant:
         x, w = ref.make_core_case(56, 128, 128)
@@ -126,6 +136,39 @@ def main():
                       "roof_us": round(info.roof_us, 4), "frac": round(info.roof_us / us, 4),
                       "gflops": round(info.flops / us * 1e-3, 1), "tile": list(info.tile.astuple())})
 
+    # -- comparator: MIOpen's convolution for the same layers (what torch.nn.functional.conv2d dispatches to on
+    #    ROCm), graph-replayed the same way; the reference compares against cuDNN the same way
+    #    (template_benchmark_cudnn.template:455-475).  Reported next to each layer, not part of `value`.
+    if not a.no_miopen:
+        import torch.nn.functional as F
+        torch.backends.cudnn.benchmark = True     # let MIOpen search its algorithms
+        for l, row in zip(layers, table):
+            wd = l["wc"].cuda()
+            for _ in range(5):
+                F.conv2d(l["x"], wd, None, 1, 1)
+            torch.cuda.synchronize()
+            side = torch.cuda.Stream()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.stream(side):
+                F.conv2d(l["x"], wd, None, 1, 1)
+                side.synchronize()
+                with torch.cuda.graph(g, stream=side):
+                    for _ in range(20):
+                        F.conv2d(l["x"], wd, None, 1, 1)
+            g.replay()
+            torch.cuda.synchronize()
+            best = float("inf")
+            for _ in range(3):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                for _ in range(5):
+                    g.replay()
+                e1.record()
+                e1.synchronize()
+                best = min(best, e0.elapsed_time(e1) * 1e3 / 100)
+            row["miopen_us"] = round(best, 3)
+            row["speedup_vs_miopen"] = round(best / row["us"], 2)
+
     # -- dominant kernel: the largest layer of the sweep --------------------------
     dom = max(range(len(layers)), key=lambda i: table[i]["us"])
     dl, dinfo = layers[dom], layers[dom]["plan"].info
@@ -154,6 +197,8 @@ def main():
         "roofline": roofline,
         "geomean_frac": round(float(torch.tensor([t["frac"] for t in table]).log().mean().exp()), 4),
         "layers": table,
+        "layers_faster_than_miopen": (sum(1 for t in table if t.get("speedup_vs_miopen", 0) > 1.0) if not a.no_miopen
+                                      else None),
         "host_wall_ms_timed_region": round(wall_ms, 3),
     }
 
