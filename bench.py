@@ -223,6 +223,23 @@ def main():
                                      "config": "ResNet-18 [2,2,2,2], every 3x3 conv = TKConv with R1=R2=planes/2, "
                                                "BN folded, batch 1, fp32 3x224x224, random init seed 18"}
         net.close()
+        # Tucker DenseNet-121 (configuration 5), batch 1 and batch 8, same treatment
+        dparams = nets.densenet121_params(seed=121)
+        dres = {}
+        for b in (1, 8):
+            dx = torch.randn(b, 3, 224, 224, generator=torch.Generator().manual_seed(121))
+            dnet = nets.build_tucker_densenet121(dparams, batch=b)
+            dlog = dnet(dx.cuda()).cpu().reshape(b, -1)
+            if b == 1:
+                dwant = nets_ref.tucker_densenet121_forward(dparams, dx)
+                derr = float((dlog - dwant).abs().max())
+                if not derr <= 1e-5 + 1e-4 * float(dwant.abs().max()):
+                    sys.exit("bench.py: DenseNet-121 parity check failed (max err %g)" % derr)
+            dnet.time_ms(iters=5)
+            dres["b%d_ms" % b] = round(min(dnet.time_ms(iters=20) for _ in range(3)), 4)
+            dres["kernels_per_forward"] = dnet.num_kernels
+            dnet.close()
+        out["tucker_densenet121"] = dres
 
     # -- CPU baseline: the reference operator's CPU path (F.conv2d), same layers --
     if not a.no_cpu_baseline:

@@ -111,6 +111,11 @@ int tdc_conv_plan_query(const tdc_conv_plan *plan, tdc_tile_info *info_out);
 /* d_residual may be NULL.  Output need not be pre-zeroed.  Asynchronous. */
 int tdc_conv_forward(tdc_conv_plan *plan, const float *d_in, const float *d_residual,
                      float *d_out, void *stream);
+/* Same with explicit distances (in floats) between consecutive images of the batch, so that a tensor can be
+ * a channel slice of a wider NCHW buffer; 0 = densely packed. */
+int tdc_conv_forward_strided(tdc_conv_plan *plan, const float *d_in, int64_t in_batch_stride,
+                             const float *d_residual, int64_t residual_batch_stride, float *d_out,
+                             int64_t out_batch_stride, void *stream);
 /* Measurement helper (the reference times its kernel with one cudaEvent pair
  * around a single cold launch, template_benchmark_cudnn.template:491-496): run
  * `iters` back-to-back forwards on a private stream between two hipEvents
@@ -149,6 +154,9 @@ int tdc_tkconv_set_weights(tdc_tkconv *op, const float *first, const float *core
 /* Full operator; intermediates live in op-owned device buffers. */
 int tdc_tkconv_forward(tdc_tkconv *op, const float *d_in, const float *d_residual,
                        float *d_out, void *stream);
+int tdc_tkconv_forward_strided(tdc_tkconv *op, const float *d_in, int64_t in_batch_stride,
+                               const float *d_residual, int64_t residual_batch_stride, float *d_out,
+                               int64_t out_batch_stride, void *stream);
 /* Same, also copying out the two intermediates (either may be NULL). */
 int tdc_tkconv_forward_features(tdc_tkconv *op, const float *d_in, float *d_feat_first,
                                 float *d_feat_core, float *d_out, void *stream);
@@ -169,17 +177,28 @@ void tdc_tkconv_destroy(tdc_tkconv *op);
 typedef struct tdc_net tdc_net;
 
 int tdc_net_create(int32_t batch, int32_t C, int32_t H, int32_t W, tdc_net **net_out);
-/* Dense convolution (also the classifier: a 1x1 convolution on a [C,1,1] tensor).  residual = -1 for none. */
+/* An uninitialised tensor (e.g. a concatenation buffer that producers fill slice by slice), and a view of
+ * channels [c0, c0+C) of an existing tensor that shares its memory.  Views are valid inputs, residuals and
+ * destinations. */
+int tdc_net_tensor(tdc_net *net, int32_t C, int32_t H, int32_t W, int32_t *out);
+int tdc_net_view(tdc_net *net, int32_t id, int32_t c0, int32_t C, int32_t *out);
+/* Operators.  `dst` = -1 allocates the result tensor, otherwise the result is written into that tensor/view
+ * (its shape must match).  `residual` = -1 for none.  *out receives the id of the result. */
+/* Dense convolution (also the classifier: a 1x1 convolution on a [C,1,1] tensor). */
 int tdc_net_conv(tdc_net *net, int32_t in, int32_t N, int32_t KH, int32_t KW, int32_t stride, int32_t pad,
-                 const float *w_oihw, const float *bias, int32_t residual, int32_t relu, int32_t *out);
+                 const float *w_oihw, const float *bias, int32_t residual, int32_t relu, int32_t dst, int32_t *out);
 /* Tucker convolution 1x1 C->R1, KxK R1->R2 (stride, pad), 1x1 R2->N, then +bias, +residual, ReLU. */
 int tdc_net_tkconv(tdc_net *net, int32_t in, int32_t R1, int32_t R2, int32_t N, int32_t K, int32_t stride,
                    int32_t pad, const float *first, const float *core, const float *last, const float *bias,
-                   int32_t residual, int32_t relu, int32_t *out);
+                   int32_t residual, int32_t relu, int32_t dst, int32_t *out);
 /* mode 0 = max, 1 = average (window count includes padding). */
-int tdc_net_pool(tdc_net *net, int32_t in, int32_t mode, int32_t k, int32_t stride, int32_t pad, int32_t *out);
+int tdc_net_pool(tdc_net *net, int32_t in, int32_t mode, int32_t k, int32_t stride, int32_t pad, int32_t dst,
+                 int32_t *out);
 int tdc_net_global_avgpool(tdc_net *net, int32_t in, int32_t *out);
-/* Channel concatenation of n tensors of equal height/width. */
+/* Per-channel y = x*scale[c] + shift[c], then ReLU if relu != 0 (inference BatchNorm in front of a convolution). */
+int tdc_net_affine(tdc_net *net, int32_t in, const float *scale, const float *shift, int32_t relu, int32_t dst,
+                   int32_t *out);
+/* Channel concatenation of n tensors of equal height/width into a new tensor (by copy). */
 int tdc_net_concat(tdc_net *net, const int32_t *ins, int32_t n, int32_t *out);
 int tdc_net_tensor_shape(const tdc_net *net, int32_t id, int32_t *C, int32_t *H, int32_t *W);
 int tdc_net_num_kernels(const tdc_net *net);

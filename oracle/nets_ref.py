@@ -43,3 +43,35 @@ def tucker_resnet18_forward(p, x, return_features=False):
     x = torch.flatten(x, 1)
     x = F.linear(x, p["fc.weight"], p["fc.bias"])
     return (x, feats) if return_features else x
+
+
+DENSENET121_BLOCKS = (6, 12, 24, 16)
+
+
+@torch.no_grad()
+def tucker_densenet121_forward(p, x):
+    """inference/densenet_inet_tt.py: TenDenseLayer.forward (:96-112, norm1 -> conv1 -> norm2 -> conv2 on the
+    concatenation of all earlier features), TenDenseBlock.forward (:132-137), TenDenseTransition (:140-158),
+    features -> norm5 -> global pool -> classifier.  The norm layers are BatchNorm + ReLU."""
+    def bnrelu(t, prefix):
+        return F.relu(_bn(t, p, prefix))
+
+    x = bnrelu(F.conv2d(x, p["features.conv0.weight"], None, 2, 3), "features.norm0")
+    x = F.max_pool2d(x, 3, 2, 1)
+    for b, nl in enumerate(DENSENET121_BLOCKS, start=1):
+        feats = [x]
+        for l in range(1, nl + 1):
+            pre = f"features.denseblock{b}.denselayer{l}"
+            y = F.conv2d(bnrelu(torch.cat(feats, 1), pre + ".norm1"), p[pre + ".conv1.weight"])
+            y = bnrelu(y, pre + ".norm2")
+            y = F.conv2d(y, p[pre + ".conv2.first_kernel"])
+            y = F.conv2d(y, p[pre + ".conv2.core_kernel"], None, 1, 1, 1, 1)
+            y = F.conv2d(y, p[pre + ".conv2.last_kernel"], None)
+            feats.append(y)
+        x = torch.cat(feats, 1)
+        if b < len(DENSENET121_BLOCKS):
+            pre = f"features.transition{b}"
+            x = F.avg_pool2d(F.conv2d(bnrelu(x, pre + ".norm"), p[pre + ".conv.weight"]), 2, 2)
+    x = bnrelu(x, "features.norm5")
+    x = torch.flatten(F.adaptive_avg_pool2d(x, (1, 1)), 1)
+    return F.linear(x, p["classifier.weight"], p["classifier.bias"])

@@ -184,10 +184,10 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
     const float *__restrict__ in = p.in + (long long)blockIdx.z * p.in_bstride;
     float *__restrict__ out = p.out + (long long)blockIdx.z * p.out_bstride;
     const float *__restrict__ resid =
-        p.resid ? p.resid + (long long)blockIdx.z * p.out_bstride : nullptr;
+        p.resid ? p.resid + (long long)blockIdx.z * p.resid_bstride : nullptr;
     // Raw buffers: byte offsets at or beyond num_records read as zero.
     const __amdgpu_buffer_rsrc_t in_rsrc =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(in), (short)0, (int)(p.in_bstride * 4), 0x00020000);
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(in), (short)0, (int)p.in_image_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t w_rsrc =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.wpk), (short)0, (int)p.wpk_bytes, 0x00020000);
 

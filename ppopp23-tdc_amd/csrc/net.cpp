@@ -1,11 +1,13 @@
-// Whole-network forward graphs: a list of Tucker / dense convolutions, pools and
-// concatenations over net-owned device tensors, captured once into a HIP graph
-// and replayed per inference.  This is what the reference's native E2E drivers
-// do layer object by layer object on the default stream
-// (2080Ti-evaluation/EndToEnd/resnet18-tk/src/main.cu:19-156,
-// src/BasicBlock.cu:43-50) — here with the topology supplied by the caller, the
-// BatchNorm/ReLU/residual work fused into the convolution epilogues, and one
-// graph launch instead of ~55 kernel launches.
+// Whole-network forward graphs: a list of Tucker / dense convolutions, pools,
+// per-channel affine(+ReLU) layers and concatenations over net-owned device
+// tensors, captured once into a HIP graph and replayed per inference.  This is
+// what the reference's native E2E drivers do layer object by layer object on the
+// default stream (2080Ti-evaluation/EndToEnd/resnet18-tk/src/main.cu:19-156,
+// src/BasicBlock.cu:43-50, densenet121-tk/src/main.cu:6-84) — here with the
+// topology supplied by the caller, BatchNorm/ReLU/residual work fused into the
+// convolution epilogues where the network allows it, concatenation done in place
+// (producers write into channel slices of one buffer), and one graph launch
+// instead of one launch per layer.
 #include <hip/hip_runtime_api.h>
 
 #include <memory>
@@ -21,16 +23,19 @@ namespace {
 
 struct NetTensor {
     int C = 0, H = 0, W = 0;
-    float *d = nullptr;
-    size_t floats = 0;
+    float *d = nullptr;       // first element (of image 0)
+    long long bstride = 0;    // floats between images
+    bool owner = false;
+    size_t floats = 0;        // allocation size (owners only)
 };
 
 struct NetOp {
-    enum Kind { CONV, TKCONV, POOL, GAP, COPYCH } kind = CONV;
+    enum Kind { CONV, TKCONV, POOL, GAP, COPY, AFFINE } kind = CONV;
     tdc_conv_plan *conv = nullptr;
     tdc_tkconv *tk = nullptr;
+    float *d_scale = nullptr, *d_shift = nullptr;
     int in = -1, out = -1, resid = -1;
-    int k = 0, stride = 0, pad = 0, mode = 0, c0 = 0;
+    int k = 0, stride = 0, pad = 0, mode = 0, relu = 0;
 };
 
 }  // namespace
@@ -56,7 +61,9 @@ int hipf(const char *what, hipError_t e) {
 int new_tensor(tdc_net *net, int C, int H, int W, int *id) {
     NetTensor t;
     t.C = C; t.H = H; t.W = W;
+    t.bstride = (long long)C * H * W;
     t.floats = (size_t)net->batch * C * H * W;
+    t.owner = true;
     hipError_t e = hipMalloc((void **)&t.d, t.floats * sizeof(float));
     if (e != hipSuccess) return hipf("hipMalloc(net tensor)", e);
     net->tensors.push_back(t);
@@ -72,20 +79,36 @@ int check_open(const tdc_net *net) {
     return TDC_OK;
 }
 
+// Destination of an operator: an existing tensor/view of exactly the produced shape, or a new tensor.
+int resolve_dst(tdc_net *net, int dst, int C, int H, int W, int *id) {
+    if (dst < 0) return new_tensor(net, C, H, W, id);
+    if (!valid_id(net, dst)) return api_fail(TDC_ERR_INVALID, "bad destination tensor id");
+    const NetTensor &t = net->tensors[dst];
+    if (t.C != C || t.H != H || t.W != W) return api_fail(TDC_ERR_INVALID, "destination tensor shape does not match the result");
+    *id = dst;
+    return TDC_OK;
+}
+
 int run_ops(tdc_net *net, hipStream_t s) {
     for (const NetOp &op : net->ops) {
         const NetTensor &ti = net->tensors[op.in];
         const NetTensor &to = net->tensors[op.out];
         const float *resid = op.resid >= 0 ? net->tensors[op.resid].d : nullptr;
+        const long long rbs = op.resid >= 0 ? net->tensors[op.resid].bstride : 0;
         int st = TDC_OK, he = 0;
         switch (op.kind) {
-            case NetOp::CONV: st = tdc_conv_forward(op.conv, ti.d, resid, to.d, s); break;
-            case NetOp::TKCONV: st = tdc_tkconv_forward(op.tk, ti.d, resid, to.d, s); break;
+            case NetOp::CONV: st = tdc_conv_forward_strided(op.conv, ti.d, ti.bstride, resid, rbs, to.d, to.bstride, s); break;
+            case NetOp::TKCONV: st = tdc_tkconv_forward_strided(op.tk, ti.d, ti.bstride, resid, rbs, to.d, to.bstride, s); break;
             case NetOp::POOL:
-                he = launch_pool2d(ti.d, to.d, net->batch * ti.C, ti.H, ti.W, to.H, to.W, op.k, op.stride, op.pad, op.mode, s);
+                he = launch_pool2d(ti.d, ti.bstride, to.d, to.bstride, net->batch, ti.C, ti.H, ti.W, to.H, to.W, op.k, op.stride,
+                                   op.pad, op.mode, s);
                 break;
-            case NetOp::GAP: he = launch_global_avgpool(ti.d, to.d, net->batch * ti.C, ti.H * ti.W, s); break;
-            case NetOp::COPYCH: he = launch_copy_channels(ti.d, to.d, net->batch, ti.C, ti.H * ti.W, to.C, op.c0, s); break;
+            case NetOp::GAP: he = launch_global_avgpool(ti.d, ti.bstride, to.d, to.bstride, net->batch, ti.C, ti.H * ti.W, s); break;
+            case NetOp::COPY: he = launch_copy_channels(ti.d, ti.bstride, to.d, to.bstride, net->batch, ti.C, ti.H * ti.W, s); break;
+            case NetOp::AFFINE:
+                he = launch_affine(ti.d, ti.bstride, to.d, to.bstride, op.d_scale, op.d_shift, net->batch, ti.C, ti.H * ti.W,
+                                   op.relu, s);
+                break;
         }
         if (st != TDC_OK) return st;
         if (he) return hipf("net kernel launch", (hipError_t)he);
@@ -115,30 +138,53 @@ int tdc_net_create(int32_t batch, int32_t C, int32_t H, int32_t W, tdc_net **net
     return TDC_OK;
 }
 
+int tdc_net_tensor(tdc_net *net, int32_t C, int32_t H, int32_t W, int32_t *out) {
+    int st = check_open(net);
+    if (st != TDC_OK) return st;
+    if (!out || C < 1 || H < 1 || W < 1) return api_fail(TDC_ERR_INVALID, "bad argument");
+    int id;
+    if ((st = new_tensor(net, C, H, W, &id)) != TDC_OK) return st;
+    *out = id;
+    return TDC_OK;
+}
+
+int tdc_net_view(tdc_net *net, int32_t id, int32_t c0, int32_t C, int32_t *out) {
+    int st = check_open(net);
+    if (st != TDC_OK) return st;
+    if (!out || !valid_id(net, id)) return api_fail(TDC_ERR_INVALID, "bad tensor id");
+    const NetTensor base = net->tensors[id];
+    if (c0 < 0 || C < 1 || c0 + C > base.C) return api_fail(TDC_ERR_INVALID, "channel range outside the tensor");
+    NetTensor v;
+    v.C = C; v.H = base.H; v.W = base.W;
+    v.d = base.d + (long long)c0 * base.H * base.W;
+    v.bstride = base.bstride;
+    v.owner = false;
+    net->tensors.push_back(v);
+    *out = (int)net->tensors.size() - 1;
+    return TDC_OK;
+}
+
 int tdc_net_conv(tdc_net *net, int32_t in, int32_t N, int32_t KH, int32_t KW, int32_t stride, int32_t pad, const float *w,
-                 const float *bias, int32_t residual, int32_t relu, int32_t *out) {
+                 const float *bias, int32_t residual, int32_t relu, int32_t dst, int32_t *out) {
     int st = check_open(net);
     if (st != TDC_OK) return st;
     if (!out || !w || !valid_id(net, in) || (residual >= 0 && !valid_id(net, residual)))
         return api_fail(TDC_ERR_INVALID, "bad tensor id or null argument");
     const NetTensor ti = net->tensors[in];
     tdc_conv_desc d{net->batch, ti.C, N, ti.H, ti.W, KH, KW, stride, pad, 1, bias != nullptr, relu != 0};
-    tdc_conv_plan *plan = nullptr;
-    if ((st = tdc_conv_plan_create(&d, nullptr, &plan)) != TDC_OK) return st;
-    if ((st = tdc_conv_plan_set_weights(plan, w, bias)) != TDC_OK) {
-        tdc_conv_plan_destroy(plan);
-        return st;
-    }
+    std::string why;
+    if (!check_desc(d, &why)) return api_fail(TDC_ERR_INVALID, why);
     const int Ho = (ti.H + 2 * pad - (KH - 1) - 1) / stride + 1, Wo = (ti.W + 2 * pad - (KW - 1) - 1) / stride + 1;
     if (residual >= 0) {
         const NetTensor &tr = net->tensors[residual];
-        if (tr.C != N || tr.H != Ho || tr.W != Wo) {
-            tdc_conv_plan_destroy(plan);
+        if (tr.C != N || tr.H != Ho || tr.W != Wo)
             return api_fail(TDC_ERR_INVALID, "residual tensor shape does not match the convolution output");
-        }
     }
     int id;
-    if ((st = new_tensor(net, N, Ho, Wo, &id)) != TDC_OK) {
+    if ((st = resolve_dst(net, dst, N, Ho, Wo, &id)) != TDC_OK) return st;
+    tdc_conv_plan *plan = nullptr;
+    if ((st = tdc_conv_plan_create(&d, nullptr, &plan)) != TDC_OK) return st;
+    if ((st = tdc_conv_plan_set_weights(plan, w, bias)) != TDC_OK) {
         tdc_conv_plan_destroy(plan);
         return st;
     }
@@ -152,29 +198,26 @@ int tdc_net_conv(tdc_net *net, int32_t in, int32_t N, int32_t KH, int32_t KW, in
 
 int tdc_net_tkconv(tdc_net *net, int32_t in, int32_t R1, int32_t R2, int32_t N, int32_t K, int32_t stride, int32_t pad,
                    const float *first, const float *core, const float *last, const float *bias, int32_t residual,
-                   int32_t relu, int32_t *out) {
+                   int32_t relu, int32_t dst, int32_t *out) {
     int st = check_open(net);
     if (st != TDC_OK) return st;
     if (!out || !first || !core || !last || !valid_id(net, in) || (residual >= 0 && !valid_id(net, residual)))
         return api_fail(TDC_ERR_INVALID, "bad tensor id or null argument");
+    if (K < 1 || stride < 1 || pad < 0) return api_fail(TDC_ERR_INVALID, "bad core convolution geometry");
     const NetTensor ti = net->tensors[in];
+    if (ti.H + 2 * pad < K || ti.W + 2 * pad < K) return api_fail(TDC_ERR_INVALID, "core filter larger than the padded input");
+    const int Ho = (ti.H + 2 * pad - (K - 1) - 1) / stride + 1, Wo = (ti.W + 2 * pad - (K - 1) - 1) / stride + 1;
+    if (residual >= 0) {
+        const NetTensor &tr = net->tensors[residual];
+        if (tr.C != N || tr.H != Ho || tr.W != Wo)
+            return api_fail(TDC_ERR_INVALID, "residual tensor shape does not match the operator output");
+    }
+    int id;
+    if ((st = resolve_dst(net, dst, N, Ho, Wo, &id)) != TDC_OK) return st;
     tdc_tkconv_desc d{net->batch, ti.C, R1, R2, N, ti.H, ti.W, K, stride, pad, 1, bias != nullptr, relu != 0};
     tdc_tkconv *tk = nullptr;
     if ((st = tdc_tkconv_create(&d, &tk)) != TDC_OK) return st;
     if ((st = tdc_tkconv_set_weights(tk, first, core, last, bias)) != TDC_OK) {
-        tdc_tkconv_destroy(tk);
-        return st;
-    }
-    const int Ho = (ti.H + 2 * pad - (K - 1) - 1) / stride + 1, Wo = (ti.W + 2 * pad - (K - 1) - 1) / stride + 1;
-    if (residual >= 0) {
-        const NetTensor &tr = net->tensors[residual];
-        if (tr.C != N || tr.H != Ho || tr.W != Wo) {
-            tdc_tkconv_destroy(tk);
-            return api_fail(TDC_ERR_INVALID, "residual tensor shape does not match the operator output");
-        }
-    }
-    int id;
-    if ((st = new_tensor(net, N, Ho, Wo, &id)) != TDC_OK) {
         tdc_tkconv_destroy(tk);
         return st;
     }
@@ -186,7 +229,7 @@ int tdc_net_tkconv(tdc_net *net, int32_t in, int32_t R1, int32_t R2, int32_t N, 
     return TDC_OK;
 }
 
-int tdc_net_pool(tdc_net *net, int32_t in, int32_t mode, int32_t k, int32_t stride, int32_t pad, int32_t *out) {
+int tdc_net_pool(tdc_net *net, int32_t in, int32_t mode, int32_t k, int32_t stride, int32_t pad, int32_t dst, int32_t *out) {
     int st = check_open(net);
     if (st != TDC_OK) return st;
     if (!out || !valid_id(net, in) || k < 1 || stride < 1 || pad < 0 || 2 * pad > k || (mode != 0 && mode != 1))
@@ -195,7 +238,7 @@ int tdc_net_pool(tdc_net *net, int32_t in, int32_t mode, int32_t k, int32_t stri
     if (ti.H + 2 * pad < k || ti.W + 2 * pad < k) return api_fail(TDC_ERR_INVALID, "pooling window larger than the input");
     const int Ho = (ti.H + 2 * pad - k) / stride + 1, Wo = (ti.W + 2 * pad - k) / stride + 1;
     int id;
-    if ((st = new_tensor(net, ti.C, Ho, Wo, &id)) != TDC_OK) return st;
+    if ((st = resolve_dst(net, dst, ti.C, Ho, Wo, &id)) != TDC_OK) return st;
     NetOp op;
     op.kind = NetOp::POOL; op.in = in; op.out = id; op.k = k; op.stride = stride; op.pad = pad; op.mode = mode;
     net->ops.push_back(op);
@@ -219,6 +262,31 @@ int tdc_net_global_avgpool(tdc_net *net, int32_t in, int32_t *out) {
     return TDC_OK;
 }
 
+int tdc_net_affine(tdc_net *net, int32_t in, const float *scale, const float *shift, int32_t relu, int32_t dst,
+                   int32_t *out) {
+    int st = check_open(net);
+    if (st != TDC_OK) return st;
+    if (!out || !scale || !shift || !valid_id(net, in)) return api_fail(TDC_ERR_INVALID, "bad tensor id or null argument");
+    const NetTensor ti = net->tensors[in];
+    int id;
+    if ((st = resolve_dst(net, dst, ti.C, ti.H, ti.W, &id)) != TDC_OK) return st;
+    NetOp op;
+    op.kind = NetOp::AFFINE; op.in = in; op.out = id; op.relu = relu != 0;
+    hipError_t e = hipMalloc((void **)&op.d_scale, 2 * (size_t)ti.C * sizeof(float));
+    if (e != hipSuccess) return hipf("hipMalloc(affine)", e);
+    op.d_shift = op.d_scale + ti.C;
+    e = hipMemcpy(op.d_scale, scale, (size_t)ti.C * sizeof(float), hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = hipMemcpy(op.d_shift, shift, (size_t)ti.C * sizeof(float), hipMemcpyHostToDevice);
+    if (e != hipSuccess) {
+        (void)hipFree(op.d_scale);
+        return hipf("hipMemcpy(affine)", e);
+    }
+    net->ops.push_back(op);
+    net->kernels += 1;
+    *out = id;
+    return TDC_OK;
+}
+
 int tdc_net_concat(tdc_net *net, const int32_t *ins, int32_t n, int32_t *out) {
     int st = check_open(net);
     if (st != TDC_OK) return st;
@@ -235,8 +303,10 @@ int tdc_net_concat(tdc_net *net, const int32_t *ins, int32_t n, int32_t *out) {
     if ((st = new_tensor(net, Ctot, net->tensors[ins[0]].H, net->tensors[ins[0]].W, &id)) != TDC_OK) return st;
     int c0 = 0;
     for (int i = 0; i < n; ++i) {
+        int view;
+        if ((st = tdc_net_view(net, id, c0, net->tensors[ins[i]].C, &view)) != TDC_OK) return st;
         NetOp op;
-        op.kind = NetOp::COPYCH; op.in = ins[i]; op.out = id; op.c0 = c0;
+        op.kind = NetOp::COPY; op.in = ins[i]; op.out = view;
         net->ops.push_back(op);
         net->kernels += 1;
         c0 += net->tensors[ins[i]].C;
@@ -280,11 +350,13 @@ int tdc_net_forward(tdc_net *net, const float *d_in, float *d_out, void *stream)
     hipStream_t s = (hipStream_t)stream;
     const NetTensor &ti = net->tensors[0];
     const NetTensor &to = net->tensors[net->out_id];
+    if (d_out && to.bstride != (long long)to.C * to.H * to.W)
+        return api_fail(TDC_ERR_UNSUPPORTED, "the output tensor is a channel slice; read it with tdc_net_read_tensor");
     hipError_t e = hipSuccess;
     if (d_in && d_in != ti.d) e = hipMemcpyAsync(ti.d, d_in, ti.floats * sizeof(float), hipMemcpyDeviceToDevice, s);
     if (e == hipSuccess) e = hipGraphLaunch(net->exec, s);
     if (e == hipSuccess && d_out && d_out != to.d)
-        e = hipMemcpyAsync(d_out, to.d, to.floats * sizeof(float), hipMemcpyDeviceToDevice, s);
+        e = hipMemcpyAsync(d_out, to.d, (size_t)net->batch * to.C * to.H * to.W * sizeof(float), hipMemcpyDeviceToDevice, s);
     if (e != hipSuccess) return hipf("tdc_net_forward", e);
     return TDC_OK;
 }
@@ -314,9 +386,11 @@ int tdc_net_time(tdc_net *net, int32_t iters, int32_t use_graph, float *total_ms
 
 int tdc_net_read_tensor(tdc_net *net, int32_t id, float *host_out) {
     if (!net || !valid_id(net, id) || !host_out) return api_fail(TDC_ERR_INVALID, "bad argument");
+    const NetTensor &t = net->tensors[id];
+    const size_t image = (size_t)t.C * t.H * t.W;
     hipError_t e = hipDeviceSynchronize();
-    if (e == hipSuccess)
-        e = hipMemcpy(host_out, net->tensors[id].d, net->tensors[id].floats * sizeof(float), hipMemcpyDeviceToHost);
+    for (int b = 0; b < net->batch && e == hipSuccess; ++b)
+        e = hipMemcpy(host_out + b * image, t.d + b * t.bstride, image * sizeof(float), hipMemcpyDeviceToHost);
     if (e != hipSuccess) return hipf("tdc_net_read_tensor", e);
     return TDC_OK;
 }
@@ -328,9 +402,10 @@ void tdc_net_destroy(tdc_net *net) {
     for (NetOp &op : net->ops) {
         if (op.conv) tdc_conv_plan_destroy(op.conv);
         if (op.tk) tdc_tkconv_destroy(op.tk);
+        if (op.d_scale) (void)hipFree(op.d_scale);
     }
     for (NetTensor &t : net->tensors)
-        if (t.d) (void)hipFree(t.d);
+        if (t.owner && t.d) (void)hipFree(t.d);
     if (net->stream) (void)hipStreamDestroy(net->stream);
     delete net;
 }

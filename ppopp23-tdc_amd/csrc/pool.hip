@@ -12,20 +12,25 @@
 
 namespace tdc {
 
+// Every kernel takes batch strides in floats, so a tensor may be a channel slice of a wider
+// buffer (DenseNet's growing concatenation is written in place).
+
 // mode 0 = max (padding never wins), 1 = average over the full k*k window
 // including padding zeros (count_include_pad, which equals PyTorch's AvgPool2d
 // default and is irrelevant when pad == 0).
-__global__ void __launch_bounds__(256) pool2d_kernel(const float *__restrict__ in, float *__restrict__ out,
-                                                     int planes, int H, int W, int Ho, int Wo, int k, int stride,
-                                                     int pad, int mode) {
-    const long long total = (long long)planes * Ho * Wo;
+__global__ void __launch_bounds__(256) pool2d_kernel(const float *__restrict__ in, long long in_bs,
+                                                     float *__restrict__ out, long long out_bs, int B, int C, int H,
+                                                     int W, int Ho, int Wo, int k, int stride, int pad, int mode) {
+    const long long per = (long long)C * Ho * Wo;
     const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= total) return;
-    const int ox = (int)(idx % Wo);
-    const long long t = idx / Wo;
+    if (idx >= per * B) return;
+    const int b = (int)(idx / per);
+    const long long rem = idx - (long long)b * per;
+    const int ox = (int)(rem % Wo);
+    const long long t = rem / Wo;
     const int oy = (int)(t % Ho);
-    const long long pl = t / Ho;
-    const float *src = in + pl * H * W;
+    const int c = (int)(t / Ho);
+    const float *src = in + b * in_bs + (long long)c * H * W;
     float acc = mode == 0 ? -FLT_MAX : 0.0f;
     for (int r = 0; r < k; ++r) {
         const int iy = oy * stride - pad + r;
@@ -38,54 +43,82 @@ __global__ void __launch_bounds__(256) pool2d_kernel(const float *__restrict__ i
         }
     }
     if (mode == 1) acc *= 1.0f / (float)(k * k);
-    out[idx] = acc;
+    out[b * out_bs + rem] = acc;
 }
 
-// Global average pool: one wave per plane, lanes stride over the H*W pixels, DPP-free shuffle reduction.
-__global__ void __launch_bounds__(256) global_avgpool_kernel(const float *__restrict__ in, float *__restrict__ out,
-                                                             int planes, int HW) {
+// Global average pool: one wave per plane, lanes stride over the H*W pixels, shuffle reduction.
+__global__ void __launch_bounds__(256) global_avgpool_kernel(const float *__restrict__ in, long long in_bs,
+                                                             float *__restrict__ out, long long out_bs, int B, int C,
+                                                             int HW) {
     const int wave = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
     const int lane = threadIdx.x & 63;
-    if (wave >= planes) return;
-    const float *src = in + (long long)wave * HW;
+    if (wave >= B * C) return;
+    const int b = wave / C, c = wave - b * C;
+    const float *src = in + b * in_bs + (long long)c * HW;
     float acc = 0.0f;
     for (int i = lane; i < HW; i += 64) acc += src[i];
     for (int off = 32; off > 0; off >>= 1) acc += __shfl_down(acc, off, 64);
-    if (lane == 0) out[wave] = acc / (float)HW;
+    if (lane == 0) out[b * out_bs + c] = acc / (float)HW;
 }
 
-// Copy [B, C, HW] into channels [c0, c0+C) of a [B, Ctot, HW] buffer (DenseNet concatenation;
-// the reference's concate kernel, 2080Ti-evaluation/EndToEnd/densenet121-tk/src/Conv.cu:126-155).
-__global__ void __launch_bounds__(256) copy_channels_kernel(const float *__restrict__ in, float *__restrict__ out,
-                                                            int B, int C, int HW, int Ctot, int c0) {
-    const long long total = (long long)B * C * HW;
-    const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= total) return;
+// Copy [B, C, HW] between (possibly strided) tensors — channel concatenation (the reference's concate
+// kernel, 2080Ti-evaluation/EndToEnd/densenet121-tk/src/Conv.cu:126-155).
+__global__ void __launch_bounds__(256) copy_channels_kernel(const float *__restrict__ in, long long in_bs,
+                                                            float *__restrict__ out, long long out_bs, int B, int C,
+                                                            int HW) {
     const long long per = (long long)C * HW;
+    const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= per * B) return;
     const long long b = idx / per;
     const long long rem = idx - b * per;
-    out[b * (long long)Ctot * HW + (long long)c0 * HW + rem] = in[idx];
+    out[b * out_bs + rem] = in[b * in_bs + rem];
 }
 
-int launch_pool2d(const float *in, float *out, int planes, int H, int W, int Ho, int Wo, int k, int stride, int pad,
-                  int mode, void *stream) {
-    const long long total = (long long)planes * Ho * Wo;
-    const unsigned blocks = (unsigned)((total + 255) / 256);
-    hipLaunchKernelGGL(pool2d_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, in, out, planes, H, W, Ho, Wo, k,
-                       stride, pad, mode);
+// Inference-mode BatchNorm (+ReLU) in front of a convolution: out = max(in*scale[c] + shift[c], 0).
+// DenseNet normalises the concatenated features separately for every consumer
+// (inference/densenet_inet_tt.py:66-70), so it cannot be folded into the producer.
+__global__ void __launch_bounds__(256) affine_kernel(const float *__restrict__ in, long long in_bs,
+                                                     float *__restrict__ out, long long out_bs,
+                                                     const float *__restrict__ scale, const float *__restrict__ shift,
+                                                     int B, int C, int HW, int relu) {
+    const long long per = (long long)C * HW;
+    const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= per * B) return;
+    const long long b = idx / per;
+    const long long rem = idx - b * per;
+    const int c = (int)(rem / HW);
+    float v = in[b * in_bs + rem] * scale[c] + shift[c];
+    if (relu) v = fmaxf(v, 0.0f);
+    out[b * out_bs + rem] = v;
+}
+
+static unsigned blocks_for(long long total) { return (unsigned)((total + 255) / 256); }
+
+int launch_pool2d(const float *in, long long in_bs, float *out, long long out_bs, int B, int C, int H, int W, int Ho,
+                  int Wo, int k, int stride, int pad, int mode, void *stream) {
+    hipLaunchKernelGGL(pool2d_kernel, dim3(blocks_for((long long)B * C * Ho * Wo)), dim3(256), 0, (hipStream_t)stream, in,
+                       in_bs, out, out_bs, B, C, H, W, Ho, Wo, k, stride, pad, mode);
     return (int)hipGetLastError();
 }
 
-int launch_global_avgpool(const float *in, float *out, int planes, int HW, void *stream) {
-    const unsigned blocks = (unsigned)((planes + 3) / 4);  // 4 waves per block
-    hipLaunchKernelGGL(global_avgpool_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, in, out, planes, HW);
+int launch_global_avgpool(const float *in, long long in_bs, float *out, long long out_bs, int B, int C, int HW,
+                          void *stream) {
+    hipLaunchKernelGGL(global_avgpool_kernel, dim3((unsigned)((B * C + 3) / 4)), dim3(256), 0, (hipStream_t)stream, in,
+                       in_bs, out, out_bs, B, C, HW);
     return (int)hipGetLastError();
 }
 
-int launch_copy_channels(const float *in, float *out, int B, int C, int HW, int Ctot, int c0, void *stream) {
-    const long long total = (long long)B * C * HW;
-    const unsigned blocks = (unsigned)((total + 255) / 256);
-    hipLaunchKernelGGL(copy_channels_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, in, out, B, C, HW, Ctot, c0);
+int launch_copy_channels(const float *in, long long in_bs, float *out, long long out_bs, int B, int C, int HW,
+                         void *stream) {
+    hipLaunchKernelGGL(copy_channels_kernel, dim3(blocks_for((long long)B * C * HW)), dim3(256), 0, (hipStream_t)stream,
+                       in, in_bs, out, out_bs, B, C, HW);
+    return (int)hipGetLastError();
+}
+
+int launch_affine(const float *in, long long in_bs, float *out, long long out_bs, const float *scale, const float *shift,
+                  int B, int C, int HW, int relu, void *stream) {
+    hipLaunchKernelGGL(affine_kernel, dim3(blocks_for((long long)B * C * HW)), dim3(256), 0, (hipStream_t)stream, in, in_bs,
+                       out, out_bs, scale, shift, B, C, HW, relu);
     return (int)hipGetLastError();
 }
 

@@ -168,16 +168,31 @@ int tdc_conv_plan_query(const tdc_conv_plan *plan, tdc_tile_info *info_out) {
 }
 
 int tdc_conv_forward(tdc_conv_plan *plan, const float *d_in, const float *d_residual, float *d_out, void *stream) {
+    return tdc_conv_forward_strided(plan, d_in, 0, d_residual, 0, d_out, 0, stream);
+}
+
+int tdc_conv_forward_strided(tdc_conv_plan *plan, const float *d_in, int64_t in_batch_stride, const float *d_residual,
+                             int64_t residual_batch_stride, float *d_out, int64_t out_batch_stride, void *stream) {
     if (!plan || !d_in || !d_out) return fail(TDC_ERR_INVALID, "null argument");
+    if (in_batch_stride < 0 || out_batch_stride < 0 || residual_batch_stride < 0)
+        return fail(TDC_ERR_INVALID, "negative batch stride");
     if (!plan->have_weights) return fail(TDC_ERR_STATE, "tdc_conv_forward before tdc_conv_plan_set_weights");
     const tdc_conv_desc &d = plan->desc;
     const Geometry &g = plan->geo;
+    const long long in_image = (long long)d.C * d.H * d.W, out_image = (long long)d.N * g.P;
+    if ((in_batch_stride && in_batch_stride < in_image) || (out_batch_stride && out_batch_stride < out_image) ||
+        (residual_batch_stride && residual_batch_stride < out_image))
+        return fail(TDC_ERR_INVALID, "batch stride smaller than one image");
     ConvKParams kp{};
     kp.in = d_in;
     kp.wpk = plan->d_wpk;
     kp.bias = plan->d_bias;
     kp.resid = d_residual;
     kp.out = d_out;
+    kp.in_image_bytes = (unsigned)(in_image * 4);
+    kp.in_bstride = in_batch_stride ? in_batch_stride : in_image;
+    kp.out_bstride = out_batch_stride ? out_batch_stride : out_image;
+    kp.resid_bstride = residual_batch_stride ? residual_batch_stride : out_image;
     kp.C = d.C; kp.H = g.He; kp.W = g.We; kp.N = d.N;
     kp.Ho = g.Ho; kp.Wo = g.Wo; kp.P = g.P;
     kp.KH = d.KH; kp.KW = d.KW; kp.stride = d.stride; kp.pad = d.pad; kp.dil = d.dilation;
@@ -185,8 +200,9 @@ int tdc_conv_forward(tdc_conv_plan *plan, const float *d_in, const float *d_resi
     kp.WM = plan->tile.wm; kp.WN = plan->tile.wn; kp.WK = plan->tile.wk;
     kp.CCH = plan->tile.cch; kp.nchunks = g.nchunks; kp.CPW = g.cpw;
     kp.RS = g.RS; kp.CS = g.CS; kp.nrows = g.nrows;
-    // 16-byte copy elements need 16-byte aligned activations; otherwise fall back to 4-byte elements.
-    kp.VW = (reinterpret_cast<uintptr_t>(d_in) % (4 * g.VW) == 0) ? g.VW : 1;
+    // 16-byte copy elements need every image of the batch 16-byte aligned; otherwise 4-byte elements.
+    const bool aligned = reinterpret_cast<uintptr_t>(d_in) % 16 == 0 && kp.in_bstride % 4 == 0;
+    kp.VW = (g.VW == 4 && aligned) ? 4 : 1;
     kp.in_stage_floats = g.in_stage_floats; kp.wslab_floats = g.wslab_floats;
     kp.stage_floats = g.stage_floats; kp.nstage = g.nstage;
     kp.relu = d.relu;
@@ -198,8 +214,6 @@ int tdc_conv_forward(tdc_conv_plan *plan, const float *d_in, const float *d_resi
     kp.fd_wk = make_fastdiv(plan->tile.wk);
     kp.fd_wn = make_fastdiv(plan->tile.wn);
     kp.wpk_bytes = (unsigned)(packed_weight_floats(g) * sizeof(float));
-    kp.in_bstride = (long long)d.C * d.H * d.W;
-    kp.out_bstride = (long long)d.N * g.P;
     int he = launch_conv(plan->kernel, g, kp, stream);
     if (he) return hip_fail("kernel launch", he);
     return TDC_OK;
@@ -361,11 +375,16 @@ int tdc_tkconv_set_weights(tdc_tkconv *op, const float *first, const float *core
 }
 
 int tdc_tkconv_forward(tdc_tkconv *op, const float *d_in, const float *d_residual, float *d_out, void *stream) {
+    return tdc_tkconv_forward_strided(op, d_in, 0, d_residual, 0, d_out, 0, stream);
+}
+
+int tdc_tkconv_forward_strided(tdc_tkconv *op, const float *d_in, int64_t in_batch_stride, const float *d_residual,
+                               int64_t residual_batch_stride, float *d_out, int64_t out_batch_stride, void *stream) {
     if (!op || !d_in || !d_out) return fail(TDC_ERR_INVALID, "null argument");
     int st;
-    if ((st = tdc_conv_forward(op->first, d_in, nullptr, op->d_f1, stream)) != TDC_OK) return st;
+    if ((st = tdc_conv_forward_strided(op->first, d_in, in_batch_stride, nullptr, 0, op->d_f1, 0, stream)) != TDC_OK) return st;
     if ((st = tdc_conv_forward(op->core, op->d_f1, nullptr, op->d_f2, stream)) != TDC_OK) return st;
-    return tdc_conv_forward(op->last, op->d_f2, d_residual, d_out, stream);
+    return tdc_conv_forward_strided(op->last, op->d_f2, 0, d_residual, residual_batch_stride, d_out, out_batch_stride, stream);
 }
 
 int tdc_tkconv_forward_features(tdc_tkconv *op, const float *d_in, float *d_feat_first, float *d_feat_core,

@@ -104,8 +104,10 @@ struct ConvKParams {
     FastDiv fd_tw, fd_ntx, fd_pt;
     FastDiv fd_wk, fd_wn;
     unsigned wpk_bytes;
-    long long in_bstride;   // C*H*W
-    long long out_bstride;  // N*P
+    unsigned in_image_bytes;   // C*H*W*4: reads at or past it return zero
+    long long in_bstride;      // floats between consecutive images of the input (C*H*W when dense)
+    long long out_bstride;     // ... of the output (N*P when dense)
+    long long resid_bstride;   // ... of the residual
 };
 
 // The instantiated kernel for a tile and filter size (nullptr if none).
@@ -116,10 +118,16 @@ int prepare_conv_kernel(const void *fn, const Geometry &g);
 int launch_conv(const void *fn, const Geometry &g, const ConvKParams &kp, void *stream);
 
 // Pooling / concatenation kernels of the whole-network graphs (hipError_t as int).
-int launch_pool2d(const float *in, float *out, int planes, int H, int W, int Ho, int Wo, int k, int stride, int pad,
-                  int mode, void *stream);
-int launch_global_avgpool(const float *in, float *out, int planes, int HW, void *stream);
-int launch_copy_channels(const float *in, float *out, int B, int C, int HW, int Ctot, int c0, void *stream);
+// Batch strides are in floats; a tensor may be a channel slice of a wider buffer.
+int launch_pool2d(const float *in, long long in_bstride, float *out, long long out_bstride, int B, int C, int H, int W,
+                  int Ho, int Wo, int k, int stride, int pad, int mode, void *stream);
+int launch_global_avgpool(const float *in, long long in_bstride, float *out, long long out_bstride, int B, int C, int HW,
+                          void *stream);
+int launch_copy_channels(const float *in, long long in_bstride, float *out, long long out_bstride, int B, int C, int HW,
+                         void *stream);
+// out = max(in * scale[c] + shift[c], 0) (relu != 0) per channel.
+int launch_affine(const float *in, long long in_bstride, float *out, long long out_bstride, const float *scale,
+                  const float *shift, int B, int C, int HW, int relu, void *stream);
 
 void set_error(const std::string &msg);
 int api_fail(int status, const std::string &msg);   // records the message, returns status

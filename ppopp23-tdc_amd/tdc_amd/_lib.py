@@ -18,12 +18,13 @@ TDC_OK, TDC_ERR_INVALID, TDC_ERR_UNSUPPORTED, TDC_ERR_HIP, TDC_ERR_NOMEM, TDC_ER
 EXPORTS = (
     "tdc_last_error_string", "tdc_version",
     "tdc_conv_plan_create", "tdc_conv_plan_set_weights", "tdc_conv_plan_query", "tdc_conv_forward",
+    "tdc_conv_forward_strided", "tdc_tkconv_forward_strided",
     "tdc_conv_time", "tdc_conv_time_many", "tdc_conv_plan_destroy",
     "tdc_tkconv_create", "tdc_tkconv_set_weights", "tdc_tkconv_forward", "tdc_tkconv_forward_features",
     "tdc_tkconv_core_forward", "tdc_tkconv_query", "tdc_tkconv_destroy",
     "tdc_model_evaluate", "tdc_model_enumerate", "tdc_model_select", "tdc_model_get_constants",
     "tdc_model_set_constants",
-    "tdc_net_create", "tdc_net_conv", "tdc_net_tkconv", "tdc_net_pool", "tdc_net_global_avgpool", "tdc_net_concat",
+    "tdc_net_create", "tdc_net_tensor", "tdc_net_view", "tdc_net_affine", "tdc_net_conv", "tdc_net_tkconv", "tdc_net_pool", "tdc_net_global_avgpool", "tdc_net_concat",
     "tdc_net_tensor_shape", "tdc_net_num_kernels", "tdc_net_finalize", "tdc_net_forward", "tdc_net_time",
     "tdc_net_read_tensor", "tdc_net_destroy",
 )
@@ -107,9 +108,15 @@ def lib():
     L.tdc_model_set_constants.argtypes = [POINTER(c_double), c_int32]
     i32, i32p, fpv = c_int32, POINTER(c_int32), c_void_p
     L.tdc_net_create.argtypes = [i32, i32, i32, i32, POINTER(c_void_p)]
-    L.tdc_net_conv.argtypes = [c_void_p, i32, i32, i32, i32, i32, i32, fpv, fpv, i32, i32, i32p]
-    L.tdc_net_tkconv.argtypes = [c_void_p, i32, i32, i32, i32, i32, i32, i32, fpv, fpv, fpv, fpv, i32, i32, i32p]
-    L.tdc_net_pool.argtypes = [c_void_p, i32, i32, i32, i32, i32, i32p]
+    i64 = ctypes.c_int64
+    L.tdc_conv_forward_strided.argtypes = [c_void_p, c_void_p, i64, c_void_p, i64, c_void_p, i64, c_void_p]
+    L.tdc_tkconv_forward_strided.argtypes = [c_void_p, c_void_p, i64, c_void_p, i64, c_void_p, i64, c_void_p]
+    L.tdc_net_tensor.argtypes = [c_void_p, i32, i32, i32, i32p]
+    L.tdc_net_view.argtypes = [c_void_p, i32, i32, i32, i32p]
+    L.tdc_net_affine.argtypes = [c_void_p, i32, fpv, fpv, i32, i32, i32p]
+    L.tdc_net_conv.argtypes = [c_void_p, i32, i32, i32, i32, i32, i32, fpv, fpv, i32, i32, i32, i32p]
+    L.tdc_net_tkconv.argtypes = [c_void_p, i32, i32, i32, i32, i32, i32, i32, fpv, fpv, fpv, fpv, i32, i32, i32, i32p]
+    L.tdc_net_pool.argtypes = [c_void_p, i32, i32, i32, i32, i32, i32, i32p]
     L.tdc_net_global_avgpool.argtypes = [c_void_p, i32, i32p]
     L.tdc_net_concat.argtypes = [c_void_p, i32p, i32, i32p]
     L.tdc_net_tensor_shape.argtypes = [c_void_p, i32, i32p, i32p, i32p]

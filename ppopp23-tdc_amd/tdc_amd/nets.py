@@ -39,23 +39,39 @@ class Net:
         self.output_id = None
         self._keep = []
 
-    def conv(self, x, weight, bias=None, stride=1, pad=0, residual=-1, relu=False):
+    def tensor(self, C, H, W):
+        out = c_int32()
+        check(lib().tdc_net_tensor(self._h, C, H, W, byref(out)))
+        return out.value
+
+    def view(self, tid, c0, C):
+        out = c_int32()
+        check(lib().tdc_net_view(self._h, tid, c0, C, byref(out)))
+        return out.value
+
+    def conv(self, x, weight, bias=None, stride=1, pad=0, residual=-1, relu=False, dst=-1):
         w, b = _h(weight), _h(bias)
         out = c_int32()
         check(lib().tdc_net_conv(self._h, x, w.shape[0], w.shape[2], w.shape[3], stride, pad, _p(w), _p(b), residual,
-                                 int(relu), byref(out)))
+                                 int(relu), dst, byref(out)))
         return out.value
 
-    def tkconv(self, x, first, core, last, bias=None, stride=1, pad=0, residual=-1, relu=False):
+    def tkconv(self, x, first, core, last, bias=None, stride=1, pad=0, residual=-1, relu=False, dst=-1):
         f, c, l, b = _h(first), _h(core), _h(last), _h(bias)
         out = c_int32()
         check(lib().tdc_net_tkconv(self._h, x, f.shape[0], c.shape[0], l.shape[0], c.shape[2], stride, pad, _p(f), _p(c),
-                                   _p(l), _p(b), residual, int(relu), byref(out)))
+                                   _p(l), _p(b), residual, int(relu), dst, byref(out)))
         return out.value
 
-    def pool(self, x, mode, k, stride, pad=0):
+    def pool(self, x, mode, k, stride, pad=0, dst=-1):
         out = c_int32()
-        check(lib().tdc_net_pool(self._h, x, {"max": 0, "avg": 1}[mode], k, stride, pad, byref(out)))
+        check(lib().tdc_net_pool(self._h, x, {"max": 0, "avg": 1}[mode], k, stride, pad, dst, byref(out)))
+        return out.value
+
+    def affine(self, x, scale, shift, relu=True, dst=-1):
+        s, t = _h(scale), _h(shift)
+        out = c_int32()
+        check(lib().tdc_net_affine(self._h, x, _p(s), _p(t), int(relu), dst, byref(out)))
         return out.value
 
     def global_avgpool(self, x):
@@ -192,3 +208,87 @@ def build_tucker_resnet18(params, batch=1, H=224, W=224):
     x = net.global_avgpool(x)
     x = net.conv(x, p["fc.weight"].reshape(p["fc.weight"].shape[0], -1, 1, 1), p["fc.bias"])
     return net.finalize(x)
+
+
+# ---------------------------------------------------------------------------------------------------
+# Tucker DenseNet-121 (inference/densenet_inet_tt.py:36-158 TenDenseLayer / TenDenseBlock /
+# TenDenseTransition; growth 32, bn_size 4, blocks (6, 12, 24, 16)); every 3x3 convolution 128->32 a
+# TKConv2dC with ranks (R1, R2) = (64, 16).
+DENSENET121_BLOCKS = (6, 12, 24, 16)
+
+
+def densenet121_params(seed=121, num_classes=1000, growth=32, bn_size=4, ranks=(64, 16)):
+    g = torch.Generator().manual_seed(seed)
+
+    def kaiming(*shape):
+        fan_in = shape[1] * shape[2] * shape[3]
+        return torch.empty(*shape).normal_(0, math.sqrt(2.0 / fan_in), generator=g)
+
+    def bn(prefix, n, p):
+        p[prefix + ".weight"] = torch.rand(n, generator=g) * 0.5 + 0.75
+        p[prefix + ".bias"] = torch.randn(n, generator=g) * 0.1
+        p[prefix + ".running_mean"] = torch.randn(n, generator=g) * 0.1
+        p[prefix + ".running_var"] = torch.rand(n, generator=g) * 0.5 + 0.75
+
+    r1, r2 = ranks
+    mid = bn_size * growth
+    p = {"features.conv0.weight": kaiming(64, 3, 7, 7)}
+    bn("features.norm0", 64, p)
+    c = 64
+    for b, nl in enumerate(DENSENET121_BLOCKS, start=1):
+        for l in range(1, nl + 1):
+            pre = f"features.denseblock{b}.denselayer{l}"
+            bn(pre + ".norm1", c, p)
+            p[pre + ".conv1.weight"] = kaiming(mid, c, 1, 1)
+            bn(pre + ".norm2", mid, p)
+            p[pre + ".conv2.first_kernel"] = kaiming(r1, mid, 1, 1)
+            p[pre + ".conv2.core_kernel"] = kaiming(r2, r1, 3, 3)
+            p[pre + ".conv2.last_kernel"] = kaiming(growth, r2, 1, 1)
+            c += growth
+        if b < len(DENSENET121_BLOCKS):
+            pre = f"features.transition{b}"
+            bn(pre + ".norm", c, p)
+            p[pre + ".conv.weight"] = kaiming(c // 2, c, 1, 1)
+            c //= 2
+    bn("features.norm5", c, p)
+    p["classifier.weight"] = torch.empty(num_classes, c).normal_(0, 0.01, generator=g)
+    p["classifier.bias"] = torch.randn(num_classes, generator=g) * 0.01
+    return p
+
+
+def build_tucker_densenet121(params, batch=1, H=224, W=224, growth=32):
+    """Finalized Net for the logits [batch, num_classes, 1, 1].  The concatenation of a dense block is one
+    buffer; every layer's Tucker convolution writes its 32 new channels straight into its slice."""
+    p = params
+    net = Net(batch, 3, H, W)
+    s, t = bn_scale_shift(p, "features.norm0")
+    x = net.conv(0, fold_dense(p["features.conv0.weight"], s), t, stride=2, pad=3, relu=True)
+    c = 64
+    h, w = net.shape(x)[2], net.shape(x)[3]
+    h, w = (h + 2 - 3) // 2 + 1, (w + 2 - 3) // 2 + 1
+    cat = net.tensor(c + DENSENET121_BLOCKS[0] * growth, h, w)
+    net.pool(x, "max", 3, 2, 1, dst=net.view(cat, 0, c))
+    for b, nl in enumerate(DENSENET121_BLOCKS, start=1):
+        for l in range(1, nl + 1):
+            pre = f"features.denseblock{b}.denselayer{l}"
+            s1, t1 = bn_scale_shift(p, pre + ".norm1")
+            y = net.affine(net.view(cat, 0, c), s1, t1, relu=True)                 # norm1 + relu on the concatenation
+            s2, t2 = bn_scale_shift(p, pre + ".norm2")
+            y = net.conv(y, fold_dense(p[pre + ".conv1.weight"], s2), t2, relu=True)   # conv1 + norm2 + relu
+            net.tkconv(y, p[pre + ".conv2.first_kernel"], p[pre + ".conv2.core_kernel"], p[pre + ".conv2.last_kernel"],
+                       pad=1, dst=net.view(cat, c, growth))
+            c += growth
+        if b < len(DENSENET121_BLOCKS):
+            pre = f"features.transition{b}"
+            st, tt = bn_scale_shift(p, pre + ".norm")
+            y = net.affine(cat, st, tt, relu=True)
+            y = net.conv(y, p[pre + ".conv.weight"])
+            c //= 2
+            h, w = h // 2, w // 2
+            cat = net.tensor(c + DENSENET121_BLOCKS[b] * growth, h, w)
+            net.pool(y, "avg", 2, 2, 0, dst=net.view(cat, 0, c))
+    s5, t5 = bn_scale_shift(p, "features.norm5")
+    y = net.affine(cat, s5, t5, relu=True)
+    y = net.global_avgpool(y)
+    y = net.conv(y, p["classifier.weight"].reshape(p["classifier.weight"].shape[0], -1, 1, 1), p["classifier.bias"])
+    return net.finalize(y)

@@ -33,6 +33,12 @@ def test_pool_and_concat_ops():
     d = net.concat([0, 0])
     w = torch.randn(4, 12, 1, 1, generator=g)
     e = net.conv(d, w)
+    # in-place concatenation: two producers write channel slices of one buffer, a consumer reads a prefix
+    cat = net.tensor(10, 13, 11)
+    scale, shift = torch.randn(6, generator=g), torch.randn(6, generator=g)
+    net.affine(0, scale, shift, relu=True, dst=net.view(cat, 0, 6))
+    w2 = torch.randn(4, 6, 3, 3, generator=g) * 0.2
+    net.conv(net.view(cat, 0, 6), w2, pad=1, dst=net.view(cat, 6, 4))
     net.finalize(e)
     out = net(x.cuda()).cpu()
     F = torch.nn.functional
@@ -41,7 +47,11 @@ def test_pool_and_concat_ops():
     assert torch.allclose(net.read(c), F.adaptive_avg_pool2d(x, 1), atol=1e-6)
     assert torch.equal(net.read(d), torch.cat([x, x], 1))
     assert torch.allclose(out, F.conv2d(torch.cat([x, x], 1), w), rtol=1e-4, atol=1e-5)
-    assert net.num_kernels == 6
+    aff = torch.relu(x * scale.reshape(1, -1, 1, 1) + shift.reshape(1, -1, 1, 1))
+    got_cat = net.read(cat)
+    assert torch.allclose(got_cat[:, :6], aff, atol=1e-6)
+    assert torch.allclose(got_cat[:, 6:], F.conv2d(aff, w2, None, 1, 1), rtol=1e-4, atol=1e-5)
+    assert net.num_kernels == 8
     net.close()
 
 
@@ -77,4 +87,17 @@ def test_resnet18_batch2_small_resolution():
     net = nets.build_tucker_resnet18(p, batch=2, H=64, W=64)
     got = net(x.cuda()).cpu().numpy().reshape(2, 10)
     scale_close(got, want.numpy(), "logits b2")
+    net.close()
+
+
+@pytest.mark.parametrize("batch,res", [(1, 224), (8, 64)])
+def test_tucker_densenet121(batch, res):
+    """Benchmark configuration 5 (batch 1 at 224x224; batch 8 at a reduced resolution to keep the CPU side short)."""
+    p = nets.densenet121_params(seed=121)
+    x = torch.randn(batch, 3, res, res, generator=torch.Generator().manual_seed(121))
+    want = nets_ref.tucker_densenet121_forward(p, x)
+    net = nets.build_tucker_densenet121(p, batch=batch, H=res, W=res)
+    print("densenet kernels per forward:", net.num_kernels, flush=True)
+    got = net(x.cuda()).cpu().numpy().reshape(batch, 1000)
+    scale_close(got, want.numpy(), f"densenet logits b{batch}")
     net.close()
