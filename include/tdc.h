@@ -166,6 +166,13 @@ int tdc_tkconv_core_forward(tdc_tkconv *op, const float *d_in, float *d_out, voi
 int tdc_tkconv_query(const tdc_tkconv *op, int which, tdc_tile_info *info_out);
 void tdc_tkconv_destroy(tdc_tkconv *op);
 
+/* ---- weight files --------------------------------------------------------------------
+ * Raw little-endian float32, no header: the format of the reference's load_input
+ * (2080Ti-evaluation/EndToEnd/resnet18-tk/src/common.cpp:2-19).  Unlike the reference, a file whose
+ * length is not exactly `count` floats is an error (TDC_ERR_INVALID), not a warning. */
+int tdc_load_bin(const char *path, float *dst_host, uint64_t count);
+int tdc_save_bin(const char *path, const float *src_host, uint64_t count);
+
 /* ---- whole-network forward graphs ----------------------------------------------
  * A net is a list of operators over net-owned device tensors (tensor 0 is the
  * input), captured into one HIP graph by tdc_net_finalize and replayed by

@@ -90,6 +90,31 @@ int tdc_model_select(const tdc_conv_desc *desc, tdc_tile_info *info_out) {
     return TDC_OK;
 }
 
+int tdc_load_bin(const char *path, float *dst, uint64_t count) {
+    if (!path || (!dst && count)) return fail(TDC_ERR_INVALID, "null argument");
+    FILE *f = std::fopen(path, "rb");
+    if (!f) return fail(TDC_ERR_INVALID, std::string("cannot open weight file ") + path);
+    const size_t got = std::fread(dst, sizeof(float), (size_t)count, f);
+    // exactly `count` floats: neither fewer nor a longer file
+    char extra;
+    const bool longer = std::fread(&extra, 1, 1, f) == 1;
+    std::fclose(f);
+    if (got != count || longer)
+        return fail(TDC_ERR_INVALID, std::string("weight file ") + path + " does not hold exactly " + std::to_string(count) +
+                                         " float32 values");
+    return TDC_OK;
+}
+
+int tdc_save_bin(const char *path, const float *src, uint64_t count) {
+    if (!path || (!src && count)) return fail(TDC_ERR_INVALID, "null argument");
+    FILE *f = std::fopen(path, "wb");
+    if (!f) return fail(TDC_ERR_INVALID, std::string("cannot create weight file ") + path);
+    const size_t put = std::fwrite(src, sizeof(float), (size_t)count, f);
+    const int rc = std::fclose(f);
+    if (put != count || rc != 0) return fail(TDC_ERR_INVALID, std::string("short write to ") + path);
+    return TDC_OK;
+}
+
 int tdc_model_get_constants(double *out, int32_t cap, int32_t *count_out) {
     if (!count_out || (cap > 0 && !out)) return fail(TDC_ERR_INVALID, "null argument");
     *count_out = model_constants(out, cap);

@@ -16,7 +16,7 @@ TDC_OK, TDC_ERR_INVALID, TDC_ERR_UNSUPPORTED, TDC_ERR_HIP, TDC_ERR_NOMEM, TDC_ER
 
 # Every symbol include/tdc.h declares.
 EXPORTS = (
-    "tdc_last_error_string", "tdc_version",
+    "tdc_last_error_string", "tdc_version", "tdc_load_bin", "tdc_save_bin",
     "tdc_conv_plan_create", "tdc_conv_plan_set_weights", "tdc_conv_plan_query", "tdc_conv_forward",
     "tdc_conv_forward_strided", "tdc_tkconv_forward_strided",
     "tdc_conv_time", "tdc_conv_time_many", "tdc_conv_plan_destroy",
@@ -84,6 +84,8 @@ def lib():
     fp = POINTER(ctypes.c_float)
     L.tdc_last_error_string.restype = c_char_p
     L.tdc_version.restype = c_char_p
+    L.tdc_load_bin.argtypes = [c_char_p, c_void_p, ctypes.c_uint64]
+    L.tdc_save_bin.argtypes = [c_char_p, c_void_p, ctypes.c_uint64]
     L.tdc_conv_plan_create.argtypes = [POINTER(ConvDesc), POINTER(Tile), POINTER(c_void_p)]
     L.tdc_conv_plan_set_weights.argtypes = [c_void_p, c_void_p, c_void_p]
     L.tdc_conv_plan_query.argtypes = [c_void_p, POINTER(TileInfo)]
