@@ -75,17 +75,20 @@ typedef struct tdc_tile {
     int32_t wk;   /* waves along input channels (in-workgroup split-K)          */
     int32_t cch;  /* input channels staged in LDS per pass                      */
     int32_t tw;   /* output tile width in pixels                               */
+    int32_t ks;   /* workgroups sharing the LDS passes of one tile (split-K across
+                     workgroups, >= 1); partials meet in a plan-owned workspace and are
+                     added in index order by the last workgroup to arrive             */
 } tdc_tile;
 
 typedef struct tdc_tile_info {
     tdc_tile tile;
-    int32_t grid_x, grid_y, grid_z;  /* pixel tiles, channel tiles, batch      */
+    int32_t grid_x, grid_y, grid_z;  /* pixel tiles, channel tiles, batch * ks */
     int32_t block_threads;
     int32_t lds_bytes;
     int32_t vgpr_estimate;           /* per lane, arch+acc                     */
     int32_t waves_per_simd;          /* resident, limited by VGPR/LDS/slots    */
     int32_t wg_per_cu;
-    int32_t nchunks;                 /* LDS passes over input channels         */
+    int32_t nchunks;                 /* LDS passes over all input channels (each workgroup runs ceil(nchunks/ks)) */
     int32_t th;                      /* output tile height in pixels           */
     double flops;                    /* algorithmic 2*Ho*Wo*C*N*KH*KW*batch    */
     double bytes;                    /* algorithmic: in + out + weights once   */

@@ -30,6 +30,11 @@
 //     pre-zeroed output) happens across the wavefronts of ONE workgroup and is
 //     reduced through LDS in a fixed order: no atomics, no pre-zeroing,
 //     bit-reproducible;
+//   * when a layer has too few tiles to occupy the chip, the slabs can also be
+//     dealt to KS workgroups: each writes its partial tile to a workspace, takes
+//     a ticket from a per-tile counter, and the workgroup that draws the last
+//     ticket adds the KS partials in index order — still no atomics on data
+//     and no dependence on arrival order;
 //   * tiles are two-dimensional (TH x TW), so the halo is paid on a short
 //     perimeter instead of on whole image rows;
 //   * bias, residual add and ReLU are fused into the store.
@@ -163,7 +168,7 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
                  "s"(p.ntx), "s"(p.stride), "s"(p.pad), "s"(p.VW), "s"(p.in_stage_floats), "s"(p.wslab_floats),
                  "s"(p.stage_floats), "s"(p.nstage), "s"(p.nchunks), "s"(p.fd_csv.m), "s"(p.fd_csv.d),
                  "s"(p.fd_rsv.m), "s"(p.fd_rsv.d), "s"(p.fd_ntx.m), "s"(p.fd_wk.m), "s"(p.fd_wn.m), "s"(p.WK),
-                 "s"(p.WN), "s"(p.in_bstride), "s"(p.wpk_bytes));
+                 "s"(p.WN), "s"(p.in_bstride), "s"(p.wpk_bytes), "s"(p.KS), "s"(p.cps), "s"(p.fd_ks.m));
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -181,10 +186,14 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
     const int oy0 = tile_y * p.TH;
     const int ox0 = tile_x * p.TW;
     const int m0 = blockIdx.y * MT;
-    const float *__restrict__ in = p.in + (long long)blockIdx.z * p.in_bstride;
-    float *__restrict__ out = p.out + (long long)blockIdx.z * p.out_bstride;
-    const float *__restrict__ resid =
-        p.resid ? p.resid + (long long)blockIdx.z * p.resid_bstride : nullptr;
+    // blockIdx.z = image * KS + slice of the input-channel passes
+    const int img = fdiv(blockIdx.z, p.fd_ks);
+    const int ks = blockIdx.z - img * p.KS;
+    const int chunk0 = ks * p.cps;
+    const int chunk1 = min(chunk0 + p.cps, p.nchunks);
+    const float *__restrict__ in = p.in + (long long)img * p.in_bstride;
+    float *__restrict__ out = p.out + (long long)img * p.out_bstride;
+    const float *__restrict__ resid = p.resid ? p.resid + (long long)img * p.resid_bstride : nullptr;
     // Raw buffers: byte offsets at or beyond num_records read as zero.
     const __amdgpu_buffer_rsrc_t in_rsrc =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(in), (short)0, (int)p.in_image_bytes, 0x00020000);
@@ -210,11 +219,11 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
     }
     const int lane16 = lane * 16;
     auto issue = [&](int chunk) {
-        float *stage = lds + (chunk & (p.nstage - 1)) * p.stage_floats;
+        float *stage = lds + ((chunk - chunk0) & (p.nstage - 1)) * p.stage_floats;
         const int w_byte0 = (int)(w_byte_base + (unsigned)chunk * w_pass_bytes);
         issue_pass(p, in_rsrc, w_rsrc, stage, pre, lane16, chunk, iy0, ix0a, w_byte0, wave, nwaves, lane);
     };
-    issue(0);
+    issue(chunk0);
 
     // Per-lane LDS offset (floats) of tap (0,0) for each pixel block, channel sub-index included.
     int boff[NB];
@@ -239,14 +248,14 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
     const int ncg_pass = p.CCH / KC;  // channel groups per pass
     const int ncgw = p.CPW / KC;      // ... of which this wave takes [wk*ncgw, (wk+1)*ncgw)
 
-    for (int chunk = 0; chunk < p.nchunks; ++chunk) {
+    for (int chunk = chunk0; chunk < chunk1; ++chunk) {
         // My copies of this pass have landed; after the barrier everybody's have, and
         // everybody is done reading the stage the next pass is about to overwrite.
         __builtin_amdgcn_s_waitcnt(0);
         __syncthreads();
-        if (chunk + 1 < p.nchunks) issue(chunk + 1);
+        if (chunk + 1 < chunk1) issue(chunk + 1);
 
-        const float *stage = lds + (chunk & (p.nstage - 1)) * p.stage_floats;
+        const float *stage = lds + ((chunk - chunk0) & (p.nstage - 1)) * p.stage_floats;
         const float *sin = stage + wk * p.CPW * p.CS;
         const float *sw[MB];
 #pragma unroll
@@ -353,36 +362,11 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
         }
     }
 
-    if (p.WK == 1) {
-        // Straight from the accumulators: each store instruction writes runs of
-        // consecutive pixels of one output channel.
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb) {
-            const int j = (wn * NB + nb) * MF + M::col(lane);
-            const int jy = fdiv(j, p.fd_tw);
-            const int jx = j - jy * p.TW;
-            const int oy = oy0 + jy, ox = ox0 + jx;
-            const bool pix_ok = jy < p.TH && oy < p.Ho && ox < p.Wo;
-            const int pp = oy * p.Wo + ox;
-#pragma unroll
-            for (int mb = 0; mb < MB; ++mb) {
-#pragma unroll
-                for (int v = 0; v < NACC; ++v) {
-                    const int n = m0 + (wm * MB + mb) * MF + M::row(v, lane);
-                    if (n < p.N && pix_ok) {
-                        float val = acc[mb][nb][v];
-                        if (p.bias) val += p.bias[n];
-                        const long long o = (long long)n * p.P + pp;
-                        if (resid) val += resid[o];
-                        if (p.relu) val = fmaxf(val, 0.0f);
-                        out[o] = val;
-                    }
-                }
-            }
-        }
-    } else {
+    // Epilogue.  `each_output(sink)` walks this thread's share of the workgroup's output tile and
+    // hands (channel, pixel offset in the image, accumulated value) to the sink.
+    if (p.WK > 1) {
         // Split-K across waves: park every wave's partial tile in LDS
-        // ([wk][channel][pixel lane]) and add the WK slices in index order.
+        // ([wk][channel][pixel lane]); the walk below adds the WK slices in index order.
         __syncthreads();
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) {
@@ -397,25 +381,104 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
             }
         }
         __syncthreads();
-        const int total = MT * PT;
-        for (int idx = tid; idx < total; idx += nthreads) {
-            const int ml = fdiv(idx, p.fd_pt);
-            const int j = idx - ml * PT;
-            const int jy = fdiv(j, p.fd_tw);
-            const int jx = j - jy * p.TW;
-            const int n = m0 + ml;
-            const int oy = oy0 + jy, ox = ox0 + jx;
-            if (n < p.N && jy < p.TH && oy < p.Ho && ox < p.Wo) {
-                float val = lds[idx];
-                for (int k = 1; k < p.WK; ++k) val += lds[k * total + idx];
-                if (p.bias) val += p.bias[n];
-                const long long o = (long long)n * p.P + oy * p.Wo + ox;
-                if (resid) val += resid[o];
-                if (p.relu) val = fmaxf(val, 0.0f);
-                out[o] = val;
+    }
+    auto each_output = [&](auto &&sink, bool want_value) {
+        if (p.WK == 1) {
+            // Straight from the accumulators: each store instruction writes runs of
+            // consecutive pixels of one output channel.
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+                const int j = (wn * NB + nb) * MF + M::col(lane);
+                const int jy = fdiv(j, p.fd_tw);
+                const int jx = j - jy * p.TW;
+                const int oy = oy0 + jy, ox = ox0 + jx;
+                const bool pix_ok = jy < p.TH && oy < p.Ho && ox < p.Wo;
+                const int pp = oy * p.Wo + ox;
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb) {
+#pragma unroll
+                    for (int v = 0; v < NACC; ++v) {
+                        const int n = m0 + (wm * MB + mb) * MF + M::row(v, lane);
+                        if (n < p.N && pix_ok) sink(n, pp, acc[mb][nb][v]);
+                    }
+                }
+            }
+        } else {
+            const int total = MT * PT;
+            for (int idx = tid; idx < total; idx += nthreads) {
+                const int ml = fdiv(idx, p.fd_pt);
+                const int j = idx - ml * PT;
+                const int jy = fdiv(j, p.fd_tw);
+                const int jx = j - jy * p.TW;
+                const int n = m0 + ml;
+                const int oy = oy0 + jy, ox = ox0 + jx;
+                if (n < p.N && jy < p.TH && oy < p.Ho && ox < p.Wo) {
+                    float val = 0.0f;
+                    if (want_value) {
+                        val = lds[idx];
+                        for (int k = 1; k < p.WK; ++k) val += lds[k * total + idx];
+                    }
+                    sink(n, oy * p.Wo + ox, val);
+                }
             }
         }
+    };
+    auto finish = [&](int n, int pp, float val) {
+        if (p.bias) val += p.bias[n];
+        const long long o = (long long)n * p.P + pp;
+        if (resid) val += resid[o];
+        if (p.relu) val = fmaxf(val, 0.0f);
+        out[o] = val;
+    };
+    if (p.KS == 1) {
+        each_output(finish, true);
+        return;
     }
+
+    // Split-K across workgroups.  Partial tiles go to ws[image][slice][channel][pixel]; the counter of
+    // this (image, channel tile, pixel tile) hands out tickets, and whoever draws the last one finds
+    // all KS partials complete.  The compute dies do not share an L2, and a device-scope fence would
+    // write back and invalidate a whole L2 per workgroup — tens of microseconds.  Instead every access
+    // to the workspace is itself a device-scope (relaxed) atomic: the stores write through, the loads
+    // bypass the die-local L2, and "my stores are done" is the plain wait below.
+    const long long NP = (long long)p.N * p.P;
+    float *wsz = p.ws + (long long)blockIdx.z * NP;
+    each_output(
+        [&](int n, int pp, float val) {
+            __hip_atomic_store(wsz + (long long)n * p.P + pp, val, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        },
+        true);
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    unsigned *ticket = p.ctr + ((unsigned)img * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
+    if (tid == 0) {
+        const unsigned drawn = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        reinterpret_cast<unsigned *>(lds)[0] = drawn;
+    }
+    __syncthreads();
+    const unsigned drawn = reinterpret_cast<const unsigned *>(lds)[0];
+    if (drawn != (unsigned)p.KS - 1u) return;
+    if (tid == 0) __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
+    const float *ws0 = p.ws + (long long)img * p.KS * NP;
+    each_output(
+        [&](int n, int pp, float) {
+            const long long o = (long long)n * p.P + pp;
+            // Four loads in flight at a time; the additions stay in slice order.
+            float val = 0.0f;
+            for (int k0 = 0; k0 < p.KS; k0 += 4) {
+                float part[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const int k = min(k0 + u, p.KS - 1);
+                    part[u] = __hip_atomic_load(ws0 + k * NP + o, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u)
+                    if (k0 + u < p.KS) val += part[u];
+            }
+            finish(n, pp, val);
+        },
+        false);
 }
 
 // ---------------------------------------------------------------------------

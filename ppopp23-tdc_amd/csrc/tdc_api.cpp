@@ -43,8 +43,19 @@ struct tdc_conv_plan {
     const void *kernel = nullptr;
     float *d_wpk = nullptr;
     float *d_bias = nullptr;
+    float *d_ws = nullptr;        // tile.ks > 1: partial tiles [batch][ks][N][P]
+    unsigned *d_ctr = nullptr;    // tile.ks > 1: ticket counters, zero between launches
     bool have_weights = false;
 };
+
+static void free_plan_buffers(tdc_conv_plan *p) {
+    if (p->d_wpk) (void)hipFree(p->d_wpk);
+    if (p->d_bias) (void)hipFree(p->d_bias);
+    if (p->d_ws) (void)hipFree(p->d_ws);
+    if (p->d_ctr) (void)hipFree(p->d_ctr);
+    p->d_wpk = p->d_bias = p->d_ws = nullptr;
+    p->d_ctr = nullptr;
+}
 
 struct tdc_tkconv {
     tdc_tkconv_desc desc{};
@@ -156,8 +167,19 @@ int tdc_conv_plan_create(const tdc_conv_desc *desc, const tdc_tile *forced_tile,
     if (desc->has_bias) {
         e = hipMalloc((void **)&p->d_bias, (size_t)desc->N * sizeof(float));
         if (e != hipSuccess) {
-            (void)hipFree(p->d_wpk);
+            free_plan_buffers(p.get());
             return hip_fail("hipMalloc(bias)", e);
+        }
+    }
+    if (p->tile.ks > 1) {
+        const size_t ws_floats = (size_t)p->geo.grid_z * desc->N * p->geo.P;
+        const size_t nctr = (size_t)desc->batch * p->geo.grid_y * p->geo.grid_x;
+        e = hipMalloc((void **)&p->d_ws, ws_floats * sizeof(float));
+        if (e == hipSuccess) e = hipMalloc((void **)&p->d_ctr, nctr * sizeof(unsigned));
+        if (e == hipSuccess) e = hipMemset(p->d_ctr, 0, nctr * sizeof(unsigned));
+        if (e != hipSuccess) {
+            free_plan_buffers(p.get());
+            return hip_fail("hipMalloc(split-K workspace)", e);
         }
     }
     *plan_out = p.release();
@@ -214,6 +236,8 @@ int tdc_conv_forward_strided(tdc_conv_plan *plan, const float *d_in, int64_t in_
     kp.bias = plan->d_bias;
     kp.resid = d_residual;
     kp.out = d_out;
+    kp.ws = plan->d_ws;
+    kp.ctr = plan->d_ctr;
     kp.in_image_bytes = (unsigned)(in_image * 4);
     kp.in_bstride = in_batch_stride ? in_batch_stride : in_image;
     kp.out_bstride = out_batch_stride ? out_batch_stride : out_image;
@@ -224,6 +248,7 @@ int tdc_conv_forward_strided(tdc_conv_plan *plan, const float *d_in, int64_t in_
     kp.TW = g.TW; kp.TH = g.TH; kp.ntx = g.ntx;
     kp.WM = plan->tile.wm; kp.WN = plan->tile.wn; kp.WK = plan->tile.wk;
     kp.CCH = plan->tile.cch; kp.nchunks = g.nchunks; kp.CPW = g.cpw;
+    kp.KS = g.ks; kp.cps = g.cps;
     kp.RS = g.RS; kp.CS = g.CS; kp.nrows = g.nrows;
     // 16-byte copy elements need every image of the batch 16-byte aligned; otherwise 4-byte elements.
     const bool aligned = reinterpret_cast<uintptr_t>(d_in) % 16 == 0 && kp.in_bstride % 4 == 0;
@@ -238,6 +263,7 @@ int tdc_conv_forward_strided(tdc_conv_plan *plan, const float *d_in, int64_t in_
     kp.fd_pt = make_fastdiv(g.PT);
     kp.fd_wk = make_fastdiv(plan->tile.wk);
     kp.fd_wn = make_fastdiv(plan->tile.wn);
+    kp.fd_ks = make_fastdiv(g.ks);
     kp.wpk_bytes = (unsigned)(packed_weight_floats(g) * sizeof(float));
     int he = launch_conv(plan->kernel, g, kp, stream);
     if (he) return hip_fail("kernel launch", he);
@@ -344,8 +370,7 @@ int tdc_conv_time(tdc_conv_plan *plan, const float *d_in, const float *d_residua
 
 void tdc_conv_plan_destroy(tdc_conv_plan *plan) {
     if (!plan) return;
-    if (plan->d_wpk) (void)hipFree(plan->d_wpk);
-    if (plan->d_bias) (void)hipFree(plan->d_bias);
+    free_plan_buffers(plan);
     delete plan;
 }
 

@@ -40,7 +40,9 @@ struct Geometry {
     int grid_x = 0, grid_y = 0, grid_z = 0;
     int waves = 0, threads = 0;
     int cpw = 0;                     // channels per wave per LDS pass (cch / wk)
-    int nchunks = 0;                 // LDS passes
+    int nchunks = 0;                 // LDS passes over all input channels
+    int ks = 1;                      // workgroups sharing those passes (split-K across workgroups)
+    int cps = 0;                     // passes per workgroup: ceil(nchunks / ks)
     int c_pad = 0;                   // nchunks * cch
     int VW = 1;                      // floats per element of the LDS fill (4 if We%4==0, else 1)
     int nrows = 0, ncols = 0;        // input window of one tile
@@ -92,17 +94,20 @@ struct ConvKParams {
     const float *bias;
     const float *resid;
     float *out;
+    float *ws;                 // partial tiles of a split across workgroups: [image][slice][N][P]
+    unsigned *ctr;             // one ticket counter per (image, channel tile, pixel tile), zero between launches
     int C, H, W, N, Ho, Wo, P;
     int KH, KW, stride, pad, dil;
     int TW, TH, ntx;
     int WM, WN, WK;
     int CCH, nchunks, CPW;
+    int KS, cps;               // slices across workgroups, passes per slice
     int RS, CS, VW, nrows;
     int in_stage_floats, wslab_floats, stage_floats, nstage;
     int relu;
     FastDiv fd_csv, fd_rsv;      // LDS channel slot / row, in copy elements
     FastDiv fd_tw, fd_ntx, fd_pt;
-    FastDiv fd_wk, fd_wn;
+    FastDiv fd_wk, fd_wn, fd_ks;
     unsigned wpk_bytes;
     unsigned in_image_bytes;   // C*H*W*4: reads at or past it return zero
     long long in_bstride;      // floats between consecutive images of the input (C*H*W when dense)

@@ -95,14 +95,19 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
     if ((long long)g.ntx * g.nty * g.ntx >= (1LL << 32)) return fail("grid too large");
     g.grid_x = g.ntx * g.nty;
     g.grid_y = ceil_div(d.N, g.MT);
-    g.grid_z = d.batch;
-    if (g.grid_y > 65535 || g.grid_z > 65535) return fail("grid too large");
+    if (t.ks < 1 || t.ks > 64) return fail("tile.ks must be in [1, 64]");
+    g.ks = t.ks;
+    if ((long long)d.batch * t.ks > 65535) return fail("grid too large");
+    g.grid_z = d.batch * t.ks;
+    if (g.grid_y > 65535) return fail("grid too large");
     const int granule = g.kc * t.wk;
     if (t.cch < granule || t.cch % granule != 0) return fail("tile.cch must be a positive multiple of kc*wk");
     if (t.cch > round_up(d.C, granule)) return fail("tile.cch exceeds the (padded) channel count");
     g.cpw = t.cch / t.wk;
     g.nchunks = ceil_div(d.C, t.cch);
     g.c_pad = g.nchunks * t.cch;
+    g.cps = ceil_div(g.nchunks, t.ks);
+    if ((t.ks - 1) * g.cps >= g.nchunks) return fail("tile.ks leaves a workgroup without input channels");
     g.nrows = (g.TH - 1) * d.stride + (d.KH - 1) * d.dilation + 1;
     g.ncols = (g.TW - 1) * d.stride + (d.KW - 1) * d.dilation + 1;
     // LDS rows are filled with 16-byte elements when image rows are a multiple of
@@ -125,7 +130,7 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
     g.in_stage_floats = round_up(t.cch * g.CS, 256);
     g.wslab_floats = (t.wm * t.mb) * (t.cch / g.kc) * g.taps * 64;
     g.stage_floats = g.in_stage_floats + round_up(g.wslab_floats, 256);
-    g.nstage = g.nchunks > 1 ? 2 : 1;
+    g.nstage = g.cps > 1 ? 2 : 1;
     const long long stage_bytes = (long long)g.nstage * g.stage_floats * 4;
     const long long red_bytes = t.wk > 1 ? (long long)t.wk * g.MT * g.PT * 4 : 0;
     const long long lds = std::max(stage_bytes, red_bytes);
@@ -179,9 +184,10 @@ struct ModelConst {
     double kstep_issue_clk = 4.35;       // vector-ALU / LDS-issue cycles per operand read, not hidden under MFMAs
     double pass_overhead_clk = 424;   // per wave and pass: copy issue, pointer set-up, pipeline fill
     double wave_setup_clk = 2.2;      // prologue cycles added per extra wave sharing a SIMD
+    double ksplit_clk = 4500;         // split across workgroups: device-scope fences and the ticket round trip
 };
 ModelConst MC;
-constexpr int kNumModelConst = 11;
+constexpr int kNumModelConst = 12;
 
 double *mc_field(int i) {
     switch (i) {
@@ -196,6 +202,7 @@ double *mc_field(int i) {
         case 8: return &MC.kstep_issue_clk;
         case 9: return &MC.pass_overhead_clk;
         case 10: return &MC.wave_setup_clk;
+        case 11: return &MC.ksplit_clk;
         default: return nullptr;
     }
 }
@@ -270,9 +277,14 @@ bool model_evaluate(const tdc_conv_desc &d, const tdc_tile &t, tdc_tile_info &in
         // First pass is exposed; afterwards the copy of pass i+1 runs under the MFMAs of pass i.
         double clk = MC.setup_clk + MC.wave_setup_clk * (waves_simd - 1.0) + MC.copy_latency_clk + copy;
         clk += compute;  // last pass: nothing left to hide
-        if (g.nchunks > 1) clk += (g.nchunks - 1) * std::max(compute, copy + MC.copy_latency_clk);
+        if (g.cps > 1) clk += (g.cps - 1) * std::max(compute, copy + MC.copy_latency_clk);
         clk += red_bytes * r / MC.lds_bytes_per_clk + out_bytes * r / MC.store_bytes_per_clk +
                (t.wk > 1 ? 2.0 * MC.sync_clk : 0.0);
+        // Split across workgroups: the partial tile goes to the workspace (the store above), and the
+        // workgroup that draws the last ticket reads all ks partials back before the real store.
+        if (t.ks > 1)
+            clk += MC.ksplit_clk + MC.copy_latency_clk + (double)t.ks * out_bytes / rate +
+                   out_bytes / MC.store_bytes_per_clk;
         return clk;
     };
     const long long slots = (long long)m.cus * wg_per_cu;
@@ -281,7 +293,7 @@ bool model_evaluate(const tdc_conv_desc &d, const tdc_tile &t, tdc_tile_info &in
     double clk = (double)full * wg_time(wg_per_cu, slots);
     if (rem) clk += wg_time((int)((rem + m.cus - 1) / m.cus), rem);
     info.pred_us = MC.launch_us + clk / (m.clock_ghz * 1e3);
-    info.pred_l2_bytes = (double)n_wg * g.nchunks * copy_bytes_pass;
+    info.pred_l2_bytes = (double)n_wg * g.cps * copy_bytes_pass;
     return true;
 }
 
@@ -333,12 +345,18 @@ std::vector<tdc_tile> model_enumerate(const tdc_conv_desc &d) {
                                 if (fixed % granule == 0 && fixed < c_full &&
                                     std::find(cchs.begin(), cchs.end(), fixed) == cchs.end())
                                     cchs.push_back(fixed);
+                            // Splitting the passes over several workgroups only pays while the
+                            // layer has fewer tiles than the chip has room for.
+                            const long long max_wgs = 4LL * machine().cus;
                             for (int tw : tws)
-                                for (int cch : cchs) {
-                                    tdc_tile t{mf, mb, nb, wm, wn, wk, cch, tw};
-                                    Geometry g;
-                                    if (make_geometry(d, t, g, nullptr)) out.push_back(t);
-                                }
+                                for (int cch : cchs)
+                                    for (int ks : {1, 2, 4, 8}) {
+                                        tdc_tile t{mf, mb, nb, wm, wn, wk, cch, tw, ks};
+                                        Geometry g;
+                                        if (!make_geometry(d, t, g, nullptr)) continue;
+                                        if (ks > 1 && (long long)g.grid_x * g.grid_y * g.grid_z > max_wgs) continue;
+                                        out.push_back(t);
+                                    }
                         }
     }
     return out;

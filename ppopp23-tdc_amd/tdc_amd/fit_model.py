@@ -25,7 +25,8 @@ def load(paths):
     for path in paths:
         for r in csv.DictReader(open(path)):
             key = tuple(int(r[k]) for k in ("C", "N", "H", "W", "K", "stride"))
-            tile = _lib.Tile(*[int(r[k]) for k in ("mf", "mb", "nb", "wm", "wn", "wk", "cch", "tw")])
+            tile = _lib.Tile(*[int(r[k]) for k in ("mf", "mb", "nb", "wm", "wn", "wk", "cch", "tw")],
+                             ks=int(r.get("ks") or 1))
             layers[key].append((tile, float(r["time_us"])))
     return layers
 

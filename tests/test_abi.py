@@ -36,10 +36,11 @@ def test_version_and_error_string():
 
 def test_struct_layouts_match_the_header():
     assert ctypes.sizeof(_lib.ConvDesc) == 12 * 4
-    assert ctypes.sizeof(_lib.Tile) == 8 * 4
+    assert ctypes.sizeof(_lib.Tile) == 9 * 4
     assert ctypes.sizeof(_lib.TKConvDesc) == 13 * 4
-    # tile (8 ints) + 10 ints + 5 doubles, 8-byte aligned
-    assert ctypes.sizeof(_lib.TileInfo) == 8 * 4 + 10 * 4 + 5 * 8
+    # tile (9 ints) + 10 ints, padded to 8-byte alignment, + 5 doubles
+    assert ctypes.sizeof(_lib.TileInfo) == 9 * 4 + 10 * 4 + 4 + 5 * 8
+    assert _lib.TileInfo.flops.offset == 80
 
 
 def test_invalid_descriptors_are_rejected_with_a_reason():

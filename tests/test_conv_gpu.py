@@ -144,6 +144,41 @@ def test_deterministic_bitwise():
     assert np.array_equal(a, b)
 
 
+@pytest.mark.parametrize("tile", [tdc_amd.Tile(16, 1, 1, 1, 1, 1, 8, 8, ks=5),      # 5 slices of one pass each
+                                  tdc_amd.Tile(16, 1, 1, 2, 1, 2, 16, 8, ks=2) ,    # 3 passes over 2 slices: 2 + 1
+                                  tdc_amd.Tile(32, 1, 2, 1, 1, 4, 8, 9, ks=3),
+                                  tdc_amd.Tile(32, 2, 2, 1, 1, 1, 4, 9, ks=10)])
+def test_split_across_workgroups(tile):
+    """Input-channel passes dealt to several workgroups (tile.ks > 1): same answer as the oracle with the whole
+    epilogue, the same bits on every launch, and the ticket counters are back at zero for the next launch."""
+    announce("ksplit", tile)
+    B, C, N, H, W = 2, 40, 37, 9, 9
+    x, w = case(6000, B, C, N, H, W, 3)
+    g = seeded(6001)
+    bias = torch.randn(N, generator=g)
+    resid = torch.randn(B, N, H, W, generator=g)
+    want = ref.conv2d_c(x.numpy(), w.numpy(), bias.numpy(), resid.numpy(), pad=1, relu=True)
+    plan = tdc_amd.Conv2dPlan(B, C, N, H, W, 3, 3, 1, 1, 1, True, True, tile=tile).set_weights(w, bias)
+    assert plan.info.grid_z == B * tile.ks
+    xd, rd = x.cuda(), resid.cuda()
+    outs = []
+    for rep in range(3):
+        out = torch.full((B, N, H, W), float("nan"), device="cuda")
+        plan.forward(xd, rd, out=out)
+        torch.cuda.synchronize()
+        outs.append(out.cpu().numpy())
+    plan.close()
+    assert_close(outs[0], want, f"split-K {tile}")
+    assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2])
+
+
+def test_split_across_workgroups_rejects_empty_slices():
+    with pytest.raises(tdc_amd.TdcError):   # 40 channels in passes of 8 = 5 passes: 4 slices take 2,2,1,0
+        tdc_amd.model_evaluate(tdc_amd.conv_desc(1, 40, 16, 9, 9, 3, 3, 1, 1), tdc_amd.Tile(16, 1, 1, 1, 1, 1, 8, 8, ks=4))
+    with pytest.raises(tdc_amd.TdcError):
+        tdc_amd.model_evaluate(tdc_amd.conv_desc(1, 40, 16, 9, 9, 3, 3, 1, 1), tdc_amd.Tile(16, 1, 1, 1, 1, 1, 8, 8, ks=0))
+
+
 def test_linearity_full_size():
     """Size-independent property at the largest sweep shape: conv(a*x1 + x2) == a*conv(x1) + conv(x2)."""
     x1, w = ref.make_core_case(56, 128, 128)
