@@ -64,7 +64,7 @@ typedef struct tdc_conv_desc {
 /* Tiling of one convolution on the gfx950 compute unit.  One workgroup computes
  * (mf*mb*wm) output channels of a th x tw tile of output pixels (th is derived:
  * as many rows as fit in the workgroup's mf*nb*wn pixel lanes); its wm*wn*wk
- * wavefronts split output channels, pixels and input channels; input channels
+ * computing wavefronts split output channels, pixels and input channels; input channels
  * are staged through LDS `cch` at a time, double-buffered. */
 typedef struct tdc_tile {
     int32_t mf;   /* MFMA block edge: 32 (v_mfma_f32_32x32x2_f32) or 16 (16x16x4) */
@@ -78,6 +78,8 @@ typedef struct tdc_tile {
     int32_t ks;   /* workgroups sharing the LDS passes of one tile (split-K across
                      workgroups, >= 1); partials meet in a plan-owned workspace and are
                      added in index order by the last workgroup to arrive             */
+    int32_t wl;   /* extra wavefronts that only issue the global->LDS copies of the
+                     next pass while the wm*wn*wk others compute (0 = every wave does both) */
 } tdc_tile;
 
 typedef struct tdc_tile_info {

@@ -128,30 +128,36 @@ __device__ __forceinline__ void copy_block(int vw, __amdgpu_buffer_rsrc_t rsrc, 
 }
 
 // Start the copies of pass `chunk` into the LDS stage at `stage`.  Nothing is
-// waited for here.  Everything that does not depend on the lane is kept in
-// scalar registers: vector ALU instructions issued next to MFMAs are not free.
+// waited for here.  The blocks are dealt to `dn` waves, of which this one is
+// number `dw`; `use_pre` says that pre[] was computed for this dealing.
+// Everything that does not depend on the lane is kept in scalar registers:
+// vector ALU instructions issued next to MFMAs are not free.
 __device__ __forceinline__ void issue_pass(const ConvKParams &p, __amdgpu_buffer_rsrc_t in_rsrc,
                                            __amdgpu_buffer_rsrc_t w_rsrc, float *__restrict__ stage,
-                                           const int (&pre)[MAXPRE], int lane16, int chunk, int iy0, int ix0a,
-                                           int w_byte0, int wave, int nwaves, int lane) {
+                                           const int (&pre)[MAXPRE], bool use_pre, int lane16, int chunk, int iy0,
+                                           int ix0a, int w_byte0, int dw, int dn, int lane) {
     const int VW = p.VW;
     const int blk_floats = 64 * VW;
     const int nblk = p.in_stage_floats / blk_floats;
     // This pass starts chunk*CCH channels further on.  The shift goes through the vector offset on
     // purpose: only that one is range-checked, and channels past C must read as zero.
     const int pass_bytes = chunk * p.CCH * p.H * p.W * 4;
+    int first_computed = dw;
+    if (use_pre) {
 #pragma unroll
-    for (int i = 0; i < MAXPRE; ++i) {
-        const int blk = wave + i * nwaves;
-        if (blk < nblk) copy_block(VW, in_rsrc, stage + blk * blk_floats, pre[i] + pass_bytes, 0);
+        for (int i = 0; i < MAXPRE; ++i) {
+            const int blk = dw + i * dn;
+            if (blk < nblk) copy_block(VW, in_rsrc, stage + blk * blk_floats, pre[i] + pass_bytes, 0);
+        }
+        first_computed = dw + MAXPRE * dn;
     }
-    for (int blk = wave + MAXPRE * nwaves; blk < nblk; blk += nwaves)
+    for (int blk = first_computed; blk < nblk; blk += dn)
         copy_block(VW, in_rsrc, stage + blk * blk_floats, input_copy_offset(p, (blk << 6) + lane, iy0, ix0a) + pass_bytes, 0);
     // Weights: a linear copy in 16-byte elements, 1 KiB per instruction; always inside the packed buffer
     // (or past its end, which reads as zero into the slack), so the block offset can ride in the scalar operand.
     float *wdst = stage + p.in_stage_floats;
     const int wnblk = (p.wslab_floats + 255) >> 8;
-    for (int blk = wave; blk < wnblk; blk += nwaves) copy_block(4, w_rsrc, wdst + (blk << 8), lane16, w_byte0 + (blk << 10));
+    for (int blk = dw; blk < wnblk; blk += dn) copy_block(4, w_rsrc, wdst + (blk << 8), lane16, w_byte0 + (blk << 10));
 }
 
 template <int MF, int MB, int NB, int TAPS, int MAXW>
@@ -168,14 +174,22 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
                  "s"(p.ntx), "s"(p.stride), "s"(p.pad), "s"(p.VW), "s"(p.in_stage_floats), "s"(p.wslab_floats),
                  "s"(p.stage_floats), "s"(p.nstage), "s"(p.nchunks), "s"(p.fd_csv.m), "s"(p.fd_csv.d),
                  "s"(p.fd_rsv.m), "s"(p.fd_rsv.d), "s"(p.fd_ntx.m), "s"(p.fd_wk.m), "s"(p.fd_wn.m), "s"(p.WK),
-                 "s"(p.WN), "s"(p.in_bstride), "s"(p.wpk_bytes), "s"(p.KS), "s"(p.cps), "s"(p.fd_ks.m));
+                 "s"(p.WN), "s"(p.in_bstride), "s"(p.wpk_bytes), "s"(p.KS), "s"(p.cps), "s"(p.fd_ks.m), "s"(p.WL));
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int nthreads = blockDim.x;
     const int nwaves = nthreads >> 6;
-    const int wave_nk = fdiv(wave, p.fd_wk);  // wave = (wm * WN + wn) * WK + wk
-    const int wk = wave - wave_nk * p.WK;
+    // The last WL waves of the workgroup are loaders: after the first pass they issue all copies and
+    // take no part in the matrix work, so the computing waves never stall on copy issue (a wave can
+    // start an LDS copy only about once per hundred cycles).  WL == 0: everybody copies and computes.
+    const int ncomp = nwaves - p.WL;
+    const bool loader = wave >= ncomp;
+    const int dw = p.WL ? wave - ncomp : wave;  // this wave's place among the dn waves that copy
+    const int dn = p.WL ? p.WL : nwaves;
+    const int cwave = loader ? 0 : wave;
+    const int wave_nk = fdiv(cwave, p.fd_wk);  // computing wave = (wm * WN + wn) * WK + wk
+    const int wk = cwave - wave_nk * p.WK;
     const int wm = fdiv(wave_nk, p.fd_wn);
     const int wn = wave_nk - wm * p.WN;
 
@@ -208,22 +222,25 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
     const unsigned w_pass_bytes = (unsigned)p.wslab_floats * 4u;
     const unsigned w_byte_base = (unsigned)blockIdx.y * (unsigned)p.nchunks * w_pass_bytes;
 
-    // Offsets of this lane's elements in its wave's first MAXPRE input blocks (pass 0).
+    // Offsets of this lane's elements in its wave's first MAXPRE input blocks (pass 0), for the steady dealing.
     int pre[MAXPRE];
 #pragma unroll
     for (int i = 0; i < MAXPRE; ++i) {
-        const int e = ((wave + i * nwaves) << 6) + lane;
+        const int e = ((dw + i * dn) << 6) + lane;
         pre[i] = OOB_OFFSET;
-        if (e < p.in_stage_floats)  // (in elements this bound is only tighter)
+        if (e < p.in_stage_floats && dw >= 0)  // (in elements this bound is only tighter)
             pre[i] = input_copy_offset(p, e, iy0, ix0a);
     }
     const int lane16 = lane * 16;
-    auto issue = [&](int chunk) {
+    auto issue = [&](int chunk, bool everybody) {
         float *stage = lds + ((chunk - chunk0) & (p.nstage - 1)) * p.stage_floats;
         const int w_byte0 = (int)(w_byte_base + (unsigned)chunk * w_pass_bytes);
-        issue_pass(p, in_rsrc, w_rsrc, stage, pre, lane16, chunk, iy0, ix0a, w_byte0, wave, nwaves, lane);
+        if (everybody)
+            issue_pass(p, in_rsrc, w_rsrc, stage, pre, p.WL == 0, lane16, chunk, iy0, ix0a, w_byte0, wave, nwaves, lane);
+        else if (dw >= 0)
+            issue_pass(p, in_rsrc, w_rsrc, stage, pre, true, lane16, chunk, iy0, ix0a, w_byte0, dw, dn, lane);
     };
-    issue(chunk0);
+    issue(chunk0, true);
 
     // Per-lane LDS offset (floats) of tap (0,0) for each pixel block, channel sub-index included.
     int boff[NB];
@@ -253,7 +270,8 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
         // everybody is done reading the stage the next pass is about to overwrite.
         __builtin_amdgcn_s_waitcnt(0);
         __syncthreads();
-        if (chunk + 1 < chunk1) issue(chunk + 1);
+        if (chunk + 1 < chunk1) issue(chunk + 1, false);
+        if (loader) continue;
 
         const float *stage = lds + ((chunk - chunk0) & (p.nstage - 1)) * p.stage_floats;
         const float *sin = stage + wk * p.CPW * p.CS;
@@ -293,53 +311,77 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
 #pragma unroll
                         for (int nb = 0; nb < NB; ++nb) acc[mb][nb] = M::run(a[t][mb], b[t][nb], acc[mb][nb]);
             };
+            // One scheduling region = the MFMAs of one group next to the LDS reads of the following one,
+            // interleaved: a wave issues in order, so reads issued in one batch would leave the matrix
+            // pipe idle for as long as the batch takes to issue.
+            auto interleave = [&]() {
+#pragma unroll
+                for (int t = 0; t < 9; ++t) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, MB * NB, 0);  // MFMA
+                    __builtin_amdgcn_sched_group_barrier(0x100, MB + NB, 0);  // LDS reads
+                }
+            };
             load_group(0, a0, b0);
-            for (int g = 0; g < ncgw; g += 2) {
-                load_group(min(g + 1, ncgw - 1), a1, b1);
+            for (int g = 0; g + 1 < ncgw; g += 2) {
                 __builtin_amdgcn_sched_barrier(0);
+                load_group(g + 1, a1, b1);
                 mfma_group(a0, b0);
+                interleave();
                 __builtin_amdgcn_sched_barrier(0);
                 load_group(min(g + 2, ncgw - 1), a0, b0);
-                __builtin_amdgcn_sched_barrier(0);
-                if (g + 1 < ncgw) mfma_group(a1, b1);
+                mfma_group(a1, b1);
+                interleave();
                 __builtin_amdgcn_sched_barrier(0);
             }
+            if (ncgw & 1) mfma_group(a0, b0);
         } else if constexpr (TAPS == TAPS_1x1) {
-            // Same ping-pong, a group being four K-steps (channel groups).
+            // Same ping-pong and interleave, a group being four K-steps (channel groups).  K-steps past
+            // the wave's share get a zero A operand instead of a branch.
             constexpr int G = 4;
             float a0[G][MB], b0[G][NB], a1[G][MB], b1[G][NB];
+            const int ngrp = (ncgw + G - 1) / G;
             auto load_group = [&](int g0, float(&a)[G][MB], float(&b)[G][NB]) {
 #pragma unroll
                 for (int t = 0; t < G; ++t) {
-                    const int g = min(g0 + t, ncgw - 1);
+                    const bool live = g0 + t < ncgw;
+                    const int g = live ? g0 + t : ncgw - 1;
 #pragma unroll
-                    for (int mb = 0; mb < MB; ++mb) a[t][mb] = sw[mb][g * 64];
+                    for (int mb = 0; mb < MB; ++mb) {
+                        const float av = sw[mb][g * 64];
+                        a[t][mb] = live ? av : 0.0f;
+                    }
 #pragma unroll
                     for (int nb = 0; nb < NB; ++nb) b[t][nb] = sin[g * KC * p.CS + boff[nb]];
                 }
             };
-            auto mfma_group = [&](int g0, const float(&a)[G][MB], const float(&b)[G][NB]) {
+            auto mfma_group = [&](const float(&a)[G][MB], const float(&b)[G][NB]) {
+#pragma unroll
+                for (int t = 0; t < G; ++t)
+#pragma unroll
+                    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                        for (int nb = 0; nb < NB; ++nb) acc[mb][nb] = M::run(a[t][mb], b[t][nb], acc[mb][nb]);
+            };
+            auto interleave = [&]() {
 #pragma unroll
                 for (int t = 0; t < G; ++t) {
-                    if (g0 + t < ncgw) {
-#pragma unroll
-                        for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-                            for (int nb = 0; nb < NB; ++nb) acc[mb][nb] = M::run(a[t][mb], b[t][nb], acc[mb][nb]);
-                    }
+                    __builtin_amdgcn_sched_group_barrier(0x008, MB * NB, 0);  // MFMA
+                    __builtin_amdgcn_sched_group_barrier(0x100, MB + NB, 0);  // LDS reads
                 }
             };
             load_group(0, a0, b0);
-            for (int g0 = 0; g0 < ncgw; g0 += 2 * G) {
-                load_group(min(g0 + G, ncgw - 1), a1, b1);
+            for (int gi = 0; gi + 1 < ngrp; gi += 2) {
                 __builtin_amdgcn_sched_barrier(0);
-                mfma_group(g0, a0, b0);
+                load_group((gi + 1) * G, a1, b1);
+                mfma_group(a0, b0);
+                interleave();
                 __builtin_amdgcn_sched_barrier(0);
-                load_group(min(g0 + 2 * G, ncgw - 1), a0, b0);
-                __builtin_amdgcn_sched_barrier(0);
-                mfma_group(g0 + G, a1, b1);
+                load_group(min(gi + 2, ngrp - 1) * G, a0, b0);
+                mfma_group(a1, b1);
+                interleave();
                 __builtin_amdgcn_sched_barrier(0);
             }
+            if (ngrp & 1) mfma_group(a0, b0);
         } else {
             // Any filter size / dilation: taps walked at run time.
             for (int g = 0; g < ncgw; ++g) {
@@ -361,22 +403,23 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
             }
         }
     }
-
     // Epilogue.  `each_output(sink)` walks this thread's share of the workgroup's output tile and
     // hands (channel, pixel offset in the image, accumulated value) to the sink.
     if (p.WK > 1) {
         // Split-K across waves: park every wave's partial tile in LDS
         // ([wk][channel][pixel lane]); the walk below adds the WK slices in index order.
         __syncthreads();
+        if (!loader) {
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb) {
+            for (int mb = 0; mb < MB; ++mb) {
 #pragma unroll
-            for (int nb = 0; nb < NB; ++nb) {
-                const int pl = (wn * NB + nb) * MF + M::col(lane);
+                for (int nb = 0; nb < NB; ++nb) {
+                    const int pl = (wn * NB + nb) * MF + M::col(lane);
 #pragma unroll
-                for (int v = 0; v < NACC; ++v) {
-                    const int ml = (wm * MB + mb) * MF + M::row(v, lane);
-                    lds[(wk * MT + ml) * PT + pl] = acc[mb][nb][v];
+                    for (int v = 0; v < NACC; ++v) {
+                        const int ml = (wm * MB + mb) * MF + M::row(v, lane);
+                        lds[(wk * MT + ml) * PT + pl] = acc[mb][nb][v];
+                    }
                 }
             }
         }
@@ -392,7 +435,7 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
                 const int jy = fdiv(j, p.fd_tw);
                 const int jx = j - jy * p.TW;
                 const int oy = oy0 + jy, ox = ox0 + jx;
-                const bool pix_ok = jy < p.TH && oy < p.Ho && ox < p.Wo;
+                const bool pix_ok = jy < p.TH && oy < p.Ho && ox < p.Wo && !loader;
                 const int pp = oy * p.Wo + ox;
 #pragma unroll
                 for (int mb = 0; mb < MB; ++mb) {

@@ -248,7 +248,7 @@ int tdc_conv_forward_strided(tdc_conv_plan *plan, const float *d_in, int64_t in_
     kp.TW = g.TW; kp.TH = g.TH; kp.ntx = g.ntx;
     kp.WM = plan->tile.wm; kp.WN = plan->tile.wn; kp.WK = plan->tile.wk;
     kp.CCH = plan->tile.cch; kp.nchunks = g.nchunks; kp.CPW = g.cpw;
-    kp.KS = g.ks; kp.cps = g.cps;
+    kp.KS = g.ks; kp.cps = g.cps; kp.WL = plan->tile.wl;
     kp.RS = g.RS; kp.CS = g.CS; kp.nrows = g.nrows;
     // 16-byte copy elements need every image of the batch 16-byte aligned; otherwise 4-byte elements.
     const bool aligned = reinterpret_cast<uintptr_t>(d_in) % 16 == 0 && kp.in_bstride % 4 == 0;

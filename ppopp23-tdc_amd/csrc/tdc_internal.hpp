@@ -102,6 +102,7 @@ struct ConvKParams {
     int WM, WN, WK;
     int CCH, nchunks, CPW;
     int KS, cps;               // slices across workgroups, passes per slice
+    int WL;                    // loader waves (the last WL of the workgroup)
     int RS, CS, VW, nrows;
     int in_stage_floats, wslab_floats, stage_floats, nstage;
     int relu;

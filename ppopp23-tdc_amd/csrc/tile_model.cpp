@@ -72,8 +72,9 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
     if (t.wm < 1 || t.wn < 1 || t.wk < 1) return fail("tile.wm / wn / wk must be >= 1");
     g = Geometry();
     g.max_waves_kernel = (t.mb == 2 && t.nb == 2) ? 8 : 16;
-    if ((long long)t.wm * t.wn * t.wk > g.max_waves_kernel) return fail("too many waves per workgroup for this tile");
-    g.waves = t.wm * t.wn * t.wk;
+    if (t.wl < 0 || t.wl > 8) return fail("tile.wl must be in [0, 8]");
+    if ((long long)t.wm * t.wn * t.wk + t.wl > g.max_waves_kernel) return fail("too many waves per workgroup for this tile");
+    g.waves = t.wm * t.wn * t.wk + t.wl;
     g.threads = g.waves * 64;
     const bool flat = (d.KH == 1 && d.KW == 1 && d.stride == 1 && d.pad == 0);
     g.He = flat ? 1 : d.H;
@@ -173,21 +174,22 @@ namespace {
 // of num_sm / num_threads / the (a, b, c) weights / the keep-ratio in the reference's model
 // (2080Ti-evaluation/TDC-LAYERS-MODELING/model.py:265-266,278).
 struct ModelConst {
-    double launch_us = 1.7;           // device time of an empty kernel in a back-to-back stream
-    double setup_clk = 1530;          // kernel arguments and index arithmetic before the first copy is issued
-    double copy_latency_clk = 1734;   // first byte of a global->LDS copy (L2 / memory-side cache)
-    double copy_bytes_per_clk = 30.2;   // sustained global->LDS rate of one CU
-    double l2_bytes_per_clk = 8640;   // whole-chip L2->CU rate when every CU copies at once
-    double lds_bytes_per_clk = 38.8;   // LDS traffic of the split-K reduction
-    double sync_clk = 127.5;            // one workgroup barrier
-    double store_bytes_per_clk = 5.2;  // per CU, short runs per channel
-    double kstep_issue_clk = 4.35;       // vector-ALU / LDS-issue cycles per operand read, not hidden under MFMAs
-    double pass_overhead_clk = 424;   // per wave and pass: copy issue, pointer set-up, pipeline fill
-    double wave_setup_clk = 2.2;      // prologue cycles added per extra wave sharing a SIMD
-    double ksplit_clk = 4500;         // split across workgroups: device-scope fences and the ticket round trip
+    double launch_us = 1.474;           // device time of an empty kernel in a back-to-back stream
+    double setup_clk = 1399;          // kernel arguments and index arithmetic before the first copy is issued
+    double copy_latency_clk = 1083;   // first byte of a global->LDS copy (L2 / memory-side cache)
+    double copy_bytes_per_clk = 33.65;   // sustained global->LDS rate of one CU
+    double l2_bytes_per_clk = 7865;   // whole-chip L2->CU rate when every CU copies at once
+    double lds_bytes_per_clk = 15.13;   // LDS traffic of the split-K reduction
+    double sync_clk = 224.8;            // one workgroup barrier
+    double store_bytes_per_clk = 2.265;  // per CU, short runs per channel
+    double kstep_issue_clk = 1.764;      // vector-ALU / LDS-issue cycles per operand read, not hidden under MFMAs
+    double pass_overhead_clk = 567.4;   // per wave and pass: copy issue, pointer set-up, pipeline fill
+    double wave_setup_clk = 212.8;      // prologue cycles added per extra wave sharing a SIMD
+    double ksplit_clk = 3611;         // split across workgroups: write-through, ticket round trip, read-back
+    double copy_issue_clk = 118.2;      // a wave is held this long by every global->LDS copy instruction it issues
 };
 ModelConst MC;
-constexpr int kNumModelConst = 12;
+constexpr int kNumModelConst = 13;
 
 double *mc_field(int i) {
     switch (i) {
@@ -203,6 +205,7 @@ double *mc_field(int i) {
         case 9: return &MC.pass_overhead_clk;
         case 10: return &MC.wave_setup_clk;
         case 11: return &MC.ksplit_clk;
+        case 12: return &MC.copy_issue_clk;
         default: return nullptr;
     }
 }
@@ -264,20 +267,38 @@ bool model_evaluate(const tdc_conv_desc &d, const tdc_tile &t, tdc_tile_info &in
     const double red_bytes = t.wk > 1 ? (double)t.wk * g.MT * g.PT * 4.0 * 2.0 : 0.0;
     const double out_bytes = (double)g.MT * g.PT * 4.0;
 
+    // Copy instructions of one pass (64 elements each) and how long issuing them holds a wave: the first
+    // pass is dealt to every wave; later ones to the loader waves if there are any, else to everybody.
+    const int ncomp = t.wm * t.wn * t.wk;
+    const double n_instr = (double)g.in_stage_floats / (64.0 * g.VW) + std::ceil(g.wslab_floats / 256.0);
+    const double issue_first = std::ceil(n_instr / g.waves) * MC.copy_issue_clk;
+    const double issue_steady = std::ceil(n_instr / (t.wl ? t.wl : g.waves)) * MC.copy_issue_clk;
+    const int comp_waves_per_simd = ceil_div(ncomp, m.simds_per_cu);
+
     auto wg_time = [&](int r, long long concurrent_wgs) {
         // r workgroups share one CU: matrix time and the issue cycles of the operand reads add up per
         // SIMD; copies share the CU's fill rate and, chip-wide, the L2.
-        const double waves_simd = (double)wg_waves_per_simd * r;
-        const double per_wave = mfma_pass + ksteps_pass * (t.mb + t.nb) * MC.kstep_issue_clk + MC.pass_overhead_clk;
-        const double compute = per_wave * waves_simd + MC.sync_clk;
+        const double waves_simd = (double)comp_waves_per_simd * r;
+        // A wave alone on its SIMD stalls on every operand read and while it issues copies; with several
+        // waves per SIMD those gaps are filled by the others until the matrix pipe itself is the limit.
+        const double stall = ksteps_pass * (t.mb + t.nb) * MC.kstep_issue_clk + MC.pass_overhead_clk;
+        const double alone = mfma_pass + stall;
+        const double pipe = mfma_pass * waves_simd + MC.pass_overhead_clk;
+        const double compute = std::max(alone, pipe) + MC.sync_clk;
+        const double compute_issuing = std::max(alone + issue_steady, pipe) + MC.sync_clk;
         const double chip_share =
             MC.l2_bytes_per_clk / std::max<double>(1.0, (double)std::min<long long>(concurrent_wgs, m.cus));
         const double rate = std::min(MC.copy_bytes_per_clk, chip_share);
         const double copy = copy_bytes_pass * r / rate;
         // First pass is exposed; afterwards the copy of pass i+1 runs under the MFMAs of pass i.
-        double clk = MC.setup_clk + MC.wave_setup_clk * (waves_simd - 1.0) + MC.copy_latency_clk + copy;
+        double clk = MC.setup_clk + MC.wave_setup_clk * ((double)wg_waves_per_simd * r - 1.0) + issue_first +
+                     MC.copy_latency_clk + copy;
         clk += compute;  // last pass: nothing left to hide
-        if (g.cps > 1) clk += (g.cps - 1) * std::max(compute, copy + MC.copy_latency_clk);
+        if (g.cps > 1) {
+            const double pass = t.wl ? std::max(compute, std::max(issue_steady, copy) + MC.copy_latency_clk)
+                                     : std::max(compute_issuing, copy + MC.copy_latency_clk);
+            clk += (g.cps - 1) * pass;
+        }
         clk += red_bytes * r / MC.lds_bytes_per_clk + out_bytes * r / MC.store_bytes_per_clk +
                (t.wk > 1 ? 2.0 * MC.sync_clk : 0.0);
         // Split across workgroups: the partial tile goes to the workspace (the store above), and the
@@ -350,13 +371,15 @@ std::vector<tdc_tile> model_enumerate(const tdc_conv_desc &d) {
                             const long long max_wgs = 4LL * machine().cus;
                             for (int tw : tws)
                                 for (int cch : cchs)
-                                    for (int ks : {1, 2, 4, 8}) {
-                                        tdc_tile t{mf, mb, nb, wm, wn, wk, cch, tw, ks};
-                                        Geometry g;
-                                        if (!make_geometry(d, t, g, nullptr)) continue;
-                                        if (ks > 1 && (long long)g.grid_x * g.grid_y * g.grid_z > max_wgs) continue;
-                                        out.push_back(t);
-                                    }
+                                    for (int ks : {1, 2, 4, 8})
+                                        for (int wl : {0, 1, 2, 4}) {
+                                            tdc_tile t{mf, mb, nb, wm, wn, wk, cch, tw, ks, wl};
+                                            Geometry g;
+                                            if (!make_geometry(d, t, g, nullptr)) continue;
+                                            if (ks > 1 && (long long)g.grid_x * g.grid_y * g.grid_z > max_wgs) continue;
+                                            if (wl > 0 && g.cps < 2) continue;  // loaders only work from the second pass on
+                                            out.push_back(t);
+                                        }
                         }
     }
     return out;

@@ -26,7 +26,7 @@ def load(paths):
         for r in csv.DictReader(open(path)):
             key = tuple(int(r[k]) for k in ("C", "N", "H", "W", "K", "stride"))
             tile = _lib.Tile(*[int(r[k]) for k in ("mf", "mb", "nb", "wm", "wn", "wk", "cch", "tw")],
-                             ks=int(r.get("ks") or 1))
+                             ks=int(r.get("ks") or 1), wl=int(r.get("wl") or 0))
             layers[key].append((tile, float(r["time_us"])))
     return layers
 
@@ -51,7 +51,7 @@ def fit(layers, rounds=6, seed=0):
     cur = _lib.model_get_constants()
     best = score(layers)
     print("start: loss %.2f%%  log-err %.3f" % (100 * best[0], best[1]), flush=True)
-    obj = lambda s: s[0] + 0.05 * s[1]
+    obj = lambda s: s[0] + 0.3 * s[1]
     for rnd in range(rounds):
         order = list(range(len(cur)))
         rng.shuffle(order)

@@ -1,7 +1,7 @@
 """Measured tile sweep and model-loss report.
 
 For every shape, time every launchable tile through the C ABI, record
-``C,N,H,W,K,stride,mf,mb,nb,wm,wn,wk,cch,tw,ks,pred_us,time_us`` rows, and report how
+``C,N,H,W,K,stride,mf,mb,nb,wm,wn,wk,cch,tw,ks,wl,pred_us,time_us`` rows, and report how
 much slower the analytic model's pick is than the measured best
 (``loss = t(model pick) / t(best) - 1``).  This is the gfx950 counterpart of the
 reference's brute-force occupancy/timing sweep
@@ -35,9 +35,12 @@ def time_plan(plan, x, out, iters=50, warmup=5, reps=5):
     return samples[len(samples) // 2]
 
 
-def sweep_shape(C, N, H, W, K=3, stride=1, pad=1, batch=1, iters=20, every=1, log=None):
+def sweep_shape(C, N, H, W, K=3, stride=1, pad=1, batch=1, iters=20, every=1, log=None, max_tiles=0, offset=0):
     desc = _lib.conv_desc(batch, C, N, H, W, K, K, stride, pad)
-    tiles = _lib.model_enumerate(desc)[::every]
+    tiles = _lib.model_enumerate(desc)
+    if max_tiles and len(tiles) > max_tiles * every:
+        every = -(-len(tiles) // max_tiles)
+    tiles = tiles[offset % every::every]
     pick = _lib.model_select(desc)
     g = torch.Generator().manual_seed(H * 1_000_000 + C * 1_000 + N)
     x = (torch.rand(batch, C, H, W, generator=g) * 2 - 1).cuda()
@@ -57,7 +60,7 @@ def sweep_shape(C, N, H, W, K=3, stride=1, pad=1, batch=1, iters=20, every=1, lo
             log.write(",".join(f"{v:.3f}" if isinstance(v, float) else str(v) for v in row) + "\n")
             log.flush()
     best = min(rows, key=lambda r: r[-1])
-    mine = next(r for r in rows if r[6:15] == pick.tile.astuple())
+    mine = next(r for r in rows if r[6:16] == pick.tile.astuple())
     return {"shape": (C, N, H, W, K, stride), "best": best, "model": mine, "loss": mine[-1] / best[-1] - 1,
             "roof_us": pick.roof_us, "n": len(rows)}
 
@@ -67,23 +70,25 @@ def main(argv=None):
     ap.add_argument("--out", default=None, help="CSV of every (shape, tile) timing")
     ap.add_argument("--iters", type=int, default=50)
     ap.add_argument("--every", type=int, default=1, help="time every k-th candidate only")
+    ap.add_argument("--max-tiles", type=int, default=0, help="thin the candidates of a shape to about this many")
+    ap.add_argument("--offset", type=int, default=0, help="first candidate of the thinned list")
     ap.add_argument("--hw", type=int, nargs="*", default=list(SWEEP_HW))
     a = ap.parse_args(argv)
     if not torch.cuda.is_available():
         sys.exit("tdc_amd.sweep needs a GPU")
     log = open(a.out, "w") if a.out else None
     if log:
-        log.write("C,N,H,W,K,stride,mf,mb,nb,wm,wn,wk,cch,tw,ks,pred_us,time_us\n")
+        log.write("C,N,H,W,K,stride,mf,mb,nb,wm,wn,wk,cch,tw,ks,wl,pred_us,time_us\n")
     total = 0.0
     n = 0
     t0 = time.time()
     for hw in a.hw:
         for r1, r2 in SWEEP_RANKS:
-            r = sweep_shape(r1, r2, hw, hw, iters=a.iters, every=a.every, log=log)
+            r = sweep_shape(r1, r2, hw, hw, iters=a.iters, every=a.every, log=log, max_tiles=a.max_tiles, offset=a.offset)
             total += r["loss"]
             n += 1
             print("shape %s roof %.3f us | best %s %.2f us | model %s %.2f us (pred %.2f) | loss %+.1f%% | %d tiles | %.0fs"
-                  % (r["shape"], r["roof_us"], r["best"][6:15], r["best"][-1], r["model"][6:15], r["model"][-1],
+                  % (r["shape"], r["roof_us"], r["best"][6:16], r["best"][-1], r["model"][6:16], r["model"][-1],
                      r["model"][-2], 100 * r["loss"], r["n"], time.time() - t0), flush=True)
     print("average loss %.1f%% over %d shapes" % (100 * total / max(n, 1), n))
 

@@ -36,10 +36,10 @@ def test_version_and_error_string():
 
 def test_struct_layouts_match_the_header():
     assert ctypes.sizeof(_lib.ConvDesc) == 12 * 4
-    assert ctypes.sizeof(_lib.Tile) == 9 * 4
+    assert ctypes.sizeof(_lib.Tile) == 10 * 4
     assert ctypes.sizeof(_lib.TKConvDesc) == 13 * 4
-    # tile (9 ints) + 10 ints, padded to 8-byte alignment, + 5 doubles
-    assert ctypes.sizeof(_lib.TileInfo) == 9 * 4 + 10 * 4 + 4 + 5 * 8
+    # tile (10 ints) + 10 ints + 5 doubles
+    assert ctypes.sizeof(_lib.TileInfo) == 10 * 4 + 10 * 4 + 5 * 8
     assert _lib.TileInfo.flops.offset == 80
 
 

@@ -27,7 +27,7 @@ def test_every_candidate_is_launchable_and_covers_the_output(hw, r1, r2):
         assert i.grid_x == ntx * nty and ntx * t.tw >= hw and nty * i.th >= hw      # tiles cover the image
         assert i.grid_y * t.mf * t.mb * t.wm >= r2                                   # ... and all channels
         assert i.nchunks * t.cch >= r1 and t.cch % ((2 if t.mf == 32 else 4) * t.wk) == 0
-        assert i.block_threads == 64 * t.wm * t.wn * t.wk <= 1024
+        assert i.block_threads == 64 * (t.wm * t.wn * t.wk + t.wl) <= 1024      # computing waves + loader waves
         assert 0 < i.lds_bytes <= LDS_BYTES
         assert i.wg_per_cu >= 1 and i.pred_us > 0
 
