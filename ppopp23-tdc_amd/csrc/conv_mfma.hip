@@ -241,7 +241,6 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
             issue_pass(p, in_rsrc, w_rsrc, stage, pre, true, lane16, chunk, iy0, ix0a, w_byte0, dw, dn, lane);
     };
     issue(chunk0, true);
-
     // Per-lane LDS offset (floats) of tap (0,0) for each pixel block, channel sub-index included.
     int boff[NB];
 #pragma unroll

@@ -38,6 +38,7 @@ class Net:
         self.input_id = 0
         self.output_id = None
         self._keep = []
+        self.conv_shapes = []   # (C, N, H, W, K, stride, pad) of every convolution launched per forward, in order
 
     def tensor(self, C, H, W):
         out = c_int32()
@@ -52,6 +53,8 @@ class Net:
     def conv(self, x, weight, bias=None, stride=1, pad=0, residual=-1, relu=False, dst=-1):
         w, b = _h(weight), _h(bias)
         out = c_int32()
+        _, C, H, W = self.shape(x)
+        self.conv_shapes.append((C, w.shape[0], H, W, w.shape[2], stride, pad))
         check(lib().tdc_net_conv(self._h, x, w.shape[0], w.shape[2], w.shape[3], stride, pad, _p(w), _p(b), residual,
                                  int(relu), dst, byref(out)))
         return out.value
@@ -59,6 +62,11 @@ class Net:
     def tkconv(self, x, first, core, last, bias=None, stride=1, pad=0, residual=-1, relu=False, dst=-1):
         f, c, l, b = _h(first), _h(core), _h(last), _h(bias)
         out = c_int32()
+        _, C, H, W = self.shape(x)
+        K = c.shape[2]
+        Ho, Wo = (H + 2 * pad - K) // stride + 1, (W + 2 * pad - K) // stride + 1
+        self.conv_shapes += [(C, f.shape[0], H, W, 1, 1, 0), (f.shape[0], c.shape[0], H, W, K, stride, pad),
+                             (c.shape[0], l.shape[0], Ho, Wo, 1, 1, 0)]
         check(lib().tdc_net_tkconv(self._h, x, f.shape[0], c.shape[0], l.shape[0], c.shape[2], stride, pad, _p(f), _p(c),
                                    _p(l), _p(b), residual, int(relu), dst, byref(out)))
         return out.value

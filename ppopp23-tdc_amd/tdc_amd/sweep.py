@@ -72,6 +72,8 @@ def main(argv=None):
     ap.add_argument("--every", type=int, default=1, help="time every k-th candidate only")
     ap.add_argument("--max-tiles", type=int, default=0, help="thin the candidates of a shape to about this many")
     ap.add_argument("--offset", type=int, default=0, help="first candidate of the thinned list")
+    ap.add_argument("--net", choices=("resnet18", "densenet121"), default=None,
+                    help="sweep the distinct convolution shapes of a whole network instead of the core-conv layers")
     ap.add_argument("--hw", type=int, nargs="*", default=list(SWEEP_HW))
     a = ap.parse_args(argv)
     if not torch.cuda.is_available():
@@ -82,14 +84,24 @@ def main(argv=None):
     total = 0.0
     n = 0
     t0 = time.time()
-    for hw in a.hw:
-        for r1, r2 in SWEEP_RANKS:
-            r = sweep_shape(r1, r2, hw, hw, iters=a.iters, every=a.every, log=log, max_tiles=a.max_tiles, offset=a.offset)
-            total += r["loss"]
-            n += 1
-            print("shape %s roof %.3f us | best %s %.2f us | model %s %.2f us (pred %.2f) | loss %+.1f%% | %d tiles | %.0fs"
-                  % (r["shape"], r["roof_us"], r["best"][6:16], r["best"][-1], r["model"][6:16], r["model"][-1],
-                     r["model"][-2], 100 * r["loss"], r["n"], time.time() - t0), flush=True)
+    if a.net:
+        from . import nets
+        if a.net == "resnet18":
+            net = nets.build_tucker_resnet18(nets.resnet18_params())
+        else:
+            net = nets.build_tucker_densenet121(nets.densenet121_params())
+        shapes = sorted(set(net.conv_shapes))
+        net.close()
+    else:
+        shapes = [(r1, r2, hw, hw, 3, 1, 1) for hw in a.hw for r1, r2 in SWEEP_RANKS]
+    for (C, N, H, W, K, stride, pad) in shapes:
+        r = sweep_shape(C, N, H, W, K=K, stride=stride, pad=pad, iters=a.iters, every=a.every, log=log,
+                        max_tiles=a.max_tiles, offset=a.offset)
+        total += r["loss"]
+        n += 1
+        print("shape %s roof %.3f us | best %s %.2f us | model %s %.2f us (pred %.2f) | loss %+.1f%% | %d tiles | %.0fs"
+              % (r["shape"], r["roof_us"], r["best"][6:16], r["best"][-1], r["model"][6:16], r["model"][-1],
+                 r["model"][-2], 100 * r["loss"], r["n"], time.time() - t0), flush=True)
     print("average loss %.1f%% over %d shapes" % (100 * total / max(n, 1), n))
 
 
