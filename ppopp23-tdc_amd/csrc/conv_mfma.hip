@@ -174,7 +174,8 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
                  "s"(p.ntx), "s"(p.stride), "s"(p.pad), "s"(p.VW), "s"(p.in_stage_floats), "s"(p.wslab_floats),
                  "s"(p.stage_floats), "s"(p.nstage), "s"(p.nchunks), "s"(p.fd_csv.m), "s"(p.fd_csv.d),
                  "s"(p.fd_rsv.m), "s"(p.fd_rsv.d), "s"(p.fd_ntx.m), "s"(p.fd_wk.m), "s"(p.fd_wn.m), "s"(p.WK),
-                 "s"(p.WN), "s"(p.in_bstride), "s"(p.wpk_bytes), "s"(p.KS), "s"(p.cps), "s"(p.fd_ks.m), "s"(p.WL));
+                 "s"(p.WN), "s"(p.in_bstride), "s"(p.wpk_bytes), "s"(p.KS), "s"(p.cps), "s"(p.fd_ks.m), "s"(p.WL), "s"(p.xcd_chunk), "s"(p.n_wg), "s"(p.fd_g1.m),
+                 "s"(p.fd_g1.d), "s"(p.fd_g2.m), "s"(p.fd_g2.d), "s"(p.channel_major));
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -195,14 +196,28 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
 
     const int PT = MF * NB * p.WN;  // pixel lanes of the workgroup (>= TH*TW)
     const int MT = MF * MB * p.WM;
-    const int tile_y = fdiv(blockIdx.x, p.fd_ntx);
-    const int tile_x = blockIdx.x - tile_y * p.ntx;
+    // Workgroups are handed to the eight compute dies (XCDs, each with its own L2) round-robin by launch
+    // index.  The launch is one-dimensional and the index is re-read as (die, slot), so that each die
+    // works on a contiguous run of the logical order; that order has either the channel tiles of one
+    // pixel tile adjacent (a die then reads its own part of the input, and all the weights) or the
+    // pixel tiles of one channel tile adjacent (a die reads few weights, and all the input) — whichever
+    // the host found cheaper for this layer.
+    const int logical = (int)(blockIdx.x & 7u) * p.xcd_chunk + (int)(blockIdx.x >> 3);
+    if (logical >= p.n_wg) return;
+    const int q1 = fdiv(logical, p.fd_g1);
+    const int r1 = logical - q1 * p.fd_g1.d;
+    const int bz = fdiv(q1, p.fd_g2);
+    const int r2 = q1 - bz * p.fd_g2.d;
+    const int bx = p.channel_major ? r1 : r2;  // pixel tile
+    const int by = p.channel_major ? r2 : r1;  // channel tile
+    const int tile_y = fdiv(bx, p.fd_ntx);
+    const int tile_x = bx - tile_y * p.ntx;
     const int oy0 = tile_y * p.TH;
     const int ox0 = tile_x * p.TW;
-    const int m0 = blockIdx.y * MT;
-    // blockIdx.z = image * KS + slice of the input-channel passes
-    const int img = fdiv(blockIdx.z, p.fd_ks);
-    const int ks = blockIdx.z - img * p.KS;
+    const int m0 = by * MT;
+    // bz = image * KS + slice of the input-channel passes
+    const int img = fdiv(bz, p.fd_ks);
+    const int ks = bz - img * p.KS;
     const int chunk0 = ks * p.cps;
     const int chunk1 = min(chunk0 + p.cps, p.nchunks);
     const float *__restrict__ in = p.in + (long long)img * p.in_bstride;
@@ -220,7 +235,7 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
     const int ix0a = (p.VW == 4) ? ((ix0 >> 2) << 2) : ix0;
     // Packed weights: [channel tile][pass][...]; one pass of this channel tile is contiguous.
     const unsigned w_pass_bytes = (unsigned)p.wslab_floats * 4u;
-    const unsigned w_byte_base = (unsigned)blockIdx.y * (unsigned)p.nchunks * w_pass_bytes;
+    const unsigned w_byte_base = (unsigned)by * (unsigned)p.nchunks * w_pass_bytes;
 
     // Offsets of this lane's elements in its wave's first MAXPRE input blocks (pass 0), for the steady dealing.
     int pre[MAXPRE];
@@ -484,7 +499,7 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
     // to the workspace is itself a device-scope (relaxed) atomic: the stores write through, the loads
     // bypass the die-local L2, and "my stores are done" is the plain wait below.
     const long long NP = (long long)p.N * p.P;
-    float *wsz = p.ws + (long long)blockIdx.z * NP;
+    float *wsz = p.ws + (long long)bz * NP;
     each_output(
         [&](int n, int pp, float val) {
             __hip_atomic_store(wsz + (long long)n * p.P + pp, val, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -492,7 +507,7 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
         true);
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
-    unsigned *ticket = p.ctr + ((unsigned)img * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
+    unsigned *ticket = p.ctr + ((unsigned)img * p.grid_y + by) * p.grid_x + bx;
     if (tid == 0) {
         const unsigned drawn = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         reinterpret_cast<unsigned *>(lds)[0] = drawn;
@@ -573,7 +588,7 @@ int prepare_conv_kernel(const void *fn, const Geometry &g) {
 
 int launch_conv(const void *fn, const Geometry &g, const ConvKParams &kp, void *stream) {
     if (!fn) return (int)hipErrorInvalidValue;
-    dim3 grid(g.grid_x, g.grid_y, g.grid_z), block(g.threads);
+    dim3 grid(8 * kp.xcd_chunk), block(g.threads);
     hipLaunchKernelGGL(reinterpret_cast<kernel_fn>(const_cast<void *>(fn)), grid, block,
                        (size_t)g.lds_bytes, (hipStream_t)stream, kp);
     return (int)hipGetLastError();

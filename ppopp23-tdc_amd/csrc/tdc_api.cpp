@@ -264,6 +264,12 @@ int tdc_conv_forward_strided(tdc_conv_plan *plan, const float *d_in, int64_t in_
     kp.fd_wk = make_fastdiv(plan->tile.wk);
     kp.fd_wn = make_fastdiv(plan->tile.wn);
     kp.fd_ks = make_fastdiv(g.ks);
+    kp.grid_x = g.grid_x; kp.grid_y = g.grid_y;
+    kp.n_wg = g.grid_x * g.grid_y * g.grid_z;
+    kp.xcd_chunk = (kp.n_wg + 7) / 8;
+    kp.channel_major = g.channel_major;
+    kp.fd_g1 = make_fastdiv(g.channel_major ? g.grid_x : g.grid_y);
+    kp.fd_g2 = make_fastdiv(g.channel_major ? g.grid_y : g.grid_x);
     kp.wpk_bytes = (unsigned)(packed_weight_floats(g) * sizeof(float));
     int he = launch_conv(plan->kernel, g, kp, stream);
     if (he) return hip_fail("kernel launch", he);

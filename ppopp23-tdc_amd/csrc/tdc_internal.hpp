@@ -54,6 +54,7 @@ struct Geometry {
     int nstage = 1;
     int lds_bytes = 0;
     int max_waves_kernel = 0;        // launch bound of the instantiated kernel
+    int channel_major = 0;           // which logical workgroup order costs fewer L2 fills (see conv_mfma.hip)
 };
 
 // Returns false (and a reason) when the tile cannot be launched for this shape.
@@ -103,6 +104,11 @@ struct ConvKParams {
     int CCH, nchunks, CPW;
     int KS, cps;               // slices across workgroups, passes per slice
     int WL;                    // loader waves (the last WL of the workgroup)
+    int grid_x, grid_y;        // pixel tiles, channel tiles
+    int n_wg;                  // grid_x * grid_y * batch * KS
+    int xcd_chunk;             // ceil(n_wg / 8): logical workgroups per compute die
+    int channel_major;         // logical order: 1 = pixel tile fastest, 0 = channel tile fastest
+    FastDiv fd_g1, fd_g2;      // the fastest / second extent of the logical order
     int RS, CS, VW, nrows;
     int in_stage_floats, wslab_floats, stage_floats, nstage;
     int relu;

@@ -139,6 +139,18 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
     g.lds_bytes = (int)lds;
     if (const char *e = std::getenv("TDC_EXPERIMENT_MIN_LDS")) g.lds_bytes = std::max(g.lds_bytes, std::atoi(e));
     if ((long long)g.grid_y * g.nchunks * g.wslab_floats * 4 >= (1LL << 31)) return fail("packed weights exceed 2 GiB");
+    // (the kernel decodes a one-dimensional launch index with 32-bit multiply-high divisions)
+    const long long n_wg = (long long)g.grid_x * g.grid_y * g.grid_z;
+    if (n_wg + 8 >= (1LL << 28) || n_wg * std::max(g.grid_x, g.grid_y) >= (1LL << 32)) return fail("grid too large");
+    // Bytes the eight die-private L2s fill in total, for the two logical workgroup orders: with the channel
+    // tiles of a pixel tile adjacent a die reads its share of the input and every weight; with the pixel tiles
+    // of a channel tile adjacent it reads every input pixel of min(channel tiles, 8) ... and its own weights.
+    const double in_bytes = 4.0 * d.C * d.H * d.W, w_bytes = 4.0 * d.N * d.C * g.taps;
+    const double dies = (double)std::min<long long>(8, n_wg);
+    const double pixel_major = in_bytes + dies * w_bytes;
+    const double channel_major = std::min<double>(g.grid_y, dies) * in_bytes + std::max(1.0, dies / g.grid_y) * w_bytes;
+    g.channel_major = channel_major < pixel_major ? 1 : 0;
+    if (const char *e = std::getenv("TDC_EXPERIMENT_XCD_ORDER")) g.channel_major = std::atoi(e) != 0;
     return true;
 }
 
