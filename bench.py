@@ -240,6 +240,28 @@ def main():
             dres["kernels_per_forward"] = dnet.num_kernels
             dnet.close()
         out["tucker_densenet121"] = dres
+        # The four full Tucker blocks (configuration 3): 1x1 C->R1, 3x3 R1->R2, 1x1 R2->N as three launches in a graph.
+        # roof_us is the FUSED block's roofline: every flop, but input, output and weights moved once.
+        blocks = []
+        for (C, R1, R2, N, hw) in ref.BLOCKS:
+            bx, first, core, last = ref.make_block_case(C, R1, R2, N, hw)
+            bnet = nets.Net(1, C, hw, hw)
+            y = bnet.tkconv(0, first, core, last, pad=1)
+            bnet.finalize(y)
+            got = bnet(bx.cuda()).cpu()
+            want = ref.tkconv_torch(bx, first, core, last, pad=1)
+            berr = float((got - want).abs().max())
+            if not berr <= 1e-5 + 1e-4 * float(want.abs().max()):
+                sys.exit("bench.py: Tucker block parity check failed (max err %g)" % berr)
+            bnet.time_ms(iters=20)
+            us = min(bnet.time_ms(iters=200) for _ in range(3)) * 1e3
+            flops = 2.0 * hw * hw * (C * R1 + 9 * R1 * R2 + R2 * N)
+            nbytes = 4.0 * (hw * hw * (C + N) + C * R1 + 9 * R1 * R2 + R2 * N)
+            roof = max(nbytes / 8e6, flops / 157.3e6)
+            blocks.append({"C": C, "R1": R1, "R2": R2, "N": N, "H": hw, "us": round(us, 3), "roof_us": round(roof, 3),
+                           "frac": round(roof / us, 4), "kernels": bnet.num_kernels})
+            bnet.close()
+        out["tucker_blocks_b1"] = blocks
 
     # -- CPU baseline: the reference operator's CPU path (F.conv2d), same layers --
     if not a.no_cpu_baseline:

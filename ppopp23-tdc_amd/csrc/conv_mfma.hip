@@ -250,10 +250,15 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
     auto issue = [&](int chunk, bool everybody) {
         float *stage = lds + ((chunk - chunk0) & (p.nstage - 1)) * p.stage_floats;
         const int w_byte0 = (int)(w_byte_base + (unsigned)chunk * w_pass_bytes);
-        if (everybody)
+        if (everybody) {
             issue_pass(p, in_rsrc, w_rsrc, stage, pre, p.WL == 0, lane16, chunk, iy0, ix0a, w_byte0, wave, nwaves, lane);
-        else if (dw >= 0)
+        } else if (dw >= 0) {
+            // Copy issue competes for the SIMD with other waves' MFMA streams and loses by default (measured:
+            // ~330 cycles per copy instruction instead of ~115); it is short, so let it go first.
+            __builtin_amdgcn_s_setprio(3);
             issue_pass(p, in_rsrc, w_rsrc, stage, pre, true, lane16, chunk, iy0, ix0a, w_byte0, dw, dn, lane);
+            __builtin_amdgcn_s_setprio(0);
+        }
     };
     issue(chunk0, true);
     // Per-lane LDS offset (floats) of tap (0,0) for each pixel block, channel sub-index included.

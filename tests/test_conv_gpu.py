@@ -172,6 +172,20 @@ def test_split_across_workgroups(tile):
     assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2])
 
 
+@pytest.mark.parametrize("order", ["0", "1"])
+def test_both_logical_workgroup_orders(order, monkeypatch):
+    """The launch is one-dimensional and decoded in the kernel; both decode orders (channel tile fastest / pixel
+    tile fastest) must give the oracle's answer, also when the number of workgroups is not a multiple of 8."""
+    monkeypatch.setenv("TDC_EXPERIMENT_XCD_ORDER", order)
+    for (B, C, N, H, W, K, stride) in ((1, 12, 40, 13, 11, 3, 1), (3, 8, 24, 9, 10, 3, 2), (2, 20, 18, 7, 7, 1, 1)):
+        announce("order", order, B, C, N, H, W, K, stride)
+        x, w = case(7000 + C + N, B, C, N, H, W, K)
+        want = ref.conv2d_c(x.numpy(), w.numpy(), stride=stride, pad=K // 2)
+        tiles = tdc_amd.model_enumerate(tdc_amd.conv_desc(B, C, N, H, W, K, K, stride, K // 2))
+        for t in tiles[::max(1, len(tiles) // 40)]:
+            assert_close(run_conv(x, w, stride=stride, pad=K // 2, tile=t), want, f"order {order} {t}")
+
+
 def test_split_across_workgroups_rejects_empty_slices():
     with pytest.raises(tdc_amd.TdcError):   # 40 channels in passes of 8 = 5 passes: 4 slices take 2,2,1,0
         tdc_amd.model_evaluate(tdc_amd.conv_desc(1, 40, 16, 9, 9, 3, 3, 1, 1), tdc_amd.Tile(16, 1, 1, 1, 1, 1, 8, 8, ks=4))
