@@ -3,10 +3,16 @@
 (inference/TKConv.py:23-141), with the three ``F.conv2d`` calls of its forward
 (:90-95) replaced by the native 1x1 -> KxK core -> 1x1 kernels.
 
-Not carried over: initialisation from a dense weight (``dense_w``), which the
-reference does with ``tensorly.partial_tucker`` at construction time (:75-80) —
-it is init-time work off the inference path; pass already-decomposed kernels
-with ``load_kernels`` or a state dict instead.
+Initialisation from a dense weight (``dense_w``) is done by the reference with
+``tensorly.partial_tucker(dense_w, modes=[0, 1], rank=ranks, init='svd')`` at
+construction time (:75-80; tensorly 0.7.0 is pinned by the reference's README
+and is not installed here).  ``partial_tucker2`` below restates that published
+algorithm (higher-order orthogonal iteration on the two channel modes, started
+from the truncated SVDs of the unfoldings) on the host.  It is init-time work off
+the inference path.  Parity with tensorly is unpinned: the factors are determined
+only up to the sign/rotation conventions of the SVD routine; what the tests pin
+are the properties the mathematics fixes (orthonormal factors, exact
+reconstruction at full or true rank, never worse than the truncated HOSVD).
 """
 from __future__ import annotations
 
@@ -23,6 +29,47 @@ def _pair(v):
     return tuple(v) if isinstance(v, (tuple, list)) else (v, v)
 
 
+def partial_tucker2(weight, ranks, n_iter_max=100, tol=1e-4):
+    """Tucker-2 decomposition of an OIHW weight along its two channel modes.
+
+    Returns ``(core [R_out, R_in, KH, KW], last_factor [N, R_out], first_factor [C, R_in])`` with
+    ``weight ~= einsum('abhw,na,cb->nchw', core, last_factor, first_factor)`` and orthonormal factor columns.
+    ``ranks = [R_out, R_in]`` as in the reference's hp_dict tables."""
+    w = weight.detach().to(dtype=torch.float64, device="cpu")
+    N, C = w.shape[0], w.shape[1]
+    r_out, r_in = int(ranks[0]), int(ranks[1])
+    if not (1 <= r_out <= N and 1 <= r_in <= C):
+        raise ValueError(f"ranks {list(ranks)} out of range for a weight of shape {tuple(weight.shape)}")
+
+    def leading(mat, r):      # first r left singular vectors
+        u, _, _ = torch.linalg.svd(mat, full_matrices=False)
+        if u.shape[1] < r:    # unfolding has fewer columns than the rank asked for: complete the basis
+            q, _ = torch.linalg.qr(torch.cat([u, torch.eye(u.shape[0], dtype=u.dtype)[:, : r - u.shape[1]]], 1))
+            u = q
+        return u[:, :r]
+
+    unfold0 = w.reshape(N, -1)
+    unfold1 = w.transpose(0, 1).reshape(C, -1)
+    last = leading(unfold0, r_out)
+    first = leading(unfold1, r_in)
+    norm_w = torch.linalg.norm(w)
+    prev = None
+    for _ in range(n_iter_max):
+        # mode 0 given the mode-1 factor, then mode 1 given the new mode-0 factor
+        proj1 = torch.einsum("nchw,cb->nbhw", w, first)
+        last = leading(proj1.reshape(N, -1), r_out)
+        proj0 = torch.einsum("nchw,na->achw", w, last)
+        first = leading(proj0.transpose(0, 1).reshape(C, -1), r_in)
+        core = torch.einsum("achw,cb->abhw", proj0, first)
+        err = torch.sqrt(torch.clamp(norm_w ** 2 - torch.linalg.norm(core) ** 2, min=0.0)) / norm_w
+        if prev is not None and abs(float(prev - err)) < tol:
+            break
+        prev = err
+    core = torch.einsum("nchw,na,cb->abhw", w, last, first)
+    dt = weight.dtype
+    return core.to(dt), last.to(dt), first.to(dt)
+
+
 class TKConv2dC(nn.Module):
     def __init__(self, in_channels, out_channels, kernel_size, stride=1, padding=0, dilation=1, groups=1,
                  bias=True, padding_mode="zeros", hp_dict=None, name=None, dense_w=None, dense_b=None):
@@ -30,10 +77,6 @@ class TKConv2dC(nn.Module):
             raise ValueError("groups must be 1 in this mode")
         if padding_mode != "zeros":
             raise ValueError("padding_mode must be zero in this mode")
-        if dense_w is not None:
-            raise NotImplementedError(
-                "construction from a dense weight (partial Tucker decomposition) is init-time work "
-                "outside this library; decompose offline and call load_kernels()")
         super().__init__()
         kernel_size, stride, padding, dilation = _pair(kernel_size), _pair(stride), _pair(padding), _pair(dilation)
         for what, v in (("kernel_size", kernel_size), ("stride", stride), ("padding", padding), ("dilation", dilation)):
@@ -56,7 +99,15 @@ class TKConv2dC(nn.Module):
                 self.bias.data = dense_b
         else:
             self.register_parameter("bias", None)
-        self.reset_parameters()
+        if dense_w is not None:
+            if tuple(dense_w.shape) != (out_channels, in_channels, *kernel_size):
+                raise ValueError(f"dense_w must be [{out_channels},{in_channels},{kernel_size[0]},{kernel_size[1]}]")
+            core, last_factor, first_factor = partial_tucker2(dense_w, self.ranks)
+            self.first_kernel.data = first_factor.t().contiguous().unsqueeze(-1).unsqueeze(-1)
+            self.last_kernel.data = last_factor.contiguous().unsqueeze(-1).unsqueeze(-1)
+            self.core_kernel.data = core.contiguous()
+        else:
+            self.reset_parameters()
         self._ops = {}       # (batch, H, W) -> TKConvOp
         self._stamp = None   # parameter versions the native copies were packed from
 
@@ -104,6 +155,24 @@ class TKConv2dC(nn.Module):
     @torch.no_grad()
     def forward_features(self, x):
         return self._op_for(x).forward_features(x.contiguous())
+
+    @torch.no_grad()
+    def forward_flops(self, x):
+        """The reference's parameter / FLOP report (inference/TKConv.py:108-131): prints the counts in K / M and
+        returns ``(out, base_flops, compr_flops)`` with FLOPs in millions of multiply-adds."""
+        out = self.forward(x)
+        h_in, w_in = x.shape[2], x.shape[3]
+        h_out, w_out = out.shape[2], out.shape[3]
+        compr_params = (self.first_kernel.numel() + self.core_kernel.numel() + self.last_kernel.numel()) / 1000
+        compr_flops = (h_in * w_in * self.first_kernel.numel() + h_out * w_out * self.core_kernel.numel() +
+                       h_out * w_out * self.last_kernel.numel()) / 1000 / 1000
+        base_params = self.kernel_size[0] * self.kernel_size[1] * self.in_channels * self.out_channels / 1000
+        base_flops = h_out * w_out * self.kernel_size[0] * self.kernel_size[1] * self.in_channels * \
+            self.out_channels / 1000 / 1000
+        print("baseline # params: {:.2f}K\t compressed # params: {:.2f}K\t "
+              "baseline # flops: {:.2f}M\t compressed # flops: {:.2f}M".format(base_params, compr_params, base_flops,
+                                                                               compr_flops))
+        return out, base_flops, compr_flops
 
     def extra_repr(self):
         return ("first_conv(in={}, out={}, kernel_size=(1, 1), bias=False), "

@@ -3,7 +3,7 @@ from ._lib import (LIB_PATH, ConvDesc, TdcError, Tile, TileInfo, conv_desc, lib,
                    model_select)
 
 __all__ = ["LIB_PATH", "ConvDesc", "TdcError", "Tile", "TileInfo", "conv_desc", "lib", "model_enumerate",
-           "model_evaluate", "model_select", "Conv2dPlan", "TKConvOp", "TKConv2dC", "ranks_dict"]
+           "model_evaluate", "model_select", "Conv2dPlan", "TKConvOp", "TKConv2dC", "ranks_dict", "partial_tucker2"]
 
 
 def __getattr__(name):
@@ -11,7 +11,7 @@ def __getattr__(name):
     if name in ("Conv2dPlan", "TKConvOp"):
         from . import conv
         return getattr(conv, name)
-    if name in ("TKConv2dC", "ranks_dict"):
+    if name in ("TKConv2dC", "ranks_dict", "partial_tucker2"):
         from . import TKConv
         return getattr(TKConv, name)
     raise AttributeError(name)
