@@ -354,24 +354,40 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
             }
             if (ncgw & 1) mfma_group(a0, b0);
         } else if constexpr (TAPS == TAPS_1x1) {
-            // Same ping-pong and interleave, a group being four K-steps (channel groups).  K-steps past
-            // the wave's share get a zero A operand instead of a branch.
+            // Same ping-pong and interleave, a group being four K-steps (channel groups).  All operand
+            // addresses are running pointers: one vector add per pointer and group, immediate offsets
+            // inside the group (A) or one pointer per K-step of the group (B, whose stride is a run-time
+            // value).  The pointers stop at the last whole group, so the look-ahead past it re-reads
+            // that group; the K-steps that do not fill a group come afterwards, one by one.
             constexpr int G = 4;
             float a0[G][MB], b0[G][NB], a1[G][MB], b1[G][NB];
-            const int ngrp = (ncgw + G - 1) / G;
-            auto load_group = [&](int g0, float(&a)[G][MB], float(&b)[G][NB]) {
+            const int ngrp = ncgw / G;
+            const int kstride = KC * p.CS;  // floats between the B operands of consecutive K-steps
+            const float *pa[MB];
+            const float *pb[NB][G];
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) pa[mb] = sw[mb];
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+                for (int t = 0; t < G; ++t) pb[nb][t] = sin + boff[nb] + t * kstride;
+            int at_group = 0;
+            auto load_group = [&](float(&a)[G][MB], float(&b)[G][NB]) {
 #pragma unroll
                 for (int t = 0; t < G; ++t) {
-                    const bool live = g0 + t < ncgw;
-                    const int g = live ? g0 + t : ncgw - 1;
 #pragma unroll
-                    for (int mb = 0; mb < MB; ++mb) {
-                        const float av = sw[mb][g * 64];
-                        a[t][mb] = live ? av : 0.0f;
-                    }
+                    for (int mb = 0; mb < MB; ++mb) a[t][mb] = pa[mb][t * 64];
 #pragma unroll
-                    for (int nb = 0; nb < NB; ++nb) b[t][nb] = sin[g * KC * p.CS + boff[nb]];
+                    for (int nb = 0; nb < NB; ++nb) b[t][nb] = *pb[nb][t];
                 }
+                const int adv = (at_group + 1 < ngrp) ? 1 : 0;
+                at_group += adv;
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb) pa[mb] += adv * (G * 64);
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+                    for (int t = 0; t < G; ++t) pb[nb][t] += adv * (G * kstride);
             };
             auto mfma_group = [&](const float(&a)[G][MB], const float(&b)[G][NB]) {
 #pragma unroll
@@ -388,19 +404,32 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
                     __builtin_amdgcn_sched_group_barrier(0x100, MB + NB, 0);  // LDS reads
                 }
             };
-            load_group(0, a0, b0);
-            for (int gi = 0; gi + 1 < ngrp; gi += 2) {
-                __builtin_amdgcn_sched_barrier(0);
-                load_group((gi + 1) * G, a1, b1);
-                mfma_group(a0, b0);
-                interleave();
-                __builtin_amdgcn_sched_barrier(0);
-                load_group(min(gi + 2, ngrp - 1) * G, a0, b0);
-                mfma_group(a1, b1);
-                interleave();
-                __builtin_amdgcn_sched_barrier(0);
+            if (ngrp > 0) {
+                load_group(a0, b0);
+                for (int gi = 0; gi + 1 < ngrp; gi += 2) {
+                    __builtin_amdgcn_sched_barrier(0);
+                    load_group(a1, b1);
+                    mfma_group(a0, b0);
+                    interleave();
+                    __builtin_amdgcn_sched_barrier(0);
+                    load_group(a0, b0);
+                    mfma_group(a1, b1);
+                    interleave();
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+                if (ngrp & 1) mfma_group(a0, b0);
             }
-            if (ngrp & 1) mfma_group(a0, b0);
+            for (int g = ngrp * G; g < ncgw; ++g) {
+                float a[MB], b[NB];
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb) a[mb] = sw[mb][g * 64];
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb) b[nb] = sin[g * kstride + boff[nb]];
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                    for (int nb = 0; nb < NB; ++nb) acc[mb][nb] = M::run(a[mb], b[nb], acc[mb][nb]);
+            }
         } else {
             // Any filter size / dilation: taps walked at run time.
             for (int g = 0; g < ncgw; ++g) {
