@@ -88,7 +88,7 @@ enum : int { TAPS_GENERIC = 0, TAPS_1x1 = 1, TAPS_3x3 = 9 };
 constexpr int OOB_OFFSET = 0x7ffffff0;  // beyond any buffer: the load returns zero
 
 __device__ __forceinline__ int fdiv(int n, const FastDiv &f) {
-    return f.d == 1 ? n : (int)__umulhi((unsigned)n, f.m);
+    return (int)(__umulhi((unsigned)n, f.m) + ((unsigned)n & f.pass));
 }
 
 // Copy planning.  A pass moves the input window of CCH channels and the weight
@@ -104,18 +104,18 @@ __device__ __forceinline__ int fdiv(int n, const FastDiv &f) {
 constexpr int MAXPRE = 6;
 
 __device__ __forceinline__ int input_copy_offset(const ConvKParams &p, int e, int iy0, int ix0a) {
-    const int VW = p.VW;
     const int rsv = p.fd_rsv.d;  // elements per LDS row
     const int csv = p.fd_csv.d;  // elements per LDS channel slot
+    // (every factor below is under 2^24 — checked on the host — so the full-rate 24-bit multiplier serves)
     const int cl = fdiv(e, p.fd_csv);
-    const int rem = e - cl * csv;
+    const int rem = e - (int)__umul24(cl, csv);
     const int row = fdiv(rem, p.fd_rsv);
-    const int xv = rem - row * rsv;
+    const int xv = rem - (int)__umul24(row, rsv);
     const int iy = iy0 + row;
-    const int ix = ix0a + xv * VW;
+    const int ix = ix0a + (p.VW == 4 ? xv << 2 : xv);
     // Branch-free: unsigned compares fold the lower bounds in.
     const bool inb = (cl < p.CCH) & (row < p.nrows) & ((unsigned)iy < (unsigned)p.H) & ((unsigned)ix < (unsigned)p.W);
-    const int off = ((cl * p.H + iy) * p.W + ix) * 4;
+    const int off = ((int)__umul24(__umul24(cl, p.H) + iy, p.W) + ix) << 2;
     return inb ? off : OOB_OFFSET;
 }
 
@@ -132,10 +132,18 @@ __device__ __forceinline__ void copy_block(int vw, __amdgpu_buffer_rsrc_t rsrc, 
 // number `dw`; `use_pre` says that pre[] was computed for this dealing.
 // Everything that does not depend on the lane is kept in scalar registers:
 // vector ALU instructions issued next to MFMAs are not free.
-__device__ __forceinline__ void issue_pass(const ConvKParams &p, __amdgpu_buffer_rsrc_t in_rsrc,
-                                           __amdgpu_buffer_rsrc_t w_rsrc, float *__restrict__ stage,
-                                           const int (&pre)[MAXPRE], bool use_pre, int lane16, int chunk, int iy0,
-                                           int ix0a, int w_byte0, int dw, int dn, int lane) {
+// Weights: a linear copy in 16-byte elements, 1 KiB per instruction; always inside the packed buffer
+// (or past its end, which reads as zero into the slack), so the block offset can ride in the scalar operand.
+__device__ __forceinline__ void issue_weights(const ConvKParams &p, __amdgpu_buffer_rsrc_t w_rsrc,
+                                              float *__restrict__ stage, int lane16, int w_byte0, int dw, int dn) {
+    float *wdst = stage + p.in_stage_floats;
+    const int wnblk = (p.wslab_floats + 255) >> 8;
+    for (int blk = dw; blk < wnblk; blk += dn) copy_block(4, w_rsrc, wdst + (blk << 8), lane16, w_byte0 + (blk << 10));
+}
+
+__device__ __forceinline__ void issue_inputs(const ConvKParams &p, __amdgpu_buffer_rsrc_t in_rsrc,
+                                             float *__restrict__ stage, const int (&pre)[MAXPRE], bool use_pre, int chunk,
+                                             int iy0, int ix0a, int dw, int dn, int lane) {
     const int VW = p.VW;
     const int blk_floats = 64 * VW;
     const int nblk = p.in_stage_floats / blk_floats;
@@ -153,11 +161,6 @@ __device__ __forceinline__ void issue_pass(const ConvKParams &p, __amdgpu_buffer
     }
     for (int blk = first_computed; blk < nblk; blk += dn)
         copy_block(VW, in_rsrc, stage + blk * blk_floats, input_copy_offset(p, (blk << 6) + lane, iy0, ix0a) + pass_bytes, 0);
-    // Weights: a linear copy in 16-byte elements, 1 KiB per instruction; always inside the packed buffer
-    // (or past its end, which reads as zero into the slack), so the block offset can ride in the scalar operand.
-    float *wdst = stage + p.in_stage_floats;
-    const int wnblk = (p.wslab_floats + 255) >> 8;
-    for (int blk = dw; blk < wnblk; blk += dn) copy_block(4, w_rsrc, wdst + (blk << 8), lane16, w_byte0 + (blk << 10));
 }
 
 template <int MF, int MB, int NB, int TAPS, int MAXW>
@@ -175,7 +178,9 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
                  "s"(p.stage_floats), "s"(p.nstage), "s"(p.nchunks), "s"(p.fd_csv.m), "s"(p.fd_csv.d),
                  "s"(p.fd_rsv.m), "s"(p.fd_rsv.d), "s"(p.fd_ntx.m), "s"(p.fd_wk.m), "s"(p.fd_wn.m), "s"(p.WK),
                  "s"(p.WN), "s"(p.in_bstride), "s"(p.wpk_bytes), "s"(p.KS), "s"(p.cps), "s"(p.fd_ks.m), "s"(p.WL), "s"(p.xcd_chunk), "s"(p.n_wg), "s"(p.fd_g1.m),
-                 "s"(p.fd_g1.d), "s"(p.fd_g2.m), "s"(p.fd_g2.d), "s"(p.channel_major));
+                 "s"(p.fd_g1.d), "s"(p.fd_g2.m), "s"(p.fd_g2.d), "s"(p.channel_major), "s"(p.fd_csv.pass),
+                 "s"(p.fd_rsv.pass), "s"(p.fd_ntx.pass), "s"(p.fd_wk.pass), "s"(p.fd_wn.pass), "s"(p.fd_ks.pass),
+                 "s"(p.fd_g1.pass), "s"(p.fd_g2.pass));
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -237,30 +242,43 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
     const unsigned w_pass_bytes = (unsigned)p.wslab_floats * 4u;
     const unsigned w_byte_base = (unsigned)by * (unsigned)p.nchunks * w_pass_bytes;
 
-    // Offsets of this lane's elements in its wave's first MAXPRE input blocks (pass 0), for the steady dealing.
-    int pre[MAXPRE];
-#pragma unroll
-    for (int i = 0; i < MAXPRE; ++i) {
-        const int e = ((dw + i * dn) << 6) + lane;
-        pre[i] = OOB_OFFSET;
-        if (e < p.in_stage_floats && dw >= 0)  // (in elements this bound is only tighter)
-            pre[i] = input_copy_offset(p, e, iy0, ix0a);
-    }
+    // The weight copies of the first pass need no per-lane arithmetic: start them before anything else.
     const int lane16 = lane * 16;
-    auto issue = [&](int chunk, bool everybody) {
-        float *stage = lds + ((chunk - chunk0) & (p.nstage - 1)) * p.stage_floats;
-        const int w_byte0 = (int)(w_byte_base + (unsigned)chunk * w_pass_bytes);
-        if (everybody) {
-            issue_pass(p, in_rsrc, w_rsrc, stage, pre, p.WL == 0, lane16, chunk, iy0, ix0a, w_byte0, wave, nwaves, lane);
-        } else if (dw >= 0) {
-            // Copy issue competes for the SIMD with other waves' MFMA streams and loses by default (measured:
-            // ~330 cycles per copy instruction instead of ~115); it is short, so let it go first.
-            __builtin_amdgcn_s_setprio(3);
-            issue_pass(p, in_rsrc, w_rsrc, stage, pre, true, lane16, chunk, iy0, ix0a, w_byte0, dw, dn, lane);
-            __builtin_amdgcn_s_setprio(0);
+    issue_weights(p, w_rsrc, lds, lane16, (int)(w_byte_base + (unsigned)chunk0 * w_pass_bytes), wave, nwaves);
+
+    // Offsets of this lane's elements in its wave's first MAXPRE input blocks (pass 0), for the steady dealing
+    // (positions past the stage decode to a channel >= CCH and so to the out-of-range offset).  With loader
+    // waves the first pass is dealt differently and computes its offsets on the fly, so the table is only
+    // filled afterwards, by the loaders, while the first copies are in flight.
+    int pre[MAXPRE];
+    const int in_nblk = p.in_stage_floats / (64 * p.VW);
+    auto fill_pre = [&]() {
+#pragma unroll
+        for (int i = 0; i < MAXPRE; ++i) {
+            pre[i] = OOB_OFFSET;
+            if (dw >= 0 && dw + i * dn < in_nblk)  // wave-uniform: no arithmetic for blocks this wave does not copy
+                pre[i] = input_copy_offset(p, ((dw + i * dn) << 6) + lane, iy0, ix0a);
         }
     };
-    issue(chunk0, true);
+    if (p.WL == 0) {
+        fill_pre();
+        issue_inputs(p, in_rsrc, lds, pre, true, chunk0, iy0, ix0a, wave, nwaves, lane);
+    } else {
+        issue_inputs(p, in_rsrc, lds, pre, false, chunk0, iy0, ix0a, wave, nwaves, lane);
+        fill_pre();
+    }
+    auto issue = [&](int chunk) {
+        if (dw < 0) return;
+        float *stage = lds + ((chunk - chunk0) & (p.nstage - 1)) * p.stage_floats;
+        const int w_byte0 = (int)(w_byte_base + (unsigned)chunk * w_pass_bytes);
+        // Copy issue competes for the SIMD with other waves' MFMA streams and loses by default (measured:
+        // ~330 cycles per copy instruction instead of ~115); it is short, so let it go first.
+        __builtin_amdgcn_s_setprio(3);
+        issue_weights(p, w_rsrc, stage, lane16, w_byte0, dw, dn);
+        issue_inputs(p, in_rsrc, stage, pre, true, chunk, iy0, ix0a, dw, dn, lane);
+        __builtin_amdgcn_s_setprio(0);
+    };
+
     // Per-lane LDS offset (floats) of tap (0,0) for each pixel block, channel sub-index included.
     int boff[NB];
 #pragma unroll
@@ -289,7 +307,7 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
         // everybody is done reading the stage the next pass is about to overwrite.
         __builtin_amdgcn_s_waitcnt(0);
         __syncthreads();
-        if (chunk + 1 < chunk1) issue(chunk + 1, false);
+        if (chunk + 1 < chunk1) issue(chunk + 1);
         if (loader) continue;
 
         const float *stage = lds + ((chunk - chunk0) & (p.nstage - 1)) * p.stage_floats;

@@ -74,17 +74,19 @@ bool model_set_constants(const double *in, int n);
 size_t packed_weight_floats(const Geometry &g);
 void pack_weights(const tdc_conv_desc &d, const tdc_tile &t, const Geometry &g, const float *w_oihw, float *packed);
 
-// Division of a small non-negative integer by a run-time constant as one
-// multiply-high: q = (n * m) >> 32 with m = floor(2^32 / d) + 1, exact whenever
-// n * d < 2^32.  d == 1 is passed through.
+// Division of a small non-negative integer by a run-time constant without a branch:
+// q = ((n * m) >> 32) + (n & pass) with m = floor(2^32 / d) + 1, pass = 0 for d > 1 (exact whenever
+// n * d < 2^32) and m = 0, pass = ~0 for d == 1.
 struct FastDiv {
     unsigned m;
     int d;
+    unsigned pass;
 };
 inline FastDiv make_fastdiv(int d) {
     FastDiv f;
     f.d = d;
     f.m = d > 1 ? (unsigned)((1ULL << 32) / (unsigned)d + 1ULL) : 0u;
+    f.pass = d > 1 ? 0u : ~0u;
     return f;
 }
 

@@ -79,6 +79,8 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
     const bool flat = (d.KH == 1 && d.KW == 1 && d.stride == 1 && d.pad == 0);
     g.He = flat ? 1 : d.H;
     g.We = flat ? d.H * d.W : d.W;
+    // (the copy-offset arithmetic of the kernel uses 24-bit multiplies)
+    if ((long long)(d.C + 1) * g.He >= (1LL << 24) || g.We >= (1 << 24)) return fail("image too large");
     g.Ho = (g.He + 2 * d.pad - d.dilation * (d.KH - 1) - 1) / d.stride + 1;
     g.Wo = (g.We + 2 * d.pad - d.dilation * (d.KW - 1) - 1) / d.stride + 1;
     g.P = g.Ho * g.Wo;
