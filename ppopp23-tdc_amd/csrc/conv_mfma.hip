@@ -261,8 +261,20 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
         }
     };
     if (p.WL == 0) {
-        fill_pre();
-        issue_inputs(p, in_rsrc, lds, pre, true, chunk0, iy0, ix0a, wave, nwaves, lane);
+        // Every offset goes out as a copy as soon as it is known (the scheduling barrier keeps the compiler
+        // from computing the whole table first); blocks beyond the table follow.
+        const int pass_bytes0 = chunk0 * p.CCH * p.H * p.W * 4;
+#pragma unroll
+        for (int i = 0; i < MAXPRE; ++i) {
+            pre[i] = OOB_OFFSET;
+            if (dw + i * dn < in_nblk) {
+                pre[i] = input_copy_offset(p, ((dw + i * dn) << 6) + lane, iy0, ix0a);
+                copy_block(p.VW, in_rsrc, lds + (dw + i * dn) * 64 * p.VW, pre[i] + pass_bytes0, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        for (int blk = dw + MAXPRE * dn; blk < in_nblk; blk += dn)
+            copy_block(p.VW, in_rsrc, lds + blk * 64 * p.VW, input_copy_offset(p, (blk << 6) + lane, iy0, ix0a) + pass_bytes0, 0);
     } else {
         issue_inputs(p, in_rsrc, lds, pre, false, chunk0, iy0, ix0a, wave, nwaves, lane);
         fill_pre();
