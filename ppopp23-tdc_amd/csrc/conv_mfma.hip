@@ -536,8 +536,15 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
                 if (n < p.N && jy < p.TH && oy < p.Ho && ox < p.Wo) {
                     float val = 0.0f;
                     if (want_value) {
-                        val = lds[idx];
-                        for (int k = 1; k < p.WK; ++k) val += lds[k * total + idx];
+                        // four reads in flight at a time; the additions stay in slice order
+                        for (int k0 = 0; k0 < p.WK; k0 += 4) {
+                            float part[4];
+#pragma unroll
+                            for (int u = 0; u < 4; ++u) part[u] = lds[min(k0 + u, p.WK - 1) * total + idx];
+#pragma unroll
+                            for (int u = 0; u < 4; ++u)
+                                if (k0 + u < p.WK) val += part[u];
+                        }
                     }
                     sink(n, oy * p.Wo + ox, val);
                 }
