@@ -55,6 +55,7 @@ struct Geometry {
     int lds_bytes = 0;
     int max_waves_kernel = 0;        // launch bound of the instantiated kernel
     int channel_major = 0;           // which logical workgroup order costs fewer L2 fills (see conv_mfma.hip)
+    double b_ways = 1.0;             // serialisation of the B-operand LDS read by bank conflicts (1 = none)
 };
 
 // Returns false (and a reason) when the tile cannot be launched for this shape.

@@ -10,6 +10,8 @@
 // copy volume of the staged input window and weights, and wave quantisation over
 // 256 compute units.  Host-only code: it runs without a GPU.
 #include <algorithm>
+#include <array>
+#include <map>
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
@@ -46,19 +48,60 @@ bool check_desc(const tdc_conv_desc &d, std::string *why) {
     return true;
 }
 
-// LDS channel stride: the lanes of one ds_read that belong to different input
-// channels of an MFMA K-step should fall into different banks.  With 4-byte
-// banks a stride of 32 (mod 64) separates the two halves of a 32x32x2 step and
-// a stride of 16 (mod 32) the quarters of a 16x16x4 step.  Small windows are
-// not inflated by more than a quarter for this.
-static int pad_channel_stride(int raw, int mf, int vw) {
-    const int mod = (mf == 32) ? 64 : 32;
-    const int want = (mf == 32) ? 32 : 16;
-    int cs = round_up(raw, vw);
-    int padded = cs;
-    while (padded % mod != want) padded += vw;
-    if (padded - raw <= raw / 4) cs = padded;
-    return cs;
+// LDS bank conflicts of the B-operand read.  The 64 lanes of a wave read one word each: lane l holds pixel
+// l % mf of its block and input channel l / mf of the K-step, i.e. word jy*stride*RS + jx*stride + (l/mf)*CS
+// (+ the same tap offset for everybody).  The LDS has 64 four-byte banks; lanes that hit one bank with
+// different words are served one after the other.  Returned: that serialisation factor (1 = conflict-free),
+// averaged over the pixel blocks of a workgroup tile.
+static double b_read_conflict_ways(int mf, int PT, int TW, int TH, int RS, int CS, int stride) {
+    double sum = 0.0;
+    int blocks = 0;
+    for (int j0 = 0; j0 < PT; j0 += mf, ++blocks) {
+        int words[64][8], cnt[64];
+        for (int b = 0; b < 64; ++b) cnt[b] = 0;
+        int ways = 1;
+        for (int l = 0; l < 64; ++l) {
+            const int j = j0 + l % mf;
+            const int jy = std::min(j / TW, TH - 1), jx = j % TW;
+            const int w = jy * stride * RS + jx * stride + (l / mf) * CS;
+            const int b = w & 63;
+            bool seen = false;
+            for (int i = 0; i < cnt[b]; ++i) seen |= (words[b][i] == w);
+            if (!seen && cnt[b] < 8) words[b][cnt[b]++] = w;
+            ways = std::max(ways, cnt[b]);
+        }
+        sum += ways;
+    }
+    return blocks ? sum / blocks : 1.0;
+}
+
+// LDS channel stride: the smallest stride from the raw window size upwards (inflating small windows by at
+// most a quarter, larger ones by at most 64 words) that gives the B-operand read the fewest bank conflicts.
+// For tiles whose pixel blocks lie in one row this is the classic rule — stride = 16 (mod 32) for the four
+// channel quarters of a 16x16x4 step, 32 (mod 64) for the halves of a 32x32x2 step; narrow tiles whose
+// blocks wrap over several rows cannot be made conflict-free and get the best stride there is.
+static int pad_channel_stride(int raw, int mf, int vw, int PT, int TW, int TH, int RS, int stride, double *ways_out) {
+    // Thousands of candidate tiles share a handful of window shapes: remember the answers (per thread).
+    static thread_local std::map<std::array<int, 8>, std::pair<int, double>> memo;
+    const std::array<int, 8> key{raw, mf, vw, PT, TW, TH, RS, stride};
+    auto hit = memo.find(key);
+    if (hit == memo.end()) {
+        const int first = round_up(raw, vw);
+        const int budget = std::max(raw / 4, std::min(64, raw));
+        int best = first;
+        double best_ways = 1e9;
+        for (int cs = first; cs - raw <= budget; cs += vw) {
+            const double ways = b_read_conflict_ways(mf, PT, TW, TH, RS, cs, stride);
+            if (ways < best_ways - 1e-9) {
+                best_ways = ways;
+                best = cs;
+            }
+        }
+        if (memo.size() > 100000) memo.clear();
+        hit = memo.emplace(key, std::make_pair(best, best_ways)).first;
+    }
+    *ways_out = hit->second.second;
+    return hit->second.first;
 }
 
 bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::string *why) {
@@ -127,7 +170,7 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
     } else {
         g.RS = g.ncols;
     }
-    g.CS = pad_channel_stride(g.nrows * g.RS, t.mf, g.VW);
+    g.CS = pad_channel_stride(g.nrows * g.RS, t.mf, g.VW, g.PT, g.TW, g.TH, g.RS, d.stride, &g.b_ways);
     // Copies are issued in whole blocks of 64 elements (1 KiB with 16-byte elements): both parts of
     // a stage are rounded up to that, the slack receiving zeros.
     g.in_stage_floats = round_up(t.cch * g.CS, 256);
@@ -189,21 +232,22 @@ namespace {
 // (2080Ti-evaluation/TDC-LAYERS-MODELING/model.py:265-266,278).
 struct ModelConst {
     double launch_us = 1.474;           // device time of an empty kernel in a back-to-back stream
-    double setup_clk = 1399;          // kernel arguments and index arithmetic before the first copy is issued
-    double copy_latency_clk = 1083;   // first byte of a global->LDS copy (L2 / memory-side cache)
+    double setup_clk = 1007;          // kernel arguments and index arithmetic before the first copy is issued
+    double copy_latency_clk = 920.5;   // first byte of a global->LDS copy (L2 / memory-side cache)
     double copy_bytes_per_clk = 33.65;   // sustained global->LDS rate of one CU
-    double l2_bytes_per_clk = 7865;   // whole-chip L2->CU rate when every CU copies at once
-    double lds_bytes_per_clk = 15.13;   // LDS traffic of the split-K reduction
+    double l2_bytes_per_clk = 9627;   // whole-chip L2->CU rate when every CU copies at once
+    double lds_bytes_per_clk = 21.79;   // LDS traffic of the split-K reduction
     double sync_clk = 224.8;            // one workgroup barrier
-    double store_bytes_per_clk = 2.265;  // per CU, short runs per channel
-    double kstep_issue_clk = 1.764;      // vector-ALU / LDS-issue cycles per operand read, not hidden under MFMAs
-    double pass_overhead_clk = 567.4;   // per wave and pass: copy issue, pointer set-up, pipeline fill
-    double wave_setup_clk = 212.8;      // prologue cycles added per extra wave sharing a SIMD
-    double ksplit_clk = 3611;         // split across workgroups: write-through, ticket round trip, read-back
+    double store_bytes_per_clk = 2.718;  // per CU, short runs per channel
+    double kstep_issue_clk = 2.743;      // vector-ALU / LDS-issue cycles per operand read, not hidden under MFMAs
+    double pass_overhead_clk = 578.7;   // per wave and pass: copy issue, pointer set-up, pipeline fill
+    double wave_setup_clk = 772.2;      // prologue cycles added per extra wave sharing a SIMD
+    double ksplit_clk = 4604;         // split across workgroups: write-through, ticket round trip, read-back
     double copy_issue_clk = 118.2;      // a wave is held this long by every global->LDS copy instruction it issues
+    double lds_read_clk = 2.88;        // LDS busy cycles per conflict-free operand read of one wave
 };
 ModelConst MC;
-constexpr int kNumModelConst = 13;
+constexpr int kNumModelConst = 14;
 
 double *mc_field(int i) {
     switch (i) {
@@ -220,6 +264,7 @@ double *mc_field(int i) {
         case 10: return &MC.wave_setup_clk;
         case 11: return &MC.ksplit_clk;
         case 12: return &MC.copy_issue_clk;
+        case 13: return &MC.lds_read_clk;
         default: return nullptr;
     }
 }
@@ -295,9 +340,11 @@ bool model_evaluate(const tdc_conv_desc &d, const tdc_tile &t, tdc_tile_info &in
         const double waves_simd = (double)comp_waves_per_simd * r;
         // A wave alone on its SIMD stalls on every operand read and while it issues copies; with several
         // waves per SIMD those gaps are filled by the others until the matrix pipe itself is the limit.
-        const double stall = ksteps_pass * (t.mb + t.nb) * MC.kstep_issue_clk + MC.pass_overhead_clk;
+        const double stall = ksteps_pass * (t.mb + t.nb * g.b_ways) * MC.kstep_issue_clk + MC.pass_overhead_clk;
         const double alone = mfma_pass + stall;
-        const double pipe = mfma_pass * waves_simd + MC.pass_overhead_clk;
+        // ... or the LDS: every operand read keeps it busy for lds_read_clk cycles, a conflicting one longer.
+        const double lds_busy = ksteps_pass * (t.mb + t.nb * g.b_ways) * MC.lds_read_clk * ncomp * r;
+        const double pipe = std::max(mfma_pass * waves_simd, lds_busy) + MC.pass_overhead_clk;
         const double compute = std::max(alone, pipe) + MC.sync_clk;
         const double compute_issuing = std::max(alone + issue_steady, pipe) + MC.sync_clk;
         const double chip_share =

@@ -164,7 +164,7 @@ def model_evaluate(desc: ConvDesc, tile: Tile) -> TileInfo:
 
 MODEL_CONSTANT_NAMES = ("launch_us", "setup_clk", "copy_latency_clk", "copy_bytes_per_clk", "l2_bytes_per_clk",
                         "lds_bytes_per_clk", "sync_clk", "store_bytes_per_clk", "kstep_issue_clk", "pass_overhead_clk",
-                        "wave_setup_clk", "ksplit_clk", "copy_issue_clk")
+                        "wave_setup_clk", "ksplit_clk", "copy_issue_clk", "lds_read_clk")
 
 
 def model_get_constants():
