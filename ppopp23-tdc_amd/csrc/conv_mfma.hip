@@ -649,9 +649,11 @@ const void *conv_kernel_for(const tdc_tile &t, int KH, int KW, int dilation) {
 
 int prepare_conv_kernel(const void *fn, const Geometry &g) {
     if (!fn) return (int)hipErrorInvalidValue;
-    // Dynamic LDS above the 64 KiB default has to be opted into per kernel.
+    // Dynamic LDS above the 64 KiB default has to be opted into per kernel function.  The attribute belongs to
+    // the function, not to the plan, and several plans share one instantiation: always raise it to the whole
+    // LDS, so that a later plan with a smaller request cannot lower it under an earlier plan's feet.
     if (g.lds_bytes > 64 * 1024) {
-        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, g.lds_bytes);
+        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, machine().lds_bytes_per_cu);
         if (e != hipSuccess) return (int)e;
     }
     return 0;

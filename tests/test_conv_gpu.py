@@ -186,6 +186,31 @@ def test_both_logical_workgroup_orders(order, monkeypatch):
             assert_close(run_conv(x, w, stride=stride, pad=K // 2, tile=t), want, f"order {order} {t}")
 
 
+def test_plans_sharing_a_kernel_keep_their_large_lds_requests():
+    """Two plans on the same kernel instantiation, both above the 64 KiB default of dynamic LDS, the second asking
+    for less: the first must still launch (the opt-in attribute is per function, not per plan)."""
+    B, C, N, H, W = 1, 128, 32, 28, 28
+    desc = tdc_amd.conv_desc(B, C, N, H, W, 3, 3, 1, 1)
+    cands = [(tdc_amd.model_evaluate(desc, t).lds_bytes, t) for t in tdc_amd.model_enumerate(desc)
+             if (t.mf, t.mb, t.nb, t.ks) == (16, 1, 1, 1)]
+    big = max(cands, key=lambda c: c[0])
+    mid = min((c for c in cands if c[0] > 70 * 1024), key=lambda c: c[0])
+    assert big[0] > 120 * 1024 and mid[0] < big[0] - 16 * 1024
+    announce("lds", big, mid)
+    x, w = case(8000, B, C, N, H, W, 3)
+    want = ref.conv2d_torch(x, w, pad=1).numpy()
+    pa = tdc_amd.Conv2dPlan(B, C, N, H, W, 3, 3, 1, 1, tile=big[1]).set_weights(w)
+    pb = tdc_amd.Conv2dPlan(B, C, N, H, W, 3, 3, 1, 1, tile=mid[1]).set_weights(w)
+    xd = x.cuda()
+    for plan in (pb, pa, pb, pa):
+        out = torch.full((B, N, H, W), float("nan"), device="cuda")
+        plan.forward(xd, out=out)
+        torch.cuda.synchronize()
+        assert_close(out.cpu().numpy(), want, "shared kernel, different LDS sizes")
+    pa.close()
+    pb.close()
+
+
 def test_split_across_workgroups_rejects_empty_slices():
     with pytest.raises(tdc_amd.TdcError):   # 40 channels in passes of 8 = 5 passes: 4 slices take 2,2,1,0
         tdc_amd.model_evaluate(tdc_amd.conv_desc(1, 40, 16, 9, 9, 3, 3, 1, 1), tdc_amd.Tile(16, 1, 1, 1, 1, 1, 8, 8, ks=4))
