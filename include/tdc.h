@@ -112,6 +112,10 @@ int tdc_conv_plan_create(const tdc_conv_desc *desc, const tdc_tile *forced_tile,
                          tdc_conv_plan **plan_out);
 /* Host OIHW weights [N,C,KH,KW]; bias [N] or NULL (must match has_bias). */
 int tdc_conv_plan_set_weights(tdc_conv_plan *plan, const float *w_oihw, const float *bias);
+/* Optional, 1x1 convolutions without padding only: y = conv(relu?(x * scale[c] + shift[c])) in one kernel —
+ * the norm -> relu -> conv order of the reference's DenseNet layers (inference/densenet_inet_tt.py:36-69), where the
+ * BatchNorm sits in front of the convolution and cannot be folded into its weights.  Host arrays of C floats. */
+int tdc_conv_plan_set_input_affine(tdc_conv_plan *plan, const float *scale, const float *shift, int32_t relu);
 int tdc_conv_plan_query(const tdc_conv_plan *plan, tdc_tile_info *info_out);
 /* d_residual may be NULL.  Output need not be pre-zeroed.  Asynchronous. */
 int tdc_conv_forward(tdc_conv_plan *plan, const float *d_in, const float *d_residual,
@@ -210,6 +214,10 @@ int tdc_net_global_avgpool(tdc_net *net, int32_t in, int32_t *out);
 /* Per-channel y = x*scale[c] + shift[c], then ReLU if relu != 0 (inference BatchNorm in front of a convolution). */
 int tdc_net_affine(tdc_net *net, int32_t in, const float *scale, const float *shift, int32_t relu, int32_t dst,
                    int32_t *out);
+/* tdc_net_affine followed by a 1x1 convolution (stride 1, no padding), as ONE kernel: the affine (+ReLU when
+ * affine_relu != 0) is applied to the input window inside the convolution. */
+int tdc_net_affine_conv(tdc_net *net, int32_t in, const float *scale, const float *shift, int32_t affine_relu, int32_t N,
+                        const float *w_oi11, const float *bias, int32_t residual, int32_t relu, int32_t dst, int32_t *out);
 /* Channel concatenation of n tensors of equal height/width into a new tensor (by copy). */
 int tdc_net_concat(tdc_net *net, const int32_t *ins, int32_t n, int32_t *out);
 int tdc_net_tensor_shape(const tdc_net *net, int32_t id, int32_t *C, int32_t *H, int32_t *W);

@@ -135,10 +135,19 @@ __device__ __forceinline__ void copy_block(int vw, __amdgpu_buffer_rsrc_t rsrc, 
 // Weights: a linear copy in 16-byte elements, 1 KiB per instruction; always inside the packed buffer
 // (or past its end, which reads as zero into the slack), so the block offset can ride in the scalar operand.
 __device__ __forceinline__ void issue_weights(const ConvKParams &p, __amdgpu_buffer_rsrc_t w_rsrc,
-                                              float *__restrict__ stage, int lane16, int w_byte0, int dw, int dn) {
+                                              float *__restrict__ stage, int lane16, int w_byte0, int dw, int dn, int chunk) {
     float *wdst = stage + p.in_stage_floats;
     const int wnblk = (p.wslab_floats + 255) >> 8;
     for (int blk = dw; blk < wnblk; blk += dn) copy_block(4, w_rsrc, wdst + (blk << 8), lane16, w_byte0 + (blk << 10));
+    // The per-channel scale and shift of an input affine ride behind the weights: [pass][scale(CCH) | shift(CCH)].
+    if (p.in_aff) {
+        const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<float *>(p.in_aff), (short)0, (int)(p.nchunks * p.CCH * 8), 0x00020000);
+        float *adst = wdst + (wnblk << 8);
+        const int anblk = (2 * p.CCH + 255) >> 8;
+        for (int blk = dw; blk < anblk; blk += dn)
+            copy_block(4, a_rsrc, adst + (blk << 8), lane16, chunk * p.CCH * 8 + (blk << 10));
+    }
 }
 
 __device__ __forceinline__ void issue_inputs(const ConvKParams &p, __amdgpu_buffer_rsrc_t in_rsrc,
@@ -171,16 +180,22 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
     constexpr int NACC = M::NACC;
     extern __shared__ __align__(16) float lds[];
 
-    // Fetch every kernel argument the prologue needs in one go: left alone, the compiler loads them in
-    // several dependent batches, each costing a scalar-cache round trip before the first copy can start.
-    asm volatile("" ::"s"(p.in), "s"(p.wpk), "s"(p.H), "s"(p.W), "s"(p.CCH), "s"(p.nrows), "s"(p.TW), "s"(p.TH),
-                 "s"(p.ntx), "s"(p.stride), "s"(p.pad), "s"(p.VW), "s"(p.in_stage_floats), "s"(p.wslab_floats),
-                 "s"(p.stage_floats), "s"(p.nstage), "s"(p.nchunks), "s"(p.fd_csv.m), "s"(p.fd_csv.d),
-                 "s"(p.fd_rsv.m), "s"(p.fd_rsv.d), "s"(p.fd_ntx.m), "s"(p.fd_wk.m), "s"(p.fd_wn.m), "s"(p.WK),
-                 "s"(p.WN), "s"(p.in_bstride), "s"(p.wpk_bytes), "s"(p.KS), "s"(p.cps), "s"(p.fd_ks.m), "s"(p.WL), "s"(p.xcd_chunk), "s"(p.n_wg), "s"(p.fd_g1.m),
-                 "s"(p.fd_g1.d), "s"(p.fd_g2.m), "s"(p.fd_g2.d), "s"(p.channel_major), "s"(p.fd_csv.pass),
-                 "s"(p.fd_rsv.pass), "s"(p.fd_ntx.pass), "s"(p.fd_wk.pass), "s"(p.fd_wn.pass), "s"(p.fd_ks.pass),
-                 "s"(p.fd_g1.pass), "s"(p.fd_g2.pass));
+    // The kernel arguments (about 400 bytes) are read through the scalar cache.  Left alone, the compiler fetches
+    // them in several dependent batches, and every batch that touches a cache line for the first time costs a
+    // round trip to L2 before the first copy can start.  Touch every line of the argument block at once: whatever
+    // order the compiler then loads the values in, it hits the scalar cache.
+    {
+        static_assert(sizeof(ConvKParams) <= 8 * 64, "touch more lines");
+        const auto kargs = __builtin_amdgcn_kernarg_segment_ptr();
+        unsigned t0, t1, t2, t3, t4, t5, t6, t7;
+        asm volatile(
+            "s_load_dword %0, %8, 0x0\n\ts_load_dword %1, %8, 0x40\n\ts_load_dword %2, %8, 0x80\n\t"
+            "s_load_dword %3, %8, 0xc0\n\ts_load_dword %4, %8, 0x100\n\ts_load_dword %5, %8, 0x140\n\t"
+            "s_load_dword %6, %8, 0x180\n\ts_load_dword %7, %8, 0x1c0\n\ts_waitcnt lgkmcnt(0)"
+            : "=&s"(t0), "=&s"(t1), "=&s"(t2), "=&s"(t3), "=&s"(t4), "=&s"(t5), "=&s"(t6), "=&s"(t7)
+            : "s"(kargs)
+            : "memory");
+    }
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -244,7 +259,7 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
 
     // The weight copies of the first pass need no per-lane arithmetic: start them before anything else.
     const int lane16 = lane * 16;
-    issue_weights(p, w_rsrc, lds, lane16, (int)(w_byte_base + (unsigned)chunk0 * w_pass_bytes), wave, nwaves);
+    issue_weights(p, w_rsrc, lds, lane16, (int)(w_byte_base + (unsigned)chunk0 * w_pass_bytes), wave, nwaves, chunk0);
 
     // Offsets of this lane's elements in its wave's first MAXPRE input blocks (pass 0), for the steady dealing
     // (positions past the stage decode to a channel >= CCH and so to the out-of-range offset).  With loader
@@ -286,7 +301,7 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
         // Copy issue competes for the SIMD with other waves' MFMA streams and loses by default (measured:
         // ~330 cycles per copy instruction instead of ~115); it is short, so let it go first.
         __builtin_amdgcn_s_setprio(3);
-        issue_weights(p, w_rsrc, stage, lane16, w_byte0, dw, dn);
+        issue_weights(p, w_rsrc, stage, lane16, w_byte0, dw, dn, chunk);
         issue_inputs(p, in_rsrc, stage, pre, true, chunk, iy0, ix0a, dw, dn, lane);
         __builtin_amdgcn_s_setprio(0);
     };
@@ -320,6 +335,58 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
         __builtin_amdgcn_s_waitcnt(0);
         __syncthreads();
         if (chunk + 1 < chunk1) issue(chunk + 1);
+        if constexpr (TAPS == TAPS_1x1) {
+            // Optional per-input-channel affine (+ReLU) in front of the convolution (an inference BatchNorm that
+            // cannot be folded into a producer): applied in place to the freshly landed input window.  A 1x1
+            // convolution without padding has no zero halo that would have to stay zero; lanes past the image and
+            // channels past C are multiplied by zero weights or never stored.
+            if (p.in_aff) {
+                float *win = lds + ((chunk - chunk0) & (p.nstage - 1)) * p.stage_floats;
+                const float *aff = win + p.in_stage_floats + ((p.wslab_floats + 255) & ~255);  // [scale(CCH) | shift(CCH)]
+                const int nel = p.CCH * p.fd_csv.d;
+                // four elements per thread in flight: the LDS round trips overlap
+                for (int e0 = tid; e0 < nel; e0 += 4 * nthreads) {
+                    if (p.VW == 4) {
+                        f4_t v[4];
+                        float sc[4], sh[4];
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) {
+                            const int e = min(e0 + u * nthreads, nel - 1);
+                            const int cl = fdiv(e, p.fd_csv);
+                            v[u] = *reinterpret_cast<f4_t *>(win + e * 4);
+                            sc[u] = aff[cl];
+                            sh[u] = aff[p.CCH + cl];
+                        }
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) {
+#pragma unroll
+                            for (int i = 0; i < 4; ++i) {
+                                v[u][i] = v[u][i] * sc[u] + sh[u];
+                                if (p.in_relu) v[u][i] = fmaxf(v[u][i], 0.0f);
+                            }
+                            if (e0 + u * nthreads < nel) *reinterpret_cast<f4_t *>(win + (e0 + u * nthreads) * 4) = v[u];
+                        }
+                    } else {
+                        float v[4], sc[4], sh[4];
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) {
+                            const int e = min(e0 + u * nthreads, nel - 1);
+                            const int cl = fdiv(e, p.fd_csv);
+                            v[u] = win[e];
+                            sc[u] = aff[cl];
+                            sh[u] = aff[p.CCH + cl];
+                        }
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) {
+                            v[u] = v[u] * sc[u] + sh[u];
+                            if (p.in_relu) v[u] = fmaxf(v[u], 0.0f);
+                            if (e0 + u * nthreads < nel) win[e0 + u * nthreads] = v[u];
+                        }
+                    }
+                }
+                __syncthreads();
+            }
+        }
         if (loader) continue;
 
         const float *stage = lds + ((chunk - chunk0) & (p.nstage - 1)) * p.stage_floats;

@@ -196,6 +196,15 @@ int tdc_net_conv(tdc_net *net, int32_t in, int32_t N, int32_t KH, int32_t KW, in
     return TDC_OK;
 }
 
+int tdc_net_affine_conv(tdc_net *net, int32_t in, const float *scale, const float *shift, int32_t affine_relu, int32_t N,
+                        const float *w, const float *bias, int32_t residual, int32_t relu, int32_t dst, int32_t *out) {
+    if (!scale || !shift) return api_fail(TDC_ERR_INVALID, "null argument");
+    int st = tdc_net_conv(net, in, N, 1, 1, 1, 0, w, bias, residual, relu, dst, out);
+    if (st != TDC_OK) return st;
+    // the convolution just appended is the last op
+    return tdc_conv_plan_set_input_affine(net->ops.back().conv, scale, shift, affine_relu);
+}
+
 int tdc_net_tkconv(tdc_net *net, int32_t in, int32_t R1, int32_t R2, int32_t N, int32_t K, int32_t stride, int32_t pad,
                    const float *first, const float *core, const float *last, const float *bias, int32_t residual,
                    int32_t relu, int32_t dst, int32_t *out) {

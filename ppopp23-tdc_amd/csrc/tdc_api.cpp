@@ -45,6 +45,8 @@ struct tdc_conv_plan {
     float *d_bias = nullptr;
     float *d_ws = nullptr;        // tile.ks > 1: partial tiles [batch][ks][N][P]
     unsigned *d_ctr = nullptr;    // tile.ks > 1: ticket counters, zero between launches
+    float *d_in_aff = nullptr;    // optional input affine: [pass][scale(cch) | shift(cch)]
+    int in_relu = 0;
     bool have_weights = false;
 };
 
@@ -53,6 +55,8 @@ static void free_plan_buffers(tdc_conv_plan *p) {
     if (p->d_bias) (void)hipFree(p->d_bias);
     if (p->d_ws) (void)hipFree(p->d_ws);
     if (p->d_ctr) (void)hipFree(p->d_ctr);
+    if (p->d_in_aff) (void)hipFree(p->d_in_aff);
+    p->d_in_aff = nullptr;
     p->d_wpk = p->d_bias = p->d_ws = nullptr;
     p->d_ctr = nullptr;
 }
@@ -208,6 +212,26 @@ int tdc_conv_plan_set_weights(tdc_conv_plan *plan, const float *w_oihw, const fl
     return TDC_OK;
 }
 
+int tdc_conv_plan_set_input_affine(tdc_conv_plan *plan, const float *scale, const float *shift, int32_t relu) {
+    if (!plan || !scale || !shift) return fail(TDC_ERR_INVALID, "null argument");
+    const tdc_conv_desc &d = plan->desc;
+    if (d.KH != 1 || d.KW != 1 || d.pad != 0)
+        return fail(TDC_ERR_UNSUPPORTED, "an input affine can only be fused into a 1x1 convolution without padding");
+    const int cch = plan->tile.cch, nchunks = plan->geo.nchunks;
+    const size_t n = (size_t)nchunks * 2 * cch;
+    std::vector<float> packed(n, 0.0f);   // channels past C: 0*x + 0
+    for (int c = 0; c < d.C; ++c) {
+        packed[(size_t)(c / cch) * 2 * cch + c % cch] = scale[c];
+        packed[(size_t)(c / cch) * 2 * cch + cch + c % cch] = shift[c];
+    }
+    hipError_t e = hipSuccess;
+    if (!plan->d_in_aff) e = hipMalloc((void **)&plan->d_in_aff, n * sizeof(float));
+    if (e == hipSuccess) e = hipMemcpy(plan->d_in_aff, packed.data(), n * sizeof(float), hipMemcpyHostToDevice);
+    if (e != hipSuccess) return hip_fail("input affine upload", e);
+    plan->in_relu = relu != 0;
+    return TDC_OK;
+}
+
 int tdc_conv_plan_query(const tdc_conv_plan *plan, tdc_tile_info *info_out) {
     if (!plan || !info_out) return fail(TDC_ERR_INVALID, "null argument");
     *info_out = plan->info;
@@ -237,6 +261,8 @@ int tdc_conv_forward_strided(tdc_conv_plan *plan, const float *d_in, int64_t in_
     kp.resid = d_residual;
     kp.out = d_out;
     kp.ws = plan->d_ws;
+    kp.in_aff = plan->d_in_aff;
+    kp.in_relu = plan->in_relu;
     kp.ctr = plan->d_ctr;
     kp.in_image_bytes = (unsigned)(in_image * 4);
     kp.in_bstride = in_batch_stride ? in_batch_stride : in_image;

@@ -50,6 +50,7 @@ struct Geometry {
     int CS = 0;                      // LDS channel stride (floats)
     int in_stage_floats = 0;         // cch * CS, rounded up to 4
     int wslab_floats = 0;            // weights of one pass of one channel tile
+    int aff_floats = 0;              // room for the scale/shift of an input affine (1x1 convolutions without padding)
     int stage_floats = 0;
     int nstage = 1;
     int lds_bytes = 0;
@@ -97,6 +98,7 @@ struct ConvKParams {
     const float *wpk;
     const float *bias;
     const float *resid;
+    const float *in_aff;       // optional per-input-channel affine in front of a 1x1 convolution: [pass][scale(CCH) | shift(CCH)]
     float *out;
     float *ws;                 // partial tiles of a split across workgroups: [image][slice][N][P]
     unsigned *ctr;             // one ticket counter per (image, channel tile, pixel tile), zero between launches
@@ -115,6 +117,7 @@ struct ConvKParams {
     int RS, CS, VW, nrows;
     int in_stage_floats, wslab_floats, stage_floats, nstage;
     int relu;
+    int in_relu;               // ReLU after the input affine
     FastDiv fd_csv, fd_rsv;      // LDS channel slot / row, in copy elements
     FastDiv fd_tw, fd_ntx, fd_pt;
     FastDiv fd_wk, fd_wn, fd_ks;

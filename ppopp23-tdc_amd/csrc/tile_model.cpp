@@ -175,7 +175,8 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
     // a stage are rounded up to that, the slack receiving zeros.
     g.in_stage_floats = round_up(t.cch * g.CS, 256);
     g.wslab_floats = (t.wm * t.mb) * (t.cch / g.kc) * g.taps * 64;
-    g.stage_floats = g.in_stage_floats + round_up(g.wslab_floats, 256);
+    g.aff_floats = (d.KH == 1 && d.KW == 1 && d.pad == 0) ? round_up(2 * t.cch, 256) : 0;
+    g.stage_floats = g.in_stage_floats + round_up(g.wslab_floats, 256) + g.aff_floats;
     g.nstage = g.cps > 1 ? 2 : 1;
     const long long stage_bytes = (long long)g.nstage * g.stage_floats * 4;
     const long long red_bytes = t.wk > 1 ? (long long)t.wk * g.MT * g.PT * 4 : 0;

@@ -60,6 +60,14 @@ class Conv2dPlan:
                                               c_void_p(b.data_ptr()) if b is not None else None))
         return self
 
+    def set_input_affine(self, scale, shift, relu=True):
+        """y = conv(relu?(x * scale[c] + shift[c])) in one kernel (1x1 convolutions without padding only)."""
+        sc, sh = _host_f32(scale), _host_f32(shift)
+        if sc.numel() != self.desc.C or sh.numel() != self.desc.C:
+            raise ValueError(f"scale and shift must have {self.desc.C} elements")
+        check(lib().tdc_conv_plan_set_input_affine(self._h, c_void_p(sc.data_ptr()), c_void_p(sh.data_ptr()), int(relu)))
+        return self
+
     def forward(self, x, residual=None, out=None):
         d = self.desc
         _dev_check(x, (d.batch, d.C, d.H, d.W), "input")

@@ -59,6 +59,16 @@ class Net:
                                  int(relu), dst, byref(out)))
         return out.value
 
+    def affine_conv(self, x, scale, shift, weight, bias=None, affine_relu=True, residual=-1, relu=False, dst=-1):
+        """relu?(x*scale+shift) followed by a 1x1 convolution, in one kernel."""
+        sc, sh, w, b = _h(scale), _h(shift), _h(weight), _h(bias)
+        out = c_int32()
+        _, C, H, W = self.shape(x)
+        self.conv_shapes.append((C, w.shape[0], H, W, 1, 1, 0))
+        check(lib().tdc_net_affine_conv(self._h, x, _p(sc), _p(sh), int(affine_relu), w.shape[0], _p(w), _p(b), residual,
+                                        int(relu), dst, byref(out)))
+        return out.value
+
     def tkconv(self, x, first, core, last, bias=None, stride=1, pad=0, residual=-1, relu=False, dst=-1):
         f, c, l, b = _h(first), _h(core), _h(last), _h(bias)
         out = c_int32()
@@ -280,17 +290,16 @@ def build_tucker_densenet121(params, batch=1, H=224, W=224, growth=32):
         for l in range(1, nl + 1):
             pre = f"features.denseblock{b}.denselayer{l}"
             s1, t1 = bn_scale_shift(p, pre + ".norm1")
-            y = net.affine(net.view(cat, 0, c), s1, t1, relu=True)                 # norm1 + relu on the concatenation
             s2, t2 = bn_scale_shift(p, pre + ".norm2")
-            y = net.conv(y, fold_dense(p[pre + ".conv1.weight"], s2), t2, relu=True)   # conv1 + norm2 + relu
+            # norm1 + relu on the concatenation, conv1, norm2 + relu: one kernel
+            y = net.affine_conv(net.view(cat, 0, c), s1, t1, fold_dense(p[pre + ".conv1.weight"], s2), t2, relu=True)
             net.tkconv(y, p[pre + ".conv2.first_kernel"], p[pre + ".conv2.core_kernel"], p[pre + ".conv2.last_kernel"],
                        pad=1, dst=net.view(cat, c, growth))
             c += growth
         if b < len(DENSENET121_BLOCKS):
             pre = f"features.transition{b}"
             st, tt = bn_scale_shift(p, pre + ".norm")
-            y = net.affine(cat, st, tt, relu=True)
-            y = net.conv(y, p[pre + ".conv.weight"])
+            y = net.affine_conv(cat, st, tt, p[pre + ".conv.weight"])
             c //= 2
             h, w = h // 2, w // 2
             cat = net.tensor(c + DENSENET121_BLOCKS[b] * growth, h, w)

@@ -186,6 +186,42 @@ def test_both_logical_workgroup_orders(order, monkeypatch):
             assert_close(run_conv(x, w, stride=stride, pad=K // 2, tile=t), want, f"order {order} {t}")
 
 
+@pytest.mark.parametrize("shape", [(1, 40, 24, 9, 9, 1), (2, 100, 36, 14, 14, 1), (1, 7, 5, 5, 6, 1), (2, 16, 8, 9, 9, 2)])
+@pytest.mark.parametrize("relu_in", [True, False])
+def test_input_affine_fused_into_1x1(shape, relu_in):
+    """conv1x1(relu?(x*scale[c] + shift[c])): the norm -> relu -> conv order of the reference's DenseNet layers,
+    as one kernel; every tile (multi-pass ones, loaders, split-K) against the C oracle on the transformed input."""
+    B, C, N, H, W, stride = shape
+    x, w = case(9000 + C + N, B, C, N, H, W, 1)
+    g = seeded(9001)
+    scale = torch.rand(C, generator=g) * 2 - 0.5
+    shift = torch.randn(C, generator=g) * 0.3
+    bias = torch.randn(N, generator=g)
+    xt = x * scale.view(1, C, 1, 1) + shift.view(1, C, 1, 1)
+    if relu_in:
+        xt = xt.clamp_min(0)
+    want = ref.conv2d_c(xt.numpy(), w.numpy(), bias.numpy(), stride=stride, relu=True)
+    tiles = tdc_amd.model_enumerate(tdc_amd.conv_desc(B, C, N, H, W, 1, 1, stride, 0))
+    xd = x.cuda()
+    for t in tiles[::max(1, len(tiles) // 60)]:
+        announce("affine-in", shape, relu_in, t)
+        plan = tdc_amd.Conv2dPlan(B, C, N, H, W, 1, 1, stride, 0, 1, True, True, tile=t).set_weights(w, bias)
+        plan.set_input_affine(scale, shift, relu=relu_in)
+        out = torch.full((B, N, plan.Ho, plan.Wo), float("nan"), device="cuda")
+        plan.forward(xd, out=out)
+        torch.cuda.synchronize()
+        plan.close()
+        assert_close(out.cpu().numpy(), want, f"input affine {shape} {t}")
+
+
+def test_input_affine_is_refused_where_padding_would_have_to_stay_zero():
+    plan = tdc_amd.Conv2dPlan(1, 8, 8, 9, 9, 3, 3, 1, 1)
+    with pytest.raises(tdc_amd.TdcError) as e:
+        plan.set_input_affine(torch.ones(8), torch.zeros(8))
+    assert e.value.status == tdc_amd._lib.TDC_ERR_UNSUPPORTED
+    plan.close()
+
+
 def test_plans_sharing_a_kernel_keep_their_large_lds_requests():
     """Two plans on the same kernel instantiation, both above the 64 KiB default of dynamic LDS, the second asking
     for less: the first must still launch (the opt-in attribute is per function, not per plan)."""
