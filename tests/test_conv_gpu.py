@@ -96,6 +96,36 @@ def test_general_filters(K, stride, pad, dil):
         assert_close(run_conv(x, w, stride=stride, pad=pad, dil=dil, tile=t), want, f"K{K} s{stride} p{pad} d{dil} {t}")
 
 
+def test_random_shapes_model_tile():
+    """Forty seeded random problems (ragged sizes, batch, stride, padding, dilation, rectangular images, every
+    epilogue combination) with the tile the model picks, against F.conv2d on the host."""
+    rng = np.random.default_rng(20240607)
+    done = 0
+    while done < 40:
+        B = int(rng.integers(1, 4)); C = int(rng.integers(1, 70)); N = int(rng.integers(1, 70))
+        H = int(rng.integers(1, 40)); W = int(rng.integers(1, 40))
+        K = int(rng.choice([1, 1, 3, 3, 3, 5, 2, 7])); stride = int(rng.integers(1, 4)); dil = int(rng.integers(1, 3))
+        pad = int(rng.integers(0, K + 1))
+        if H + 2 * pad < dil * (K - 1) + 1 or W + 2 * pad < dil * (K - 1) + 1:
+            continue
+        use_bias, use_res, relu = bool(rng.integers(0, 2)), bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+        announce("random", done, B, C, N, H, W, K, stride, pad, dil, use_bias, use_res, relu)
+        x, w = case(int(rng.integers(1, 1 << 30)), B, C, N, H, W, K)
+        g = seeded(done)
+        bias = torch.randn(N, generator=g) if use_bias else None
+        want = ref.conv2d_torch(x, w, stride=stride, pad=pad, dil=dil)
+        if use_bias:
+            want = want + bias.view(1, N, 1, 1)
+        resid = torch.randn(want.shape, generator=g) if use_res else None
+        if use_res:
+            want = want + resid
+        if relu:
+            want = want.clamp_min(0)
+        got = run_conv(x, w, bias, resid, stride=stride, pad=pad, dil=dil, relu=relu)
+        assert_close(got, want.numpy(), f"random case {done}")
+        done += 1
+
+
 def test_stride2_resnet_core_shapes():
     """The three stride-2 core convs of Tucker ResNet-18 (64->64 56->28, 128->128 28->14, 256->256 14->7)."""
     for r, hw in ((64, 56), (128, 28), (256, 14)):
