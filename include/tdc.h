@@ -112,6 +112,17 @@ int tdc_conv_plan_create(const tdc_conv_desc *desc, const tdc_tile *forced_tile,
                          tdc_conv_plan **plan_out);
 /* Host OIHW weights [N,C,KH,KW]; bias [N] or NULL (must match has_bias). */
 int tdc_conv_plan_set_weights(tdc_conv_plan *plan, const float *w_oihw, const float *bias);
+/* A convolution with a 1x1 convolution fused behind it in the same kernel:
+ *     out = relu2?( W_tail * relu1?(conv(x) + bias) + bias_tail + residual ),   W_tail: [tail_N, desc->N]
+ * where bias / relu1 are desc->has_bias / desc->relu.  The intermediate never leaves the compute unit.  This is the
+ * core convolution of the reference's TKConv2dC with its last factor (inference/TKConv.py:92-94), or a bottleneck
+ * convolution with the first factor of the Tucker convolution that follows it.  One workgroup must own every output
+ * channel of the convolution, which limits desc->N to 256 and suits small N; out / residual are
+ * [batch, tail_N, Ho, Wo].  tail_N == 0 is tdc_conv_plan_create. */
+int tdc_conv_plan_create_with_tail(const tdc_conv_desc *desc, int32_t tail_N, int32_t tail_has_bias, int32_t tail_relu,
+                                   const tdc_tile *forced_tile, tdc_conv_plan **plan_out);
+/* Host [tail_N, desc->N] weights of the tail and its bias [tail_N] or NULL (must match tail_has_bias). */
+int tdc_conv_plan_set_tail_weights(tdc_conv_plan *plan, const float *w_tail, const float *bias_tail);
 /* Optional, 1x1 convolutions without padding only: y = conv(relu?(x * scale[c] + shift[c])) in one kernel —
  * the norm -> relu -> conv order of the reference's DenseNet layers (inference/densenet_inet_tt.py:36-69), where the
  * BatchNorm sits in front of the convolution and cannot be folded into its weights.  Host arrays of C floats. */

@@ -625,6 +625,96 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
         if (p.relu) val = fmaxf(val, 0.0f);
         out[o] = val;
     };
+    if (p.tail_w) {
+        // Fused tail: a 1x1 convolution over the output channels of this one, out2 = W2 * act(conv + bias), in the
+        // same kernel (the last factor of a Tucker convolution behind its core, or the first factor of the next one
+        // behind a bottleneck convolution).  The workgroup owns ALL output channels of the convolution (the host
+        // guarantees one channel tile and no split across workgroups).  Its tile is parked in LDS as
+        // f[channel][pixel lane] — the B operand of a second, small MFMA GEMM whose A operand is the tail's packed
+        // weights — and the 16x16 output blocks of that GEMM are dealt to all waves.
+        float *f = lds + p.tail_f_off;
+        const int LD = p.tail_ld;
+        if (p.WK == 1) {
+            __syncthreads();  // slower waves may still be reading the last stage
+            if (!loader) {
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb) {
+#pragma unroll
+                    for (int v = 0; v < NACC; ++v) {
+                        const int ml = (wm * MB + mb) * MF + M::row(v, lane);
+                        const float b1 = (p.bias && ml < p.N) ? p.bias[ml] : 0.0f;
+#pragma unroll
+                        for (int nb = 0; nb < NB; ++nb) {
+                            float val = acc[mb][nb][v] + b1;
+                            if (p.relu) val = fmaxf(val, 0.0f);
+                            f[ml * LD + (wn * NB + nb) * MF + M::col(lane)] = val;
+                        }
+                    }
+                }
+            }
+        } else {
+            const int total = MT * PT;
+            for (int idx = tid; idx < total; idx += nthreads) {
+                const int ml = fdiv(idx, p.fd_pt);
+                const int pl = idx - ml * PT;
+                float val = 0.0f;
+                for (int k0 = 0; k0 < p.WK; k0 += 4) {
+                    float part[4];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) part[u] = lds[min(k0 + u, p.WK - 1) * total + idx];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u)
+                        if (k0 + u < p.WK) val += part[u];
+                }
+                if (p.bias && ml < p.N) val += p.bias[ml];
+                if (p.relu) val = fmaxf(val, 0.0f);
+                f[ml * LD + pl] = val;
+            }
+        }
+        __syncthreads();
+        const int npx = PT >> 4;                  // 16-pixel blocks of the tile
+        const int nblk = p.tail_mblk * npx;       // 16x16 output blocks
+        const int ksub16 = lane >> 4, px16 = lane & 15;
+        for (int blk = wave; blk < nblk; blk += nwaves) {
+            const int mblk = fdiv(blk, p.fd_npx);
+            const int pxblk = blk - mblk * npx;
+            const float *wa = p.tail_w + (size_t)mblk * p.tail_ng * 64 + lane;
+            const float *fb = f + ksub16 * LD + pxblk * 16 + px16;
+            f4_t acc2 = {0.0f, 0.0f, 0.0f, 0.0f};
+            for (int g0 = 0; g0 < p.tail_ng; g0 += 4) {
+                float a[4], b[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const int g = min(g0 + u, p.tail_ng - 1);
+                    a[u] = wa[g * 64];
+                    b[u] = fb[g * 4 * LD];
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u)
+                    if (g0 + u < p.tail_ng) acc2 = __builtin_amdgcn_mfma_f32_16x16x4f32(a[u], b[u], acc2, 0, 0, 0);
+            }
+            const int j = pxblk * 16 + px16;
+            const int jy = fdiv(j, p.fd_tw);
+            const int jx = j - jy * p.TW;
+            const int oy = oy0 + jy, ox = ox0 + jx;
+            if (jy < p.TH && oy < p.Ho && ox < p.Wo) {
+                const int pp = oy * p.Wo + ox;
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const int n2 = mblk * 16 + 4 * ksub16 + v;
+                    if (n2 < p.tail_N) {
+                        float val = acc2[v];
+                        if (p.tail_bias) val += p.tail_bias[n2];
+                        const long long o = (long long)n2 * p.P + pp;
+                        if (resid) val += resid[o];
+                        if (p.tail_relu) val = fmaxf(val, 0.0f);
+                        out[o] = val;
+                    }
+                }
+            }
+        }
+        return;
+    }
     if (p.KS == 1) {
         each_output(finish, true);
         return;

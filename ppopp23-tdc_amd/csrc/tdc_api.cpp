@@ -46,6 +46,10 @@ struct tdc_conv_plan {
     float *d_ws = nullptr;        // tile.ks > 1: partial tiles [batch][ks][N][P]
     unsigned *d_ctr = nullptr;    // tile.ks > 1: ticket counters, zero between launches
     float *d_in_aff = nullptr;    // optional input affine: [pass][scale(cch) | shift(cch)]
+    int tail_N = 0;               // fused 1x1 tail (0 = none): outputs, epilogue flags, packed weights
+    int tail_has_bias = 0, tail_relu = 0;
+    float *d_tail_w = nullptr, *d_tail_bias = nullptr;
+    bool have_tail_weights = false;
     int in_relu = 0;
     bool have_weights = false;
 };
@@ -56,7 +60,9 @@ static void free_plan_buffers(tdc_conv_plan *p) {
     if (p->d_ws) (void)hipFree(p->d_ws);
     if (p->d_ctr) (void)hipFree(p->d_ctr);
     if (p->d_in_aff) (void)hipFree(p->d_in_aff);
-    p->d_in_aff = nullptr;
+    if (p->d_tail_w) (void)hipFree(p->d_tail_w);
+    if (p->d_tail_bias) (void)hipFree(p->d_tail_bias);
+    p->d_in_aff = p->d_tail_w = p->d_tail_bias = nullptr;
     p->d_wpk = p->d_bias = p->d_ws = nullptr;
     p->d_ctr = nullptr;
 }
@@ -143,7 +149,13 @@ int tdc_model_set_constants(const double *values, int32_t count) {
 }
 
 int tdc_conv_plan_create(const tdc_conv_desc *desc, const tdc_tile *forced_tile, tdc_conv_plan **plan_out) {
+    return tdc_conv_plan_create_with_tail(desc, 0, 0, 0, forced_tile, plan_out);
+}
+
+int tdc_conv_plan_create_with_tail(const tdc_conv_desc *desc, int32_t tail_N, int32_t tail_has_bias, int32_t tail_relu,
+                                   const tdc_tile *forced_tile, tdc_conv_plan **plan_out) {
     if (!desc || !plan_out) return fail(TDC_ERR_INVALID, "null argument");
+    if (tail_N < 0) return fail(TDC_ERR_INVALID, "tail_N must be >= 0");
     *plan_out = nullptr;
     std::string why;
     if (!check_desc(*desc, &why)) return fail(TDC_ERR_INVALID, why);
@@ -154,13 +166,16 @@ int tdc_conv_plan_create(const tdc_conv_desc *desc, const tdc_tile *forced_tile,
     std::unique_ptr<tdc_conv_plan> p(new (std::nothrow) tdc_conv_plan());
     if (!p) return fail(TDC_ERR_NOMEM, "out of host memory");
     p->desc = *desc;
+    p->tail_N = tail_N;
+    p->tail_has_bias = tail_N > 0 && tail_has_bias;
+    p->tail_relu = tail_N > 0 && tail_relu;
     if (forced_tile) {
-        if (!model_evaluate(*desc, *forced_tile, p->info, &why)) return fail(TDC_ERR_INVALID, "forced tile: " + why);
+        if (!model_evaluate(*desc, *forced_tile, p->info, &why, tail_N)) return fail(TDC_ERR_INVALID, "forced tile: " + why);
     } else {
-        if (!model_select(*desc, p->info, &why)) return fail(TDC_ERR_UNSUPPORTED, why);
+        if (!model_select(*desc, p->info, &why, tail_N)) return fail(TDC_ERR_UNSUPPORTED, why);
     }
     p->tile = p->info.tile;
-    if (!make_geometry(*desc, p->tile, p->geo, &why)) return fail(TDC_ERR_INVALID, why);
+    if (!make_geometry(*desc, p->tile, p->geo, &why, tail_N)) return fail(TDC_ERR_INVALID, why);
     p->kernel = conv_kernel_for(p->tile, desc->KH, desc->KW, desc->dilation);
     if (!p->kernel) return fail(TDC_ERR_UNSUPPORTED, "no kernel instantiated for this tile");
     int he = prepare_conv_kernel(p->kernel, p->geo);
@@ -173,6 +188,15 @@ int tdc_conv_plan_create(const tdc_conv_desc *desc, const tdc_tile *forced_tile,
         if (e != hipSuccess) {
             free_plan_buffers(p.get());
             return hip_fail("hipMalloc(bias)", e);
+        }
+    }
+    if (tail_N > 0) {
+        const size_t tw = (size_t)((tail_N + 15) / 16) * p->geo.tail_ng * 64;
+        e = hipMalloc((void **)&p->d_tail_w, tw * sizeof(float));
+        if (e == hipSuccess && p->tail_has_bias) e = hipMalloc((void **)&p->d_tail_bias, (size_t)tail_N * sizeof(float));
+        if (e != hipSuccess) {
+            free_plan_buffers(p.get());
+            return hip_fail("hipMalloc(tail weights)", e);
         }
     }
     if (p->tile.ks > 1) {
@@ -212,6 +236,28 @@ int tdc_conv_plan_set_weights(tdc_conv_plan *plan, const float *w_oihw, const fl
     return TDC_OK;
 }
 
+int tdc_conv_plan_set_tail_weights(tdc_conv_plan *plan, const float *w_tail, const float *bias_tail) {
+    if (!plan || !w_tail) return fail(TDC_ERR_INVALID, "null argument");
+    if (plan->tail_N <= 0) return fail(TDC_ERR_STATE, "this plan was created without a fused tail");
+    if ((plan->tail_has_bias != 0) != (bias_tail != nullptr))
+        return fail(TDC_ERR_INVALID, "tail bias pointer does not match the plan");
+    // [16-row block][K-step][64 lanes] in MFMA A order: lane l of an entry holds w_tail[block*16 + l%16][4*kstep + l/16].
+    const int N = plan->desc.N, N2 = plan->tail_N, ng = plan->geo.tail_ng, mblk = (N2 + 15) / 16;
+    std::vector<float> packed((size_t)mblk * ng * 64, 0.0f);
+    for (int mb = 0; mb < mblk; ++mb)
+        for (int g = 0; g < ng; ++g)
+            for (int l = 0; l < 64; ++l) {
+                const int n2 = mb * 16 + l % 16, c = 4 * g + l / 16;
+                if (n2 < N2 && c < N) packed[((size_t)mb * ng + g) * 64 + l] = w_tail[(size_t)n2 * N + c];
+            }
+    hipError_t e = hipMemcpy(plan->d_tail_w, packed.data(), packed.size() * sizeof(float), hipMemcpyHostToDevice);
+    if (e == hipSuccess && bias_tail)
+        e = hipMemcpy(plan->d_tail_bias, bias_tail, (size_t)N2 * sizeof(float), hipMemcpyHostToDevice);
+    if (e != hipSuccess) return hip_fail("hipMemcpy(tail weights)", e);
+    plan->have_tail_weights = true;
+    return TDC_OK;
+}
+
 int tdc_conv_plan_set_input_affine(tdc_conv_plan *plan, const float *scale, const float *shift, int32_t relu) {
     if (!plan || !scale || !shift) return fail(TDC_ERR_INVALID, "null argument");
     const tdc_conv_desc &d = plan->desc;
@@ -248,9 +294,12 @@ int tdc_conv_forward_strided(tdc_conv_plan *plan, const float *d_in, int64_t in_
     if (in_batch_stride < 0 || out_batch_stride < 0 || residual_batch_stride < 0)
         return fail(TDC_ERR_INVALID, "negative batch stride");
     if (!plan->have_weights) return fail(TDC_ERR_STATE, "tdc_conv_forward before tdc_conv_plan_set_weights");
+    if (plan->tail_N > 0 && !plan->have_tail_weights)
+        return fail(TDC_ERR_STATE, "tdc_conv_forward before tdc_conv_plan_set_tail_weights");
     const tdc_conv_desc &d = plan->desc;
     const Geometry &g = plan->geo;
-    const long long in_image = (long long)d.C * d.H * d.W, out_image = (long long)d.N * g.P;
+    const long long in_image = (long long)d.C * d.H * d.W;
+    const long long out_image = (long long)(plan->tail_N > 0 ? plan->tail_N : d.N) * g.P;
     if ((in_batch_stride && in_batch_stride < in_image) || (out_batch_stride && out_batch_stride < out_image) ||
         (residual_batch_stride && residual_batch_stride < out_image))
         return fail(TDC_ERR_INVALID, "batch stride smaller than one image");
@@ -262,6 +311,11 @@ int tdc_conv_forward_strided(tdc_conv_plan *plan, const float *d_in, int64_t in_
     kp.out = d_out;
     kp.ws = plan->d_ws;
     kp.in_aff = plan->d_in_aff;
+    kp.tail_w = plan->tail_N > 0 ? plan->d_tail_w : nullptr;
+    kp.tail_bias = plan->d_tail_bias;
+    kp.tail_N = plan->tail_N; kp.tail_mblk = (plan->tail_N + 15) / 16; kp.tail_ng = g.tail_ng; kp.tail_relu = plan->tail_relu;
+    kp.tail_ld = g.tail_ld; kp.tail_f_off = g.tail_f_off;
+    kp.fd_npx = make_fastdiv(g.PT / 16);
     kp.in_relu = plan->in_relu;
     kp.ctr = plan->d_ctr;
     kp.in_image_bytes = (unsigned)(in_image * 4);

@@ -51,6 +51,7 @@ struct Geometry {
     int in_stage_floats = 0;         // cch * CS, rounded up to 4
     int wslab_floats = 0;            // weights of one pass of one channel tile
     int aff_floats = 0;              // room for the scale/shift of an input affine (1x1 convolutions without padding)
+    int tail_N = 0, tail_ng = 0, tail_ld = 0, tail_f_off = 0;   // fused 1x1 tail (0 = none)
     int stage_floats = 0;
     int nstage = 1;
     int lds_bytes = 0;
@@ -60,12 +61,14 @@ struct Geometry {
 };
 
 // Returns false (and a reason) when the tile cannot be launched for this shape.
-bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::string *why);
+// tail_N > 0: a 1x1 convolution with tail_N outputs is fused behind this one (needs one channel tile, no split
+// across workgroups).
+bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::string *why, int tail_N = 0);
 bool check_desc(const tdc_conv_desc &d, std::string *why);
 
-bool model_evaluate(const tdc_conv_desc &d, const tdc_tile &t, tdc_tile_info &info, std::string *why);
-std::vector<tdc_tile> model_enumerate(const tdc_conv_desc &d);
-bool model_select(const tdc_conv_desc &d, tdc_tile_info &info, std::string *why);
+bool model_evaluate(const tdc_conv_desc &d, const tdc_tile &t, tdc_tile_info &info, std::string *why, int tail_N = 0);
+std::vector<tdc_tile> model_enumerate(const tdc_conv_desc &d, int tail_N = 0);
+bool model_select(const tdc_conv_desc &d, tdc_tile_info &info, std::string *why, int tail_N = 0);
 int model_constants(double *out, int cap);            // returns the number of constants
 bool model_set_constants(const double *in, int n);
 
@@ -99,6 +102,8 @@ struct ConvKParams {
     const float *bias;
     const float *resid;
     const float *in_aff;       // optional per-input-channel affine in front of a 1x1 convolution: [pass][scale(CCH) | shift(CCH)]
+    const float *tail_w;       // fused 1x1 tail: packed weights [16-row block][K-step][64 lanes], or null
+    const float *tail_bias;
     float *out;
     float *ws;                 // partial tiles of a split across workgroups: [image][slice][N][P]
     unsigned *ctr;             // one ticket counter per (image, channel tile, pixel tile), zero between launches
@@ -118,6 +123,9 @@ struct ConvKParams {
     int in_stage_floats, wslab_floats, stage_floats, nstage;
     int relu;
     int in_relu;               // ReLU after the input affine
+    int tail_N, tail_mblk, tail_ng, tail_relu;   // tail outputs, their 16-row blocks, K-steps (ceil(N/4)), ReLU after it
+    int tail_ld, tail_f_off;   // row stride and offset (floats) of the parked tile in LDS
+    FastDiv fd_npx;            // 16-pixel blocks per tile
     FastDiv fd_csv, fd_rsv;      // LDS channel slot / row, in copy elements
     FastDiv fd_tw, fd_ntx, fd_pt;
     FastDiv fd_wk, fd_wn, fd_ks;

@@ -104,7 +104,7 @@ static int pad_channel_stride(int raw, int mf, int vw, int PT, int TW, int TH, i
     return hit->second.first;
 }
 
-bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::string *why) {
+bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::string *why, int tail_N) {
     auto fail = [&](const std::string &m) {
         if (why) *why = m;
         return false;
@@ -180,7 +180,20 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
     g.nstage = g.cps > 1 ? 2 : 1;
     const long long stage_bytes = (long long)g.nstage * g.stage_floats * 4;
     const long long red_bytes = t.wk > 1 ? (long long)t.wk * g.MT * g.PT * 4 : 0;
-    const long long lds = std::max(stage_bytes, red_bytes);
+    long long lds = std::max(stage_bytes, red_bytes);
+    if (tail_N > 0) {
+        // A fused 1x1 tail needs every output channel of the convolution in one workgroup; its tile is parked
+        // in LDS behind the split-K partials with a row stride that keeps the four channel quarters of a
+        // K-step in different banks.
+        if (tail_N > 4096) return fail("fused tail too wide");
+        if (g.grid_y != 1) return fail("a fused tail needs all output channels in one workgroup tile");
+        if (t.ks != 1) return fail("a fused tail cannot be combined with a split across workgroups");
+        g.tail_N = tail_N;
+        g.tail_ng = ceil_div(d.N, 4);
+        g.tail_ld = (g.PT % 32 == 0) ? g.PT + 16 : g.PT;
+        g.tail_f_off = t.wk > 1 ? t.wk * g.MT * g.PT : 0;
+        lds = std::max(lds, ((long long)g.tail_f_off + (long long)g.MT * g.tail_ld) * 4);
+    }
     if (lds > machine().lds_bytes_per_cu) return fail("tile needs more than 160 KiB of LDS");
     g.lds_bytes = (int)lds;
     if (const char *e = std::getenv("TDC_EXPERIMENT_MIN_LDS")) g.lds_bytes = std::max(g.lds_bytes, std::atoi(e));
@@ -280,9 +293,9 @@ int kernel_vgprs(const tdc_tile &t, int taps_mode) {
 
 }  // namespace
 
-bool model_evaluate(const tdc_conv_desc &d, const tdc_tile &t, tdc_tile_info &info, std::string *why) {
+bool model_evaluate(const tdc_conv_desc &d, const tdc_tile &t, tdc_tile_info &info, std::string *why, int tail_N) {
     Geometry g;
-    if (!make_geometry(d, t, g, why)) return false;
+    if (!make_geometry(d, t, g, why, tail_N)) return false;
     const Machine &m = machine();
     std::memset(&info, 0, sizeof(info));
     info.tile = t;
@@ -314,6 +327,10 @@ bool model_evaluate(const tdc_conv_desc &d, const tdc_tile &t, tdc_tile_info &in
     info.flops = 2.0 * P * d.C * d.N * g.taps * d.batch;
     info.bytes = 4.0 * ((double)d.batch * ((double)d.C * d.H * d.W + (double)d.N * P) +
                         (double)g.taps * d.C * d.N);
+    if (tail_N > 0) {   // the intermediate never leaves the chip
+        info.flops += 2.0 * P * d.N * tail_N * d.batch;
+        info.bytes += 4.0 * ((double)d.batch * ((double)tail_N - d.N) * P + (double)d.N * tail_N);
+    }
     info.roof_us = std::max(info.bytes / (m.hbm_tbps * 1e6), info.flops / (m.fp32_tflops * 1e6));
 
     // --- per-workgroup costs (clock cycles of one CU) ------------------------
@@ -368,6 +385,14 @@ bool model_evaluate(const tdc_conv_desc &d, const tdc_tile &t, tdc_tile_info &in
         if (t.ks > 1)
             clk += MC.ksplit_clk + MC.copy_latency_clk + (double)t.ks * out_bytes / rate +
                    out_bytes / MC.store_bytes_per_clk;
+        // Fused tail: park the tile, one more barrier, the first touch of the tail's weights, then the 16x16
+        // blocks of the small GEMM dealt over the waves, and the tail's own store.
+        if (tail_N > 0) {
+            const double blocks = std::ceil((double)ceil_div(tail_N, 16) * (g.PT / 16) / g.waves);
+            clk += out_bytes * r / MC.lds_bytes_per_clk + MC.sync_clk + MC.copy_latency_clk +
+                   blocks * (g.tail_ng * 32.0 + 64.0) * r + (double)tail_N * g.PT * 4.0 * r / MC.store_bytes_per_clk -
+                   out_bytes * r / MC.store_bytes_per_clk;
+        }
         return clk;
     };
     const long long slots = (long long)m.cus * wg_per_cu;
@@ -380,7 +405,7 @@ bool model_evaluate(const tdc_conv_desc &d, const tdc_tile &t, tdc_tile_info &in
     return true;
 }
 
-std::vector<tdc_tile> model_enumerate(const tdc_conv_desc &d) {
+std::vector<tdc_tile> model_enumerate(const tdc_conv_desc &d, int tail_N) {
     std::vector<tdc_tile> out;
     if (!check_desc(d, nullptr)) return out;
     const bool flat = (d.KH == 1 && d.KW == 1 && d.stride == 1 && d.pad == 0);
@@ -437,7 +462,7 @@ std::vector<tdc_tile> model_enumerate(const tdc_conv_desc &d) {
                                         for (int wl : {0, 1, 2, 4}) {
                                             tdc_tile t{mf, mb, nb, wm, wn, wk, cch, tw, ks, wl};
                                             Geometry g;
-                                            if (!make_geometry(d, t, g, nullptr)) continue;
+                                            if (!make_geometry(d, t, g, nullptr, tail_N)) continue;
                                             if (ks > 1 && (long long)g.grid_x * g.grid_y * g.grid_z > max_wgs) continue;
                                             if (wl > 0 && g.cps < 2) continue;  // loaders only work from the second pass on
                                             out.push_back(t);
@@ -460,13 +485,13 @@ bool model_set_constants(const double *in, int n) {
     return true;
 }
 
-bool model_select(const tdc_conv_desc &d, tdc_tile_info &best, std::string *why) {
+bool model_select(const tdc_conv_desc &d, tdc_tile_info &best, std::string *why, int tail_N) {
     if (!check_desc(d, why)) return false;
-    std::vector<tdc_tile> cands = model_enumerate(d);
+    std::vector<tdc_tile> cands = model_enumerate(d, tail_N);
     bool have = false;
     for (const tdc_tile &t : cands) {
         tdc_tile_info info;
-        if (!model_evaluate(d, t, info, nullptr)) continue;
+        if (!model_evaluate(d, t, info, nullptr, tail_N)) continue;
         if (!have || info.pred_us < best.pred_us) {
             best = info;
             have = true;

@@ -38,11 +38,19 @@ class Conv2dPlan:
     = constructor + ``set_weights``; ``forward`` takes/returns device tensors.
     """
 
-    def __init__(self, batch, C, N, H, W, KH, KW, stride=1, pad=0, dilation=1, bias=False, relu=False, tile=None):
+    def __init__(self, batch, C, N, H, W, KH, KW, stride=1, pad=0, dilation=1, bias=False, relu=False, tile=None,
+                 tail=None):
+        """``tail=(tail_N, tail_bias, tail_relu)`` fuses a 1x1 convolution with tail_N outputs behind this one
+        (``bias`` / ``relu`` then act between the two); the output has tail_N channels."""
         self.desc = _lib.conv_desc(batch, C, N, H, W, KH, KW, stride, pad, dilation, bias, relu)
         self._h = c_void_p()
         tptr = byref(tile) if tile is not None else None
-        check(lib().tdc_conv_plan_create(byref(self.desc), tptr, byref(self._h)))
+        self.tail = tail
+        if tail is None:
+            check(lib().tdc_conv_plan_create(byref(self.desc), tptr, byref(self._h)))
+        else:
+            check(lib().tdc_conv_plan_create_with_tail(byref(self.desc), int(tail[0]), int(bool(tail[1])),
+                                                       int(bool(tail[2])), tptr, byref(self._h)))
         self.info = TileInfo()
         check(lib().tdc_conv_plan_query(self._h, byref(self.info)))
         self.Ho = _out_dim(H, KH, stride, pad, dilation)
@@ -60,6 +68,15 @@ class Conv2dPlan:
                                               c_void_p(b.data_ptr()) if b is not None else None))
         return self
 
+    def set_tail_weights(self, weight, bias=None):
+        """Weights [tail_N, N] (or [tail_N, N, 1, 1]) and bias [tail_N] of the fused 1x1 tail."""
+        w, b = _host_f32(weight), _host_f32(bias)
+        if self.tail is None or w.numel() != self.tail[0] * self.desc.N:
+            raise ValueError("tail weight must be [tail_N, N]")
+        check(lib().tdc_conv_plan_set_tail_weights(self._h, c_void_p(w.data_ptr()),
+                                                   c_void_p(b.data_ptr()) if b is not None else None))
+        return self
+
     def set_input_affine(self, scale, shift, relu=True):
         """y = conv(relu?(x * scale[c] + shift[c])) in one kernel (1x1 convolutions without padding only)."""
         sc, sh = _host_f32(scale), _host_f32(shift)
@@ -71,7 +88,7 @@ class Conv2dPlan:
     def forward(self, x, residual=None, out=None):
         d = self.desc
         _dev_check(x, (d.batch, d.C, d.H, d.W), "input")
-        oshape = (d.batch, d.N, self.Ho, self.Wo)
+        oshape = (d.batch, self.tail[0] if self.tail else d.N, self.Ho, self.Wo)
         if out is None:
             out = torch.empty(oshape, device=x.device, dtype=torch.float32)
         else:
@@ -147,7 +164,7 @@ class TKConvOp:
     def forward(self, x, residual=None, out=None):
         d = self.desc
         _dev_check(x, (d.batch, d.C, d.H, d.W), "input")
-        oshape = (d.batch, d.N, self.Ho, self.Wo)
+        oshape = (d.batch, self.tail[0] if self.tail else d.N, self.Ho, self.Wo)
         if out is None:
             out = torch.empty(oshape, device=x.device, dtype=torch.float32)
         else:

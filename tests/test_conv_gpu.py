@@ -244,6 +244,58 @@ def test_input_affine_fused_into_1x1(shape, relu_in):
         assert_close(out.cpu().numpy(), want, f"input affine {shape} {t}")
 
 
+@pytest.mark.parametrize("shape", [(1, 24, 16, 40, 9, 9, 3, 1), (2, 40, 10, 33, 14, 14, 3, 1), (1, 64, 32, 64, 13, 11, 3, 2),
+                                   (2, 50, 64, 24, 7, 7, 1, 1), (1, 20, 128, 64, 9, 9, 1, 1), (1, 12, 7, 5, 6, 5, 5, 1)])
+def test_fused_1x1_tail(shape):
+    """relu(W_tail * relu(conv(x) + b1) + b2 + residual) in one kernel, every tile that can hold all output
+    channels of the convolution in one workgroup, against the two convolutions done one after the other."""
+    B, C, N, N2, H, W, K, stride = shape
+    x, w = case(9500 + C + N, B, C, N, H, W, K)
+    g = seeded(9501 + N2)
+    b1 = torch.randn(N, generator=g) * 0.5
+    w2 = torch.randn(N2, N, 1, 1, generator=g) / math.sqrt(N)
+    b2 = torch.randn(N2, generator=g)
+    mid = ref.conv2d_torch(x, w, b1, stride=stride, pad=K // 2).clamp_min(0)
+    resid = torch.randn(B, N2, mid.shape[2], mid.shape[3], generator=g)
+    want = (ref.conv2d_torch(mid, w2, b2) + resid).clamp_min(0).numpy()
+    want_c = ref.conv2d_c(ref.conv2d_c(x.numpy(), w.numpy(), b1.numpy(), stride=stride, pad=K // 2, relu=True),
+                          w2.numpy(), b2.numpy(), resid.numpy(), relu=True)
+    assert_close(want, want_c, "host references agree")
+    desc = tdc_amd.conv_desc(B, C, N, H, W, K, K, stride, K // 2, 1, True, True)
+    ok = []
+    for t in tdc_amd.model_enumerate(desc):
+        if t.ks == 1 and t.mf * t.mb * t.wm >= N:
+            ok.append(t)
+    assert ok
+    xd, rd = x.cuda(), resid.cuda()
+    ran = 0
+    for t in ok[::max(1, len(ok) // 50)] + [None]:
+        announce("tail", shape, t)
+        try:
+            plan = tdc_amd.Conv2dPlan(B, C, N, H, W, K, K, stride, K // 2, 1, True, True, tile=t, tail=(N2, True, True))
+        except tdc_amd.TdcError as e:     # the parked tile can push a candidate over the LDS limit
+            assert t is not None and "LDS" in str(e), str(e)
+            continue
+        ran += 1
+        plan.set_weights(w, b1).set_tail_weights(w2, b2)
+        out = torch.full((B, N2, plan.Ho, plan.Wo), float("nan"), device="cuda")
+        plan.forward(xd, rd, out=out)
+        torch.cuda.synchronize()
+        plan.close()
+        assert_close(out.cpu().numpy(), want_c, f"fused tail {shape} {t}")
+    assert ran >= 10
+
+
+def test_fused_tail_needs_one_channel_tile():
+    with pytest.raises(tdc_amd.TdcError):   # 40 output channels cannot sit in a 16-channel tile
+        tdc_amd.Conv2dPlan(1, 8, 40, 9, 9, 3, 3, 1, 1, tile=tdc_amd.Tile(16, 1, 1, 1, 1, 1, 8, 8), tail=(8, False, False))
+    plan = tdc_amd.Conv2dPlan(1, 8, 16, 9, 9, 3, 3, 1, 1, tail=(8, False, False)).set_weights(torch.randn(16, 8, 3, 3))
+    with pytest.raises(tdc_amd.TdcError) as e:   # tail weights missing
+        plan.forward(torch.randn(1, 8, 9, 9).cuda())
+    assert e.value.status == tdc_amd._lib.TDC_ERR_STATE
+    plan.close()
+
+
 def test_input_affine_is_refused_where_padding_would_have_to_stay_zero():
     plan = tdc_amd.Conv2dPlan(1, 8, 8, 9, 9, 3, 3, 1, 1)
     with pytest.raises(tdc_amd.TdcError) as e:
