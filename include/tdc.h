@@ -182,6 +182,9 @@ int tdc_tkconv_forward_features(tdc_tkconv *op, const float *d_in, float *d_feat
                                 float *d_feat_core, float *d_out, void *stream);
 /* Only the KxK core conv: d_in is [batch,R1,H,W], d_out [batch,R2,Ho,Wo]. */
 int tdc_tkconv_core_forward(tdc_tkconv *op, const float *d_in, float *d_out, void *stream);
+/* Launches per forward: 3, or 2 when the last factor is fused behind the core convolution (done automatically
+ * when the tile model predicts it faster; TDC_EXPERIMENT_NO_FUSED_TAIL in the environment turns it off). */
+int tdc_tkconv_num_kernels(const tdc_tkconv *op);
 /* which: 0 = first 1x1, 1 = core, 2 = last 1x1 */
 int tdc_tkconv_query(const tdc_tkconv *op, int which, tdc_tile_info *info_out);
 void tdc_tkconv_destroy(tdc_tkconv *op);

@@ -233,7 +233,7 @@ int tdc_net_tkconv(tdc_net *net, int32_t in, int32_t R1, int32_t R2, int32_t N, 
     NetOp op;
     op.kind = NetOp::TKCONV; op.tk = tk; op.in = in; op.out = id; op.resid = residual;
     net->ops.push_back(op);
-    net->kernels += 3;
+    net->kernels += tdc_tkconv_num_kernels(tk);
     *out = id;
     return TDC_OK;
 }

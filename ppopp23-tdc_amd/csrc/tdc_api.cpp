@@ -3,6 +3,7 @@
 #include <hip/hip_runtime_api.h>
 
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <memory>
 #include <new>
@@ -72,6 +73,7 @@ struct tdc_tkconv {
     tdc_conv_plan *first = nullptr;
     tdc_conv_plan *core = nullptr;
     tdc_conv_plan *last = nullptr;
+    tdc_conv_plan *core_last = nullptr;   // core convolution with the last factor fused behind it, when that is faster
     float *d_f1 = nullptr;  // [batch, R1, H, W]
     float *d_f2 = nullptr;  // [batch, R2, Ho, Wo]
     size_t f1_floats = 0, f2_floats = 0;
@@ -484,6 +486,7 @@ int tdc_tkconv_create(const tdc_tkconv_desc *desc, tdc_tkconv **op_out) {
         tdc_conv_plan_destroy(op->first);
         tdc_conv_plan_destroy(op->core);
         tdc_conv_plan_destroy(op->last);
+        tdc_conv_plan_destroy(op->core_last);
         if (op->d_f1) (void)hipFree(op->d_f1);
         if (op->d_f2) (void)hipFree(op->d_f2);
     };
@@ -496,6 +499,17 @@ int tdc_tkconv_create(const tdc_tkconv_desc *desc, tdc_tkconv **op_out) {
     if (e != hipSuccess) { cleanup(); return hip_fail("hipMalloc(first intermediate)", e); }
     e = hipMalloc((void **)&op->d_f2, op->f2_floats * sizeof(float));
     if (e != hipSuccess) { cleanup(); return hip_fail("hipMalloc(core intermediate)", e); }
+    // Core + last factor as one kernel, if the model predicts it faster than the two launches (it needs all R2
+    // channels in one workgroup, so it only pays for small R2).  The three plain plans stay: they serve
+    // forward_features and core_forward.
+    if (!std::getenv("TDC_EXPERIMENT_NO_FUSED_TAIL")) {
+        tdc_tile_info fused{};
+        if (model_select(d2, fused, nullptr, desc->N) &&
+            fused.pred_us < op->core->info.pred_us + op->last->info.pred_us) {
+            st = tdc_conv_plan_create_with_tail(&d2, desc->N, desc->has_bias, desc->relu, nullptr, &op->core_last);
+            if (st != TDC_OK) { cleanup(); return st; }
+        }
+    }
     *op_out = op.release();
     return TDC_OK;
 }
@@ -507,8 +521,22 @@ int tdc_tkconv_set_weights(tdc_tkconv *op, const float *first, const float *core
     if ((st = tdc_conv_plan_set_weights(op->first, first, nullptr)) != TDC_OK) return st;
     if ((st = tdc_conv_plan_set_weights(op->core, core, nullptr)) != TDC_OK) return st;
     if ((st = tdc_conv_plan_set_weights(op->last, last, bias)) != TDC_OK) return st;
+    if (op->core_last) {
+        if ((st = tdc_conv_plan_set_weights(op->core_last, core, nullptr)) != TDC_OK) return st;
+        if ((st = tdc_conv_plan_set_tail_weights(op->core_last, last, bias)) != TDC_OK) return st;
+    }
     return TDC_OK;
 }
+
+static int tkconv_forward_unfused(tdc_tkconv *op, const float *d_in, int64_t in_batch_stride, const float *d_residual,
+                                  int64_t residual_batch_stride, float *d_out, int64_t out_batch_stride, void *stream) {
+    int st;
+    if ((st = tdc_conv_forward_strided(op->first, d_in, in_batch_stride, nullptr, 0, op->d_f1, 0, stream)) != TDC_OK) return st;
+    if ((st = tdc_conv_forward(op->core, op->d_f1, nullptr, op->d_f2, stream)) != TDC_OK) return st;
+    return tdc_conv_forward_strided(op->last, op->d_f2, 0, d_residual, residual_batch_stride, d_out, out_batch_stride, stream);
+}
+
+int tdc_tkconv_num_kernels(const tdc_tkconv *op) { return op ? (op->core_last ? 2 : 3) : 0; }
 
 int tdc_tkconv_forward(tdc_tkconv *op, const float *d_in, const float *d_residual, float *d_out, void *stream) {
     return tdc_tkconv_forward_strided(op, d_in, 0, d_residual, 0, d_out, 0, stream);
@@ -517,15 +545,19 @@ int tdc_tkconv_forward(tdc_tkconv *op, const float *d_in, const float *d_residua
 int tdc_tkconv_forward_strided(tdc_tkconv *op, const float *d_in, int64_t in_batch_stride, const float *d_residual,
                                int64_t residual_batch_stride, float *d_out, int64_t out_batch_stride, void *stream) {
     if (!op || !d_in || !d_out) return fail(TDC_ERR_INVALID, "null argument");
+    if (!op->core_last)
+        return tkconv_forward_unfused(op, d_in, in_batch_stride, d_residual, residual_batch_stride, d_out, out_batch_stride,
+                                      stream);
     int st;
     if ((st = tdc_conv_forward_strided(op->first, d_in, in_batch_stride, nullptr, 0, op->d_f1, 0, stream)) != TDC_OK) return st;
-    if ((st = tdc_conv_forward(op->core, op->d_f1, nullptr, op->d_f2, stream)) != TDC_OK) return st;
-    return tdc_conv_forward_strided(op->last, op->d_f2, 0, d_residual, residual_batch_stride, d_out, out_batch_stride, stream);
+    return tdc_conv_forward_strided(op->core_last, op->d_f1, 0, d_residual, residual_batch_stride, d_out, out_batch_stride,
+                                    stream);
 }
 
 int tdc_tkconv_forward_features(tdc_tkconv *op, const float *d_in, float *d_feat_first, float *d_feat_core,
                                 float *d_out, void *stream) {
-    int st = tdc_tkconv_forward(op, d_in, nullptr, d_out, stream);
+    if (!op || !d_in || !d_out) return fail(TDC_ERR_INVALID, "null argument");
+    int st = tkconv_forward_unfused(op, d_in, 0, nullptr, 0, d_out, 0, stream);   // the core's output is wanted
     if (st != TDC_OK) return st;
     hipError_t e;
     if (d_feat_first) {
@@ -558,6 +590,7 @@ void tdc_tkconv_destroy(tdc_tkconv *op) {
     tdc_conv_plan_destroy(op->first);
     tdc_conv_plan_destroy(op->core);
     tdc_conv_plan_destroy(op->last);
+    tdc_conv_plan_destroy(op->core_last);
     if (op->d_f1) (void)hipFree(op->d_f1);
     if (op->d_f2) (void)hipFree(op->d_f2);
     delete op;

@@ -23,7 +23,7 @@ EXPORTS = (
     "tdc_conv_forward_strided", "tdc_tkconv_forward_strided",
     "tdc_conv_time", "tdc_conv_time_many", "tdc_conv_plan_destroy",
     "tdc_tkconv_create", "tdc_tkconv_set_weights", "tdc_tkconv_forward", "tdc_tkconv_forward_features",
-    "tdc_tkconv_core_forward", "tdc_tkconv_query", "tdc_tkconv_destroy",
+    "tdc_tkconv_core_forward", "tdc_tkconv_query", "tdc_tkconv_num_kernels", "tdc_tkconv_destroy",
     "tdc_model_evaluate", "tdc_model_enumerate", "tdc_model_select", "tdc_model_get_constants",
     "tdc_model_set_constants",
     "tdc_net_create", "tdc_net_tensor", "tdc_net_view", "tdc_net_affine", "tdc_net_affine_conv", "tdc_net_conv", "tdc_net_tkconv", "tdc_net_pool", "tdc_net_global_avgpool", "tdc_net_concat",

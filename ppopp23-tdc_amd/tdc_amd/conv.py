@@ -164,7 +164,7 @@ class TKConvOp:
     def forward(self, x, residual=None, out=None):
         d = self.desc
         _dev_check(x, (d.batch, d.C, d.H, d.W), "input")
-        oshape = (d.batch, self.tail[0] if self.tail else d.N, self.Ho, self.Wo)
+        oshape = (d.batch, d.N, self.Ho, self.Wo)
         if out is None:
             out = torch.empty(oshape, device=x.device, dtype=torch.float32)
         else:
