@@ -228,6 +228,14 @@ int tdc_net_global_avgpool(tdc_net *net, int32_t in, int32_t *out);
 /* Per-channel y = x*scale[c] + shift[c], then ReLU if relu != 0 (inference BatchNorm in front of a convolution). */
 int tdc_net_affine(tdc_net *net, int32_t in, const float *scale, const float *shift, int32_t relu, int32_t dst,
                    int32_t *out);
+/* A convolution with a 1x1 convolution (tail_N outputs) fused behind it, see tdc_conv_plan_create_with_tail:
+ * out = relu2?(W_tail * relu?(conv(x) + bias) + bias_tail + residual); the result has tail_N channels. */
+int tdc_net_conv_tail(tdc_net *net, int32_t in, int32_t N, int32_t KH, int32_t KW, int32_t stride, int32_t pad,
+                      const float *w_oihw, const float *bias, int32_t relu, int32_t tail_N, const float *w_tail,
+                      const float *bias_tail, int32_t residual, int32_t tail_relu, int32_t dst, int32_t *out);
+/* Gives the convolution added last (tdc_net_conv or tdc_net_conv_tail; 1x1, no padding) a per-channel affine
+ * (+ReLU) on its input, see tdc_conv_plan_set_input_affine. */
+int tdc_net_set_input_affine(tdc_net *net, const float *scale, const float *shift, int32_t relu);
 /* tdc_net_affine followed by a 1x1 convolution (stride 1, no padding), as ONE kernel: the affine (+ReLU when
  * affine_relu != 0) is applied to the input window inside the convolution. */
 int tdc_net_affine_conv(tdc_net *net, int32_t in, const float *scale, const float *shift, int32_t affine_relu, int32_t N,
@@ -258,6 +266,10 @@ int tdc_model_enumerate(const tdc_conv_desc *desc, tdc_tile *tiles_out, int32_t 
                         int32_t *count_out);
 /* The model's pick = argmin pred_us over tdc_model_enumerate. */
 int tdc_model_select(const tdc_conv_desc *desc, tdc_tile_info *info_out);
+/* The pick for the convolution with a 1x1 convolution of tail_N outputs fused behind it (tiles that hold all
+ * desc->N channels in one workgroup only); fails if there is none.  Compare pred_us with the sum of the two
+ * separate convolutions to decide whether the fusion pays. */
+int tdc_model_select_with_tail(const tdc_conv_desc *desc, int32_t tail_N, tdc_tile_info *info_out);
 /* Calibration constants of the latency model (launch floor, copy latency and rate, barrier cost, ...;
  * the counterpart of num_sm / num_threads / a,b,c / ratio in the reference's model.py:265-266,278).
  * get: writes up to `cap` values, *count_out = how many there are.  set: all of them, all > 0;

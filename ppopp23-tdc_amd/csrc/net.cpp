@@ -164,27 +164,33 @@ int tdc_net_view(tdc_net *net, int32_t id, int32_t c0, int32_t C, int32_t *out) 
     return TDC_OK;
 }
 
-int tdc_net_conv(tdc_net *net, int32_t in, int32_t N, int32_t KH, int32_t KW, int32_t stride, int32_t pad, const float *w,
-                 const float *bias, int32_t residual, int32_t relu, int32_t dst, int32_t *out) {
+// Shared by the plain and the tail-fused convolution operators.
+static int net_add_conv(tdc_net *net, int32_t in, int32_t N, int32_t KH, int32_t KW, int32_t stride, int32_t pad,
+                        const float *w, const float *bias, int32_t relu, int32_t tail_N, const float *w_tail,
+                        const float *bias_tail, int32_t tail_relu, int32_t residual, int32_t dst, int32_t *out) {
     int st = check_open(net);
     if (st != TDC_OK) return st;
-    if (!out || !w || !valid_id(net, in) || (residual >= 0 && !valid_id(net, residual)))
+    if (!out || !w || !valid_id(net, in) || (residual >= 0 && !valid_id(net, residual)) || (tail_N > 0 && !w_tail))
         return api_fail(TDC_ERR_INVALID, "bad tensor id or null argument");
     const NetTensor ti = net->tensors[in];
+    // without a tail the residual and the ReLU belong to the convolution's own epilogue
     tdc_conv_desc d{net->batch, ti.C, N, ti.H, ti.W, KH, KW, stride, pad, 1, bias != nullptr, relu != 0};
     std::string why;
     if (!check_desc(d, &why)) return api_fail(TDC_ERR_INVALID, why);
     const int Ho = (ti.H + 2 * pad - (KH - 1) - 1) / stride + 1, Wo = (ti.W + 2 * pad - (KW - 1) - 1) / stride + 1;
+    const int Nout = tail_N > 0 ? tail_N : N;
     if (residual >= 0) {
         const NetTensor &tr = net->tensors[residual];
-        if (tr.C != N || tr.H != Ho || tr.W != Wo)
+        if (tr.C != Nout || tr.H != Ho || tr.W != Wo)
             return api_fail(TDC_ERR_INVALID, "residual tensor shape does not match the convolution output");
     }
     int id;
-    if ((st = resolve_dst(net, dst, N, Ho, Wo, &id)) != TDC_OK) return st;
+    if ((st = resolve_dst(net, dst, Nout, Ho, Wo, &id)) != TDC_OK) return st;
     tdc_conv_plan *plan = nullptr;
-    if ((st = tdc_conv_plan_create(&d, nullptr, &plan)) != TDC_OK) return st;
-    if ((st = tdc_conv_plan_set_weights(plan, w, bias)) != TDC_OK) {
+    if ((st = tdc_conv_plan_create_with_tail(&d, tail_N, bias_tail != nullptr, tail_relu, nullptr, &plan)) != TDC_OK) return st;
+    st = tdc_conv_plan_set_weights(plan, w, bias);
+    if (st == TDC_OK && tail_N > 0) st = tdc_conv_plan_set_tail_weights(plan, w_tail, bias_tail);
+    if (st != TDC_OK) {
         tdc_conv_plan_destroy(plan);
         return st;
     }
@@ -194,6 +200,27 @@ int tdc_net_conv(tdc_net *net, int32_t in, int32_t N, int32_t KH, int32_t KW, in
     net->kernels += 1;
     *out = id;
     return TDC_OK;
+}
+
+int tdc_net_conv(tdc_net *net, int32_t in, int32_t N, int32_t KH, int32_t KW, int32_t stride, int32_t pad, const float *w,
+                 const float *bias, int32_t residual, int32_t relu, int32_t dst, int32_t *out) {
+    return net_add_conv(net, in, N, KH, KW, stride, pad, w, bias, relu, 0, nullptr, nullptr, 0, residual, dst, out);
+}
+
+int tdc_net_conv_tail(tdc_net *net, int32_t in, int32_t N, int32_t KH, int32_t KW, int32_t stride, int32_t pad,
+                      const float *w, const float *bias, int32_t relu, int32_t tail_N, const float *w_tail,
+                      const float *bias_tail, int32_t residual, int32_t tail_relu, int32_t dst, int32_t *out) {
+    if (tail_N < 1) return api_fail(TDC_ERR_INVALID, "tail_N must be >= 1");
+    return net_add_conv(net, in, N, KH, KW, stride, pad, w, bias, relu, tail_N, w_tail, bias_tail, tail_relu, residual, dst,
+                        out);
+}
+
+int tdc_net_set_input_affine(tdc_net *net, const float *scale, const float *shift, int32_t relu) {
+    int st = check_open(net);
+    if (st != TDC_OK) return st;
+    if (net->ops.empty() || net->ops.back().kind != NetOp::CONV)
+        return api_fail(TDC_ERR_STATE, "the last operator added is not a convolution");
+    return tdc_conv_plan_set_input_affine(net->ops.back().conv, scale, shift, relu);
 }
 
 int tdc_net_affine_conv(tdc_net *net, int32_t in, const float *scale, const float *shift, int32_t affine_relu, int32_t N,

@@ -113,6 +113,13 @@ int tdc_model_select(const tdc_conv_desc *desc, tdc_tile_info *info_out) {
     return TDC_OK;
 }
 
+int tdc_model_select_with_tail(const tdc_conv_desc *desc, int32_t tail_N, tdc_tile_info *info_out) {
+    if (!desc || !info_out || tail_N < 0) return fail(TDC_ERR_INVALID, "null argument");
+    std::string why;
+    if (!model_select(*desc, *info_out, &why, tail_N)) return fail(TDC_ERR_INVALID, why);
+    return TDC_OK;
+}
+
 int tdc_load_bin(const char *path, float *dst, uint64_t count) {
     if (!path || (!dst && count)) return fail(TDC_ERR_INVALID, "null argument");
     FILE *f = std::fopen(path, "rb");

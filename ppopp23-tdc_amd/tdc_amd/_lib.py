@@ -24,9 +24,9 @@ EXPORTS = (
     "tdc_conv_time", "tdc_conv_time_many", "tdc_conv_plan_destroy",
     "tdc_tkconv_create", "tdc_tkconv_set_weights", "tdc_tkconv_forward", "tdc_tkconv_forward_features",
     "tdc_tkconv_core_forward", "tdc_tkconv_query", "tdc_tkconv_num_kernels", "tdc_tkconv_destroy",
-    "tdc_model_evaluate", "tdc_model_enumerate", "tdc_model_select", "tdc_model_get_constants",
+    "tdc_model_evaluate", "tdc_model_enumerate", "tdc_model_select", "tdc_model_select_with_tail", "tdc_model_get_constants",
     "tdc_model_set_constants",
-    "tdc_net_create", "tdc_net_tensor", "tdc_net_view", "tdc_net_affine", "tdc_net_affine_conv", "tdc_net_conv", "tdc_net_tkconv", "tdc_net_pool", "tdc_net_global_avgpool", "tdc_net_concat",
+    "tdc_net_create", "tdc_net_tensor", "tdc_net_view", "tdc_net_affine", "tdc_net_affine_conv", "tdc_net_conv", "tdc_net_conv_tail", "tdc_net_set_input_affine", "tdc_net_tkconv", "tdc_net_pool", "tdc_net_global_avgpool", "tdc_net_concat",
     "tdc_net_tensor_shape", "tdc_net_num_kernels", "tdc_net_finalize", "tdc_net_forward", "tdc_net_time",
     "tdc_net_read_tensor", "tdc_net_destroy",
 )
@@ -167,6 +167,27 @@ def model_evaluate(desc: ConvDesc, tile: Tile) -> TileInfo:
 MODEL_CONSTANT_NAMES = ("launch_us", "setup_clk", "copy_latency_clk", "copy_bytes_per_clk", "l2_bytes_per_clk",
                         "lds_bytes_per_clk", "sync_clk", "store_bytes_per_clk", "kstep_issue_clk", "pass_overhead_clk",
                         "wave_setup_clk", "ksplit_clk", "copy_issue_clk", "lds_read_clk")
+
+
+def model_select_with_tail(desc: ConvDesc, tail_N: int):
+    """The model's pick for `desc` with a 1x1 convolution of tail_N outputs fused behind it, or None if no tile can
+    hold all output channels in one workgroup."""
+    info = TileInfo()
+    if lib().tdc_model_select_with_tail(byref(desc), int(tail_N), byref(info)) != TDC_OK:
+        return None
+    return info
+
+
+def fused_tail_pays(desc: ConvDesc, tail_N: int, margin: float = 0.9):
+    """True if the model predicts conv + fused 1x1 tail faster than the two convolutions launched separately
+    (by at least 10 %: measured, the model is that much too kind to the fused kernel at batch 1)."""
+    fused = model_select_with_tail(desc, tail_N)
+    if fused is None:
+        return False
+    Ho = (desc.H + 2 * desc.pad - desc.dilation * (desc.KH - 1) - 1) // desc.stride + 1
+    Wo = (desc.W + 2 * desc.pad - desc.dilation * (desc.KW - 1) - 1) // desc.stride + 1
+    tail = conv_desc(desc.batch, desc.N, tail_N, Ho, Wo, 1, 1, 1, 0)
+    return fused.pred_us < margin * (model_select(desc).pred_us + model_select(tail).pred_us)
 
 
 def model_get_constants():

@@ -17,6 +17,7 @@ from ctypes import byref, c_int32, c_void_p
 
 import torch
 
+from . import _lib
 from ._lib import check, lib
 
 BN_EPS = 1e-5
@@ -57,6 +58,21 @@ class Net:
         self.conv_shapes.append((C, w.shape[0], H, W, w.shape[2], stride, pad))
         check(lib().tdc_net_conv(self._h, x, w.shape[0], w.shape[2], w.shape[3], stride, pad, _p(w), _p(b), residual,
                                  int(relu), dst, byref(out)))
+        return out.value
+
+    def conv_tail(self, x, weight, tail_weight, bias=None, relu=False, tail_bias=None, stride=1, pad=0, residual=-1,
+                  tail_relu=False, dst=-1, in_affine=None):
+        """Convolution with a 1x1 convolution fused behind it (one kernel); ``in_affine=(scale, shift, relu)`` adds
+        a per-channel affine on the input (1x1 convolutions without padding only)."""
+        w, b, w2, b2 = _h(weight), _h(bias), _h(tail_weight), _h(tail_bias)
+        out = c_int32()
+        _, C, H, W = self.shape(x)
+        self.conv_shapes.append((C, w.shape[0], H, W, w.shape[2], stride, pad))
+        check(lib().tdc_net_conv_tail(self._h, x, w.shape[0], w.shape[2], w.shape[3], stride, pad, _p(w), _p(b), int(relu),
+                                      w2.shape[0], _p(w2), _p(b2), residual, int(tail_relu), dst, byref(out)))
+        if in_affine is not None:
+            sc, sh = _h(in_affine[0]), _h(in_affine[1])
+            check(lib().tdc_net_set_input_affine(self._h, _p(sc), _p(sh), int(in_affine[2])))
         return out.value
 
     def affine_conv(self, x, scale, shift, weight, bias=None, affine_relu=True, residual=-1, relu=False, dst=-1):
@@ -291,10 +307,18 @@ def build_tucker_densenet121(params, batch=1, H=224, W=224, growth=32):
             pre = f"features.denseblock{b}.denselayer{l}"
             s1, t1 = bn_scale_shift(p, pre + ".norm1")
             s2, t2 = bn_scale_shift(p, pre + ".norm2")
-            # norm1 + relu on the concatenation, conv1, norm2 + relu: one kernel
-            y = net.affine_conv(net.view(cat, 0, c), s1, t1, fold_dense(p[pre + ".conv1.weight"], s2), t2, relu=True)
-            net.tkconv(y, p[pre + ".conv2.first_kernel"], p[pre + ".conv2.core_kernel"], p[pre + ".conv2.last_kernel"],
-                       pad=1, dst=net.view(cat, c, growth))
+            w1 = fold_dense(p[pre + ".conv1.weight"], s2)
+            first, core, last = (p[pre + ".conv2.first_kernel"], p[pre + ".conv2.core_kernel"],
+                                 p[pre + ".conv2.last_kernel"])
+            d1 = _lib.conv_desc(batch, c, w1.shape[0], h, w, 1, 1, 1, 0, 1, True, True)
+            if _lib.fused_tail_pays(d1, first.shape[0]):
+                # norm1 + relu, conv1, norm2 + relu and the first Tucker factor in one kernel; core + last in another
+                y = net.conv_tail(net.view(cat, 0, c), w1, first, bias=t2, relu=True, in_affine=(s1, t1, True))
+                net.conv_tail(y, core, last, pad=1, dst=net.view(cat, c, growth))
+            else:
+                # norm1 + relu on the concatenation, conv1, norm2 + relu: one kernel; then the Tucker convolution
+                y = net.affine_conv(net.view(cat, 0, c), s1, t1, w1, t2, relu=True)
+                net.tkconv(y, first, core, last, pad=1, dst=net.view(cat, c, growth))
             c += growth
         if b < len(DENSENET121_BLOCKS):
             pre = f"features.transition{b}"
