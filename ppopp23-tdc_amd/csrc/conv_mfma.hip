@@ -42,6 +42,10 @@
 
 #include "tdc_internal.hpp"
 
+#ifndef TDC_TOUCH_KERNARGS
+#define TDC_TOUCH_KERNARGS 1
+#endif
+
 namespace tdc {
 
 typedef float f4_t __attribute__((ext_vector_type(4)));
@@ -134,13 +138,14 @@ __device__ __forceinline__ void copy_block(int vw, __amdgpu_buffer_rsrc_t rsrc, 
 // vector ALU instructions issued next to MFMAs are not free.
 // Weights: a linear copy in 16-byte elements, 1 KiB per instruction; always inside the packed buffer
 // (or past its end, which reads as zero into the slack), so the block offset can ride in the scalar operand.
+template <bool EXT>
 __device__ __forceinline__ void issue_weights(const ConvKParams &p, __amdgpu_buffer_rsrc_t w_rsrc,
                                               float *__restrict__ stage, int lane16, int w_byte0, int dw, int dn, int chunk) {
     float *wdst = stage + p.in_stage_floats;
     const int wnblk = (p.wslab_floats + 255) >> 8;
     for (int blk = dw; blk < wnblk; blk += dn) copy_block(4, w_rsrc, wdst + (blk << 8), lane16, w_byte0 + (blk << 10));
     // The per-channel scale and shift of an input affine ride behind the weights: [pass][scale(CCH) | shift(CCH)].
-    if (p.in_aff) {
+    if constexpr (EXT) if (p.in_aff) {
         const __amdgpu_buffer_rsrc_t a_rsrc = __builtin_amdgcn_make_buffer_rsrc(
             const_cast<float *>(p.in_aff), (short)0, (int)(p.nchunks * p.CCH * 8), 0x00020000);
         float *adst = wdst + (wnblk << 8);
@@ -172,7 +177,9 @@ __device__ __forceinline__ void issue_inputs(const ConvKParams &p, __amdgpu_buff
         copy_block(VW, in_rsrc, stage + blk * blk_floats, input_copy_offset(p, (blk << 6) + lane, iy0, ix0a) + pass_bytes, 0);
 }
 
-template <int MF, int MB, int NB, int TAPS, int MAXW>
+// EXT: the instantiation also carries the fused extras (input affine, 1x1 tail).  They are compiled out of the
+// plain kernels: their registers and code cost every layer 0.2-0.5 us otherwise (measured).
+template <int MF, int MB, int NB, int TAPS, int MAXW, bool EXT>
 __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKParams p) {
     using M = Mfma<MF>;
     using acc_t = typename M::acc_t;
@@ -184,7 +191,7 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
     // them in several dependent batches, and every batch that touches a cache line for the first time costs a
     // round trip to L2 before the first copy can start.  Touch every line of the argument block at once: whatever
     // order the compiler then loads the values in, it hits the scalar cache.
-    {
+    if constexpr (TDC_TOUCH_KERNARGS) {
         static_assert(sizeof(ConvKParams) <= 8 * 64, "touch more lines");
         const auto kargs = __builtin_amdgcn_kernarg_segment_ptr();
         unsigned t0, t1, t2, t3, t4, t5, t6, t7;
@@ -259,7 +266,7 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
 
     // The weight copies of the first pass need no per-lane arithmetic: start them before anything else.
     const int lane16 = lane * 16;
-    issue_weights(p, w_rsrc, lds, lane16, (int)(w_byte_base + (unsigned)chunk0 * w_pass_bytes), wave, nwaves, chunk0);
+    issue_weights<EXT>(p, w_rsrc, lds, lane16, (int)(w_byte_base + (unsigned)chunk0 * w_pass_bytes), wave, nwaves, chunk0);
 
     // Offsets of this lane's elements in its wave's first MAXPRE input blocks (pass 0), for the steady dealing
     // (positions past the stage decode to a channel >= CCH and so to the out-of-range offset).  With loader
@@ -301,7 +308,7 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
         // Copy issue competes for the SIMD with other waves' MFMA streams and loses by default (measured:
         // ~330 cycles per copy instruction instead of ~115); it is short, so let it go first.
         __builtin_amdgcn_s_setprio(3);
-        issue_weights(p, w_rsrc, stage, lane16, w_byte0, dw, dn, chunk);
+        issue_weights<EXT>(p, w_rsrc, stage, lane16, w_byte0, dw, dn, chunk);
         issue_inputs(p, in_rsrc, stage, pre, true, chunk, iy0, ix0a, dw, dn, lane);
         __builtin_amdgcn_s_setprio(0);
     };
@@ -335,7 +342,7 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
         __builtin_amdgcn_s_waitcnt(0);
         __syncthreads();
         if (chunk + 1 < chunk1) issue(chunk + 1);
-        if constexpr (TAPS == TAPS_1x1) {
+        if constexpr (EXT && TAPS == TAPS_1x1) {
             // Optional per-input-channel affine (+ReLU) in front of the convolution (an inference BatchNorm that
             // cannot be folded into a producer): applied in place to the freshly landed input window.  A 1x1
             // convolution without padding has no zero halo that would have to stay zero; lanes past the image and
@@ -625,7 +632,7 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
         if (p.relu) val = fmaxf(val, 0.0f);
         out[o] = val;
     };
-    if (p.tail_w) {
+    if constexpr (EXT) if (p.tail_w) {
         // Fused tail: a 1x1 convolution over the output channels of this one, out2 = W2 * act(conv + bias), in the
         // same kernel (the last factor of a Tucker convolution behind its core, or the first factor of the next one
         // behind a bottleneck convolution).  The workgroup owns ALL output channels of the convolution (the host
@@ -772,19 +779,19 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
 // ---------------------------------------------------------------------------
 typedef void (*kernel_fn)(const ConvKParams);
 
-template <int MF, int TAPS>
+template <int MF, int TAPS, bool EXT>
 static kernel_fn pick_mbnb(int mb, int nb) {
-    if (mb == 1 && nb == 1) return tdc_conv_mfma_kernel<MF, 1, 1, TAPS, 16>;
-    if (mb == 1 && nb == 2) return tdc_conv_mfma_kernel<MF, 1, 2, TAPS, 16>;
-    if (mb == 2 && nb == 1) return tdc_conv_mfma_kernel<MF, 2, 1, TAPS, 16>;
-    if (mb == 2 && nb == 2) return tdc_conv_mfma_kernel<MF, 2, 2, TAPS, 8>;
+    if (mb == 1 && nb == 1) return tdc_conv_mfma_kernel<MF, 1, 1, TAPS, 16, EXT>;
+    if (mb == 1 && nb == 2) return tdc_conv_mfma_kernel<MF, 1, 2, TAPS, 16, EXT>;
+    if (mb == 2 && nb == 1) return tdc_conv_mfma_kernel<MF, 2, 1, TAPS, 16, EXT>;
+    if (mb == 2 && nb == 2) return tdc_conv_mfma_kernel<MF, 2, 2, TAPS, 8, EXT>;
     return nullptr;
 }
 
-template <int TAPS>
+template <int TAPS, bool EXT>
 static kernel_fn pick_mf(int mf, int mb, int nb) {
-    if (mf == 32) return pick_mbnb<32, TAPS>(mb, nb);
-    if (mf == 16) return pick_mbnb<16, TAPS>(mb, nb);
+    if (mf == 32) return pick_mbnb<32, TAPS, EXT>(mb, nb);
+    if (mf == 16) return pick_mbnb<16, TAPS, EXT>(mb, nb);
     return nullptr;
 }
 
@@ -794,12 +801,12 @@ static int taps_mode(int KH, int KW, int dil) {
     return TAPS_GENERIC;
 }
 
-const void *conv_kernel_for(const tdc_tile &t, int KH, int KW, int dilation) {
+const void *conv_kernel_for(const tdc_tile &t, int KH, int KW, int dilation, bool extras) {
     kernel_fn fn = nullptr;
     switch (taps_mode(KH, KW, dilation)) {
-        case TAPS_3x3: fn = pick_mf<TAPS_3x3>(t.mf, t.mb, t.nb); break;
-        case TAPS_1x1: fn = pick_mf<TAPS_1x1>(t.mf, t.mb, t.nb); break;
-        default: fn = pick_mf<TAPS_GENERIC>(t.mf, t.mb, t.nb); break;
+        case TAPS_3x3: fn = extras ? pick_mf<TAPS_3x3, true>(t.mf, t.mb, t.nb) : pick_mf<TAPS_3x3, false>(t.mf, t.mb, t.nb); break;
+        case TAPS_1x1: fn = extras ? pick_mf<TAPS_1x1, true>(t.mf, t.mb, t.nb) : pick_mf<TAPS_1x1, false>(t.mf, t.mb, t.nb); break;
+        default: fn = extras ? pick_mf<TAPS_GENERIC, true>(t.mf, t.mb, t.nb) : pick_mf<TAPS_GENERIC, false>(t.mf, t.mb, t.nb); break;
     }
     return reinterpret_cast<const void *>(fn);
 }
