@@ -54,6 +54,8 @@ def main():
                     help="profiling aid: launch only the dominant layer (128->128 @56), `steps` times, and exit")
     ap.add_argument("--only-e2e", action="store_true",
                     help="profiling aid: run only the end-to-end Tucker ResNet-18 forward, `steps` times, and exit")
+    ap.add_argument("--e2e-net", choices=["resnet18", "densenet121"], default="resnet18",
+                    help="which Tucker network --only-e2e runs (batch 1)")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="BYTES",
                     help="profiling aid: run a plain device copy of BYTES bytes a few times (reference reading for "
                          "the FETCH_SIZE / WRITE_SIZE counters) before anything else")
@@ -81,9 +83,13 @@ def main():
 
     if a.only_e2e:
         from tdc_amd import nets
-        net = nets.build_tucker_resnet18(nets.resnet18_params(seed=18), batch=1)
+        if a.e2e_net == "densenet121":
+            net = nets.build_tucker_densenet121(nets.densenet121_params(seed=121), batch=1)
+        else:
+            net = nets.build_tucker_resnet18(nets.resnet18_params(seed=18), batch=1)
         ms = net.time_ms(iters=a.steps, graph=graph)
-        print(json.dumps({"only_e2e": True, "forwards": a.steps, "ms": ms, "kernels": net.num_kernels}))
+        print(json.dumps({"only_e2e": True, "net": a.e2e_net, "forwards": a.steps, "ms": ms,
+                          "kernels": net.num_kernels}))
         return
 
     if a.only_dominant:
@@ -239,7 +245,7 @@ def main():
                     sys.exit("bench.py: DenseNet-121 parity check failed (max err %g)" % derr)
             dnet.time_ms(iters=5)
             dres["b%d_ms" % b] = round(min(dnet.time_ms(iters=20) for _ in range(3)), 4)
-            dres["kernels_per_forward"] = dnet.num_kernels
+            dres["b%d_kernels_per_forward" % b] = dnet.num_kernels
             dnet.close()
         out["tucker_densenet121"] = dres
         # The four full Tucker blocks (configuration 3): 1x1 C->R1, 3x3 R1->R2, 1x1 R2->N as three launches in a graph.

@@ -19,31 +19,29 @@ namespace tdc {
 // including padding zeros (count_include_pad, which equals PyTorch's AvgPool2d
 // default and is irrelevant when pad == 0).
 __global__ void __launch_bounds__(256) pool2d_kernel(const float *__restrict__ in, long long in_bs,
-                                                     float *__restrict__ out, long long out_bs, int B, int C, int H,
-                                                     int W, int Ho, int Wo, int k, int stride, int pad, int mode) {
-    const long long per = (long long)C * Ho * Wo;
-    const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= per * B) return;
-    const int b = (int)(idx / per);
-    const long long rem = idx - (long long)b * per;
-    const int ox = (int)(rem % Wo);
-    const long long t = rem / Wo;
-    const int oy = (int)(t % Ho);
-    const int c = (int)(t / Ho);
+                                                     float *__restrict__ out, long long out_bs, int C, int H, int W,
+                                                     int Ho, int Wo, int k, int stride, int pad, int mode) {
+    // grid = (pixel blocks, channels, batch): no 64-bit division, one 32-bit division per thread
+    const int pix = blockIdx.x * blockDim.x + threadIdx.x;
+    if (pix >= Ho * Wo) return;
+    const int c = blockIdx.y, b = blockIdx.z;
+    const int oy = pix / Wo, ox = pix - oy * Wo;
     const float *src = in + b * in_bs + (long long)c * H * W;
     float acc = mode == 0 ? -FLT_MAX : 0.0f;
+    const int iy0 = oy * stride - pad, ix0 = ox * stride - pad;
     for (int r = 0; r < k; ++r) {
-        const int iy = oy * stride - pad + r;
-        if (iy < 0 || iy >= H) continue;
+        const int iy = iy0 + r;
+        if ((unsigned)iy >= (unsigned)H) continue;
+        const float *row = src + iy * W;
         for (int s = 0; s < k; ++s) {
-            const int ix = ox * stride - pad + s;
-            if (ix < 0 || ix >= W) continue;
-            const float v = src[iy * W + ix];
+            const int ix = ix0 + s;
+            if ((unsigned)ix >= (unsigned)W) continue;
+            const float v = row[ix];
             acc = mode == 0 ? fmaxf(acc, v) : acc + v;
         }
     }
     if (mode == 1) acc *= 1.0f / (float)(k * k);
-    out[b * out_bs + rem] = acc;
+    out[b * out_bs + (long long)c * Ho * Wo + pix] = acc;
 }
 
 // Global average pool: one wave per plane, lanes stride over the H*W pixels, shuffle reduction.
@@ -96,8 +94,9 @@ static unsigned blocks_for(long long total) { return (unsigned)((total + 255) / 
 
 int launch_pool2d(const float *in, long long in_bs, float *out, long long out_bs, int B, int C, int H, int W, int Ho,
                   int Wo, int k, int stride, int pad, int mode, void *stream) {
-    hipLaunchKernelGGL(pool2d_kernel, dim3(blocks_for((long long)B * C * Ho * Wo)), dim3(256), 0, (hipStream_t)stream, in,
-                       in_bs, out, out_bs, B, C, H, W, Ho, Wo, k, stride, pad, mode);
+    if (C > 65535 || B > 65535) return (int)hipErrorInvalidValue;
+    hipLaunchKernelGGL(pool2d_kernel, dim3(blocks_for((long long)Ho * Wo), C, B), dim3(256), 0, (hipStream_t)stream, in,
+                       in_bs, out, out_bs, C, H, W, Ho, Wo, k, stride, pad, mode);
     return (int)hipGetLastError();
 }
 

@@ -6,11 +6,14 @@ geometry (grid, workgroup, LDS) is what tells the layers apart.
 
     python -m tdc_amd.profsum kernel <dir-with-*_kernel_trace.csv>
     python -m tdc_amd.profsum pmc    <dir-with-*_counter_collection.csv> [--copy-bytes N]
+    python -m tdc_amd.profsum timeline <dir-with-*_kernel_trace.csv> --last N
 
 ``kernel``: count / mean / min / max duration in microseconds per (kernel, grid, workgroup, LDS).
 ``pmc``: mean counter value per (kernel, grid, workgroup); with ``--copy-bytes N`` the FETCH_SIZE /
 WRITE_SIZE readings (KiB) of every kernel are also shown scaled by the reading of the largest
 copy kernel in the same run, which is known to read and write N bytes.
+``timeline``: the last N dispatches of the trace in launch order (one forward of a network of N kernels):
+start offset, duration, and the idle gap since the previous kernel ended.
 """
 from __future__ import annotations
 
@@ -76,14 +79,41 @@ def pmc_summary(path, copy_bytes=None, out=sys.stdout):
             out.write(line + "\n")
 
 
+def timeline(path, last, out=sys.stdout):
+    files = sorted(glob.glob(os.path.join(path, "**", "*kernel_trace.csv"), recursive=True))
+    if not files:
+        raise SystemExit(f"no *kernel_trace.csv under {path}")
+    rows = []
+    for f in files:
+        rows += list(csv.DictReader(open(f)))
+    rows.sort(key=lambda r: int(r["Start_Timestamp"]))
+    rows = rows[-last:]
+    t0 = int(rows[0]["Start_Timestamp"])
+    prev_end, busy, idle = None, 0.0, 0.0
+    out.write("%3s %-58s %8s %5s %9s %8s %7s\n" % ("#", "kernel", "grid_x", "wg", "start_us", "dur_us", "gap_us"))
+    for i, r in enumerate(rows):
+        b, e = int(r["Start_Timestamp"]), int(r["End_Timestamp"])
+        gap = 0.0 if prev_end is None else (b - prev_end) * 1e-3
+        busy += (e - b) * 1e-3
+        idle += max(gap, 0.0)
+        out.write("%3d %-58s %8d %5d %9.2f %8.2f %7.2f\n" % (i, _short(r["Kernel_Name"])[:58], int(r["Grid_Size_X"]),
+                                                            int(r["Workgroup_Size_X"]), (b - t0) * 1e-3, (e - b) * 1e-3, gap))
+        prev_end = e
+    out.write("# %d kernels: first start to last end %.2f us; sum of durations %.2f us; idle between kernels %.2f us\n" % (
+        len(rows), (prev_end - t0) * 1e-3, busy, idle))
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser()
-    ap.add_argument("mode", choices=["kernel", "pmc"])
+    ap.add_argument("mode", choices=["kernel", "pmc", "timeline"])
     ap.add_argument("path")
     ap.add_argument("--copy-bytes", type=int, default=None)
+    ap.add_argument("--last", type=int, default=64, help="timeline: how many dispatches from the end of the trace")
     a = ap.parse_args(argv)
     if a.mode == "kernel":
         kernel_summary(a.path)
+    elif a.mode == "timeline":
+        timeline(a.path, a.last)
     else:
         pmc_summary(a.path, a.copy_bytes)
 
