@@ -191,6 +191,10 @@ def main():
         roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_TBPS * 1e3, "unit": "GB/s",
                     "frac": round(achieved / (PEAK_HBM_TBPS * 1e3), 4), "traffic": None}
     roofline["traffic"] = measured_traffic(dinfo.tile.astuple())
+    # the same kernel as isolated launches (one hipEvent pair around ONE eager launch, 200 times): includes the
+    # start-up of an idle queue, so it is reported next to the back-to-back figure, not used for `achieved`
+    singles = sorted(dl["plan"].time_us(dl["x"], dl["out"], iters=1, graph=False) for _ in range(200))
+    roofline["single_launch_us"] = {"median": round(singles[len(singles) // 2], 3), "p10": round(singles[20], 3)}
     roofline.update({"kernel": "core conv %d->%d @%dx%d" % (dl["r1"], dl["r2"], dl["hw"], dl["hw"]),
                      "avg_launch_us": round(dom_us, 3), "flops_per_launch": dinfo.flops,
                      "bytes_per_launch": dinfo.bytes, "timing": "hipEvents around 200 graph-replayed launches"})

@@ -497,7 +497,14 @@ bool model_select(const tdc_conv_desc &d, tdc_tile_info &best, std::string *why,
             have = true;
         }
     }
-    if (!have && why) *why = "no launchable tile for this shape";
+    if (!have && why) {
+        // say why the plainest tile cannot be launched: that is the limit the shape runs into
+        const tdc_tile plain{16, 1, 1, 1, 1, 1, 4, 1, 1, 0};
+        Geometry g;
+        std::string reason;
+        *why = make_geometry(d, plain, g, &reason, tail_N) ? "no launchable tile for this shape"
+                                                             : "no launchable tile for this shape: " + reason;
+    }
     return have;
 }
 

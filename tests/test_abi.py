@@ -56,6 +56,23 @@ def test_invalid_descriptors_are_rejected_with_a_reason():
         assert e.value.status == _lib.TDC_ERR_INVALID and len(str(e.value)) > 20
 
 
+def test_shapes_beyond_the_addressing_limits_are_rejected_not_truncated():
+    """One image is addressed with 32-bit byte offsets and 24-bit index products; anything larger must be
+    refused with a reason instead of wrapping around."""
+    too_big = [
+        (tdc_amd.conv_desc(1, 2048, 8, 1024, 1024, 3, 3, 1, 1), "2^29"),    # 2^31 input elements per image
+        (tdc_amd.conv_desc(1, 8, 2048, 1024, 1024, 3, 3, 1, 1), "2^29"),    # ... output elements per image
+        (tdc_amd.conv_desc(1, 20000, 20000, 8, 8, 3, 3, 1, 1), "2^28"),     # 3.6e9 weights
+        (tdc_amd.conv_desc(1, 4096, 4, 4096, 16, 3, 3, 1, 1), "too large"),  # (C+1)*H beyond 24 bits
+    ]
+    for d, reason in too_big:
+        with pytest.raises(tdc_amd.TdcError) as e:
+            tdc_amd.model_select(d)
+        assert reason in str(e.value), str(e.value)
+    # just inside the limits a tile is found
+    assert tdc_amd.model_select(tdc_amd.conv_desc(1, 4000, 4, 4000, 16, 3, 3, 1, 1)).pred_us > 0
+
+
 def test_plan_creation_without_a_gpu_fails_loudly():
     import torch
     if torch.cuda.is_available():

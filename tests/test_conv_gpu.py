@@ -126,6 +126,25 @@ def test_random_shapes_model_tile():
         done += 1
 
 
+@pytest.mark.parametrize("B,C,N,H,W,K,stride,pad", [
+    (1, 3, 5, 1030, 770, 3, 1, 1),      # a large ragged image, few channels
+    (1, 2, 3, 64, 4100, 1, 1, 0),       # 1x1 on a 262 400-pixel flattened image
+    (1, 520, 24, 9, 9, 3, 1, 1),        # many input channels (several passes, ragged last pass)
+    (1, 24, 520, 9, 9, 3, 1, 1),        # many output channels (many channel tiles)
+    (37, 5, 7, 11, 13, 3, 2, 1),        # a long batch
+    (1, 4, 4, 1, 1, 1, 1, 0),           # a single pixel
+    (2, 1, 1, 1, 300, 3, 1, 1),         # one row
+    (2, 1, 1, 300, 1, 3, 1, 1),         # one column
+])
+def test_extreme_shapes_model_tile(B, C, N, H, W, K, stride, pad):
+    """Shapes at the edges of what the layers of the networks use: very large and degenerate images, long
+    batches, channel counts far above the tile sizes; model-picked tile, against F.conv2d on the host."""
+    announce("extreme", B, C, N, H, W, K, stride, pad)
+    x, w = case(7000 + C + N + H, B, C, N, H, W, K)
+    got = run_conv(x, w, stride=stride, pad=pad)
+    assert_close(got, ref.conv2d_torch(x, w, stride=stride, pad=pad).numpy(), f"extreme {(B, C, N, H, W, K)}")
+
+
 def test_stride2_resnet_core_shapes():
     """The three stride-2 core convs of Tucker ResNet-18 (64->64 56->28, 128->128 28->14, 256->256 14->7)."""
     for r, hw in ((64, 56), (128, 28), (256, 14)):
