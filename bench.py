@@ -56,6 +56,11 @@ def main():
                     help="profiling aid: run only the end-to-end Tucker ResNet-18 forward, `steps` times, and exit")
     ap.add_argument("--e2e-net", choices=["resnet18", "densenet121"], default="resnet18",
                     help="which Tucker network --only-e2e runs (batch 1)")
+    ap.add_argument("--tile", default=None, metavar="mf,mb,nb,wm,wn,wk,cch,tw,ks,wl",
+                    help="with --only-dominant: force this tile instead of selecting one")
+    ap.add_argument("--tune", type=int, default=16, metavar="CLASSES",
+                    help="measured tile selection at plan creation: time the model's favourite tile of this many tile "
+                         "classes and keep the fastest (0 = the analytic model's pick alone)")
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="BYTES",
                     help="profiling aid: run a plain device copy of BYTES bytes a few times (reference reading for "
                          "the FETCH_SIZE / WRITE_SIZE counters) before anything else")
@@ -73,6 +78,7 @@ def main():
         sys.exit("bench.py needs a GPU")
     torch.cuda.set_device(0)
     graph = not a.no_graph
+    tdc_amd.set_autotune(a.tune)
 
     if a.calibrate_copy:
         src = torch.empty(a.calibrate_copy // 4, device="cuda").normal_()
@@ -94,7 +100,11 @@ def main():
 
     if a.only_dominant:
         x, w = ref.make_core_case(56, 128, 128)
-        plan = Conv2dPlan(1, 128, 128, 56, 56, 3, 3, 1, 1).set_weights(w)
+        forced = None
+        if a.tile:
+            v = [int(t) for t in a.tile.split(",")]
+            forced = tdc_amd.Tile(*v[:8], ks=v[8], wl=v[9])
+        plan = Conv2dPlan(1, 128, 128, 56, 56, 3, 3, 1, 1, tile=forced).set_weights(w)
         xd, out = x.cuda(), torch.empty(1, 128, 56, 56, device="cuda")
         # the same back-to-back launches as the timed region of the full run (one graph of `steps` launches)
         if a.warmup > 0:
@@ -135,6 +145,18 @@ def main():
     ms_per_step = total_ms / a.steps
     us_per_layer = ms_per_step * 1e3 / len(layers)
 
+    # -- the same step with the analytic model's picks alone (reported beside `value`) -------------
+    model_only_us = None
+    if a.tune > 0:
+        tdc_amd.set_autotune(0)
+        mplans = [Conv2dPlan(1, l["r1"], l["r2"], l["hw"], l["hw"], 3, 3, 1, 1).set_weights(l["wc"]) for l in layers]
+        tdc_amd.set_autotune(a.tune)
+        time_many_ms(mplans, xs, outs, iters=max(a.warmup, 1), graph=graph)
+        model_only_us = time_many_ms(mplans, xs, outs, iters=a.steps, graph=graph) / a.steps * 1e3 / len(layers)
+        for l, mp in zip(layers, mplans):
+            l["model_tile"] = list(mp.info.tile.astuple())
+            mp.close()
+
     # -- per-layer device time and roofline fraction ------------------------------
     table = []
     for l in layers:
@@ -143,6 +165,8 @@ def main():
         table.append({"H": l["hw"], "R1": l["r1"], "R2": l["r2"], "us": round(us, 3),
                       "roof_us": round(info.roof_us, 4), "frac": round(info.roof_us / us, 4),
                       "gflops": round(info.flops / us * 1e-3, 1), "tile": list(info.tile.astuple())})
+        if l.get("model_tile") and l["model_tile"] != table[-1]["tile"]:
+            table[-1]["model_tile"] = l["model_tile"]
 
     # -- comparator: MIOpen's convolution for the same layers (what torch.nn.functional.conv2d dispatches to on
     #    ROCm), graph-replayed the same way; the reference compares against cuDNN the same way
@@ -205,7 +229,11 @@ def main():
         "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "core-conv sweep: 28 layers, batch 1, fp32 NCHW, 3x3 s1 p1, H=W in {7,14,28,56} x "
                                "7 rank pairs; one step = one pass over all 28 layers",
-                   "launch": "HIP graph replay" if graph else "stream launches", "layers_per_step": len(layers)},
+                   "launch": "HIP graph replay" if graph else "stream launches", "layers_per_step": len(layers),
+                   "tile_selection": ("measured at plan creation: the model's favourite tile of each of the %d most "
+                                      "promising tile classes is timed, the fastest kept" % a.tune) if a.tune > 0
+                   else "analytic model"},
+        "model_only_us_per_layer": None if model_only_us is None else round(model_only_us, 4),
         "roofline": roofline,
         "geomean_frac": round(float(torch.tensor([t["frac"] for t in table]).log().mean().exp()), 4),
         "layers": table,

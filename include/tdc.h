@@ -276,6 +276,15 @@ int tdc_model_select_with_tail(const tdc_conv_desc *desc, int32_t tail_N, tdc_ti
  * process-wide, not thread-safe against concurrent model calls. */
 int tdc_model_get_constants(double *values_out, int32_t cap, int32_t *count_out);
 int tdc_model_set_constants(const double *values, int32_t count);
+/* Measured tile selection, process-wide.  With classes > 0 every plan created WITHOUT a forced tile (single
+ * convolutions, the plans inside a tdc_tkconv, the layers of a tdc_net) times, on the device and with synthetic
+ * data, the model's favourite tile of each of the `classes` most promising tile classes (same wave split, register
+ * blocking and tile width) and keeps the fastest; the answer is remembered per problem for the life of the process.
+ * The counterpart of the reference's measured oracle pick (2080Ti-evaluation/TDC-LAYERS-ORACLE/
+ * gen_from_occupancy.py:51-66: the fastest row of the occupancy sweep), restricted to what the model cannot tell
+ * apart.  0 (the default) = the model's pick alone, no device work at plan creation. */
+int tdc_set_autotune(int32_t classes);
+int tdc_get_autotune(void);
 
 #ifdef __cplusplus
 }

@@ -2,10 +2,15 @@
 // reference interfaces each entry point stands in for.
 #include <hip/hip_runtime_api.h>
 
+#include <algorithm>
+#include <array>
+#include <atomic>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <map>
 #include <memory>
+#include <mutex>
 #include <new>
 #include <string>
 #include <vector>
@@ -157,6 +162,96 @@ int tdc_model_set_constants(const double *values, int32_t count) {
     return TDC_OK;
 }
 
+// ---- Measured tile selection ------------------------------------------------
+// The model ranks tens of thousands of candidates in milliseconds and is within a few per cent of the measured
+// best on most shapes; where it is not, the better tile is usually the model's favourite of ANOTHER tile class
+// (a different split of the workgroup into waves, or another tile width).  With tuning switched on, a plan
+// created without a forced tile times the model's favourite of each of the `g_autotune` most promising classes
+// on the device (synthetic data; the timing does not depend on values) and keeps the fastest.  This is the
+// reference's measure-every-tile oracle (2080Ti-evaluation/TDC-LAYERS-ORACLE/gen_from_occupancy.py:51-66) cut
+// down to the candidates the model cannot tell apart.  Results are remembered per problem for the life of the
+// process.
+static std::atomic<int> g_autotune{0};
+static std::mutex g_tune_mutex;
+static std::map<std::array<int, 16>, tdc_tile> g_tuned;
+
+static int tune_tile(const tdc_conv_desc &d, int tail_N, int tail_has_bias, int tail_relu, int classes, tdc_tile &best_out) {
+    const std::array<int, 16> key{d.batch, d.C, d.N, d.H, d.W, d.KH, d.KW, d.stride, d.pad, d.dilation,
+                                  d.has_bias, d.relu, tail_N, tail_has_bias, tail_relu, classes};
+    {
+        std::lock_guard<std::mutex> lock(g_tune_mutex);
+        auto hit = g_tuned.find(key);
+        if (hit != g_tuned.end()) {
+            best_out = hit->second;
+            return TDC_OK;
+        }
+    }
+    // the model's favourite per class (waves and register blocks, tile width), classes in order of promise
+    std::map<std::array<int, 7>, tdc_tile_info> per_class;
+    for (const tdc_tile &t : model_enumerate(d, tail_N)) {
+        tdc_tile_info info;
+        if (!model_evaluate(d, t, info, nullptr, tail_N)) continue;
+        const std::array<int, 7> cls{t.mf, t.mb, t.nb, t.wm, t.wn, t.wk, t.tw};
+        auto it = per_class.find(cls);
+        if (it == per_class.end() || info.pred_us < it->second.pred_us) per_class[cls] = info;
+    }
+    if (per_class.empty()) return fail(TDC_ERR_UNSUPPORTED, "no launchable tile for this shape");
+    std::vector<tdc_tile_info> cands;
+    for (const auto &kv : per_class) cands.push_back(kv.second);
+    std::sort(cands.begin(), cands.end(), [](const tdc_tile_info &a, const tdc_tile_info &b) { return a.pred_us < b.pred_us; });
+    if ((int)cands.size() > classes) cands.resize(classes);
+    while (cands.size() > 1 && cands.back().pred_us > 1.3 * cands.front().pred_us) cands.pop_back();
+
+    const long long Ho = (d.H + 2LL * d.pad - (long long)d.dilation * (d.KH - 1) - 1) / d.stride + 1;
+    const long long Wo = (d.W + 2LL * d.pad - (long long)d.dilation * (d.KW - 1) - 1) / d.stride + 1;
+    const size_t in_bytes = (size_t)d.batch * d.C * d.H * d.W * sizeof(float);
+    const size_t out_bytes = (size_t)d.batch * (tail_N > 0 ? tail_N : d.N) * Ho * Wo * sizeof(float);
+    float *d_in = nullptr, *d_out = nullptr;
+    hipError_t e = hipMalloc((void **)&d_in, in_bytes);
+    if (e == hipSuccess) e = hipMalloc((void **)&d_out, out_bytes);
+    if (e == hipSuccess) e = hipMemset(d_in, 0x3c, in_bytes);   // every float = 0.0115
+    int st = e == hipSuccess ? TDC_OK : hip_fail("hipMalloc(tuning buffers)", e);
+    double best_us = 1e30;
+    for (size_t i = 0; i < cands.size() && st == TDC_OK; ++i) {
+        tdc_conv_plan *plan = nullptr;
+        st = tdc_conv_plan_create_with_tail(&d, tail_N, tail_has_bias, tail_relu, &cands[i].tile, &plan);
+        if (st != TDC_OK) break;
+        e = hipMemset(plan->d_wpk, 0x3c, packed_weight_floats(plan->geo) * sizeof(float));
+        if (e == hipSuccess && plan->d_bias) e = hipMemset(plan->d_bias, 0, (size_t)d.N * sizeof(float));
+        if (e == hipSuccess && plan->d_tail_w)
+            e = hipMemset(plan->d_tail_w, 0x3c, (size_t)((tail_N + 15) / 16) * plan->geo.tail_ng * 64 * sizeof(float));
+        if (e == hipSuccess && plan->d_tail_bias) e = hipMemset(plan->d_tail_bias, 0, (size_t)tail_N * sizeof(float));
+        if (e != hipSuccess) st = hip_fail("hipMemset(tuning weights)", e);
+        plan->have_weights = plan->have_tail_weights = true;
+        double us = 1e30;
+        for (int rep = 0; rep < 4 && st == TDC_OK; ++rep) {   // the first repetition warms up
+            float ms = 0.0f;
+            st = tdc_conv_time(plan, d_in, nullptr, d_out, 20, 1, &ms);
+            if (rep > 0) us = std::min(us, (double)ms * 1e3 / 20);
+        }
+        tdc_conv_plan_destroy(plan);
+        // the model's own favourite (first in the list) is only given up for a clear win: timings repeat to about 1 %
+        if (st == TDC_OK && (i == 0 || us < 0.985 * best_us)) {
+            best_us = us;
+            best_out = cands[i].tile;
+        }
+    }
+    if (d_in) (void)hipFree(d_in);
+    if (d_out) (void)hipFree(d_out);
+    if (st != TDC_OK) return st;
+    std::lock_guard<std::mutex> lock(g_tune_mutex);
+    g_tuned[key] = best_out;
+    return TDC_OK;
+}
+
+int tdc_set_autotune(int32_t classes) {
+    if (classes < 0 || classes > 256) return fail(TDC_ERR_INVALID, "autotune classes must be in [0, 256]");
+    g_autotune.store(classes);
+    return TDC_OK;
+}
+
+int tdc_get_autotune(void) { return g_autotune.load(); }
+
 int tdc_conv_plan_create(const tdc_conv_desc *desc, const tdc_tile *forced_tile, tdc_conv_plan **plan_out) {
     return tdc_conv_plan_create_with_tail(desc, 0, 0, 0, forced_tile, plan_out);
 }
@@ -180,6 +275,11 @@ int tdc_conv_plan_create_with_tail(const tdc_conv_desc *desc, int32_t tail_N, in
     p->tail_relu = tail_N > 0 && tail_relu;
     if (forced_tile) {
         if (!model_evaluate(*desc, *forced_tile, p->info, &why, tail_N)) return fail(TDC_ERR_INVALID, "forced tile: " + why);
+    } else if (g_autotune.load() > 0) {
+        tdc_tile tuned{};
+        const int st = tune_tile(*desc, tail_N, p->tail_has_bias, p->tail_relu, g_autotune.load(), tuned);
+        if (st != TDC_OK) return st;
+        if (!model_evaluate(*desc, tuned, p->info, &why, tail_N)) return fail(TDC_ERR_INVALID, "tuned tile: " + why);
     } else {
         if (!model_select(*desc, p->info, &why, tail_N)) return fail(TDC_ERR_UNSUPPORTED, why);
     }

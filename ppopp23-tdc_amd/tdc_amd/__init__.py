@@ -1,9 +1,9 @@
 """MI355X-native Tucker convolution (TDC hot path) — Python host layer over libtdc_amd.so."""
 from ._lib import (LIB_PATH, ConvDesc, TdcError, Tile, TileInfo, conv_desc, lib, model_enumerate, model_evaluate,
-                   model_select)
+                   model_select, set_autotune)
 
 __all__ = ["LIB_PATH", "ConvDesc", "TdcError", "Tile", "TileInfo", "conv_desc", "lib", "model_enumerate",
-           "model_evaluate", "model_select", "Conv2dPlan", "TKConvOp", "TKConv2dC", "ranks_dict", "partial_tucker2"]
+           "model_evaluate", "model_select", "set_autotune", "Conv2dPlan", "TKConvOp", "TKConv2dC", "ranks_dict", "partial_tucker2"]
 
 
 def __getattr__(name):

@@ -25,7 +25,7 @@ EXPORTS = (
     "tdc_tkconv_create", "tdc_tkconv_set_weights", "tdc_tkconv_forward", "tdc_tkconv_forward_features",
     "tdc_tkconv_core_forward", "tdc_tkconv_query", "tdc_tkconv_num_kernels", "tdc_tkconv_destroy",
     "tdc_model_evaluate", "tdc_model_enumerate", "tdc_model_select", "tdc_model_select_with_tail", "tdc_model_get_constants",
-    "tdc_model_set_constants",
+    "tdc_model_set_constants", "tdc_set_autotune", "tdc_get_autotune",
     "tdc_net_create", "tdc_net_tensor", "tdc_net_view", "tdc_net_affine", "tdc_net_affine_conv", "tdc_net_conv", "tdc_net_conv_tail", "tdc_net_set_input_affine", "tdc_net_tkconv", "tdc_net_pool", "tdc_net_global_avgpool", "tdc_net_concat",
     "tdc_net_tensor_shape", "tdc_net_num_kernels", "tdc_net_finalize", "tdc_net_forward", "tdc_net_time",
     "tdc_net_read_tensor", "tdc_net_destroy",
@@ -134,6 +134,8 @@ def lib():
     L.tdc_net_read_tensor.argtypes = [c_void_p, i32, c_void_p]
     L.tdc_net_destroy.argtypes = [c_void_p]
     L.tdc_net_destroy.restype = None
+    L.tdc_set_autotune.argtypes = [i32]
+    L.tdc_get_autotune.argtypes = []
     for name in EXPORTS:
         fn = getattr(L, name)
         if fn.restype is c_int:  # default restype: status code
@@ -200,6 +202,15 @@ def model_get_constants():
 def model_set_constants(values):
     arr = (c_double * len(values))(*values)
     check(lib().tdc_model_set_constants(arr, len(values)))
+
+
+def set_autotune(classes: int):
+    """Measured tile selection for every plan created from now on without a forced tile: time the model's
+    favourite of each of the `classes` most promising tile classes on the device and keep the fastest
+    (0 = the model's pick alone, the default).  Returns the previous setting."""
+    prev = lib().tdc_get_autotune()
+    check(lib().tdc_set_autotune(int(classes)))
+    return prev
 
 
 def model_enumerate(desc: ConvDesc, cap: int = 1 << 17):

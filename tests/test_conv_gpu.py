@@ -145,6 +145,38 @@ def test_extreme_shapes_model_tile(B, C, N, H, W, K, stride, pad):
     assert_close(got, ref.conv2d_torch(x, w, stride=stride, pad=pad).numpy(), f"extreme {(B, C, N, H, W, K)}")
 
 
+def test_measured_tile_selection():
+    """With tuning on, a plan without a forced tile gets a measured pick: results stay within tolerance, the pick
+    is one of the launchable tiles, a second plan of the same problem reuses it, and a forced tile is still obeyed."""
+    prev = tdc_amd.set_autotune(6)
+    try:
+        assert tdc_amd.lib().tdc_get_autotune() == 6
+        for (C, N, hw, K, stride, pad) in ((64, 64, 28, 3, 1, 1), (48, 200, 14, 1, 1, 0), (3, 16, 40, 7, 2, 3)):
+            announce("tuned", C, N, hw, K, stride, pad)
+            x, w = case(8100 + C, 1, C, N, hw, hw, K)
+            want = ref.conv2d_torch(x, w, stride=stride, pad=pad).numpy()
+            picks = []
+            for _ in range(2):
+                plan = tdc_amd.Conv2dPlan(1, C, N, hw, hw, K, K, stride, pad).set_weights(w)
+                out = torch.full((1, N, plan.Ho, plan.Wo), float("nan"), device="cuda")
+                plan.forward(x.cuda(), out=out)
+                torch.cuda.synchronize()
+                assert_close(out.cpu().numpy(), want, f"tuned {(C, N, hw, K)}")
+                picks.append(plan.info.tile.astuple())
+                plan.close()
+            assert picks[0] == picks[1]
+            desc = tdc_amd.conv_desc(1, C, N, hw, hw, K, K, stride, pad)
+            assert picks[0] in [t.astuple() for t in tdc_amd.model_enumerate(desc)]
+            forced = tdc_amd.model_select(desc).tile
+            plan = tdc_amd.Conv2dPlan(1, C, N, hw, hw, K, K, stride, pad, tile=forced)
+            assert plan.info.tile.astuple() == forced.astuple()
+            plan.close()
+    finally:
+        tdc_amd.set_autotune(prev)
+    with pytest.raises(tdc_amd.TdcError):
+        tdc_amd.set_autotune(-1)
+
+
 def test_stride2_resnet_core_shapes():
     """The three stride-2 core convs of Tucker ResNet-18 (64->64 56->28, 128->128 28->14, 256->256 14->7)."""
     for r, hw in ((64, 56), (128, 28), (256, 14)):
