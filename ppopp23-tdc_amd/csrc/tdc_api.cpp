@@ -84,6 +84,9 @@ struct tdc_tkconv {
     size_t f1_floats = 0, f2_floats = 0;
 };
 
+static int time_plans(tdc_conv_plan *const *plans, const float *const *d_ins, float *const *d_outs, int n, int passes,
+                      int iters, int use_graph, float *total_ms_out);
+
 extern "C" {
 
 const char *tdc_last_error_string(void) { return g_last_error.c_str(); }
@@ -175,6 +178,27 @@ static std::atomic<int> g_autotune{0};
 static std::mutex g_tune_mutex;
 static std::map<std::array<int, 16>, tdc_tile> g_tuned;
 
+// Timing runs need weights in place but not their values: fill the packed buffers with a constant (every float
+// 0.0115) and mark the plan ready; `ready = false` afterwards makes the plan ask for real weights again.
+static int synthetic_weights(tdc_conv_plan *plan, bool ready) {
+    if (ready) {
+        hipError_t e = hipMemset(plan->d_wpk, 0x3c, packed_weight_floats(plan->geo) * sizeof(float));
+        if (e == hipSuccess && plan->d_bias) e = hipMemset(plan->d_bias, 0, (size_t)plan->desc.N * sizeof(float));
+        if (e == hipSuccess && plan->d_tail_w)
+            e = hipMemset(plan->d_tail_w, 0x3c, (size_t)((plan->tail_N + 15) / 16) * plan->geo.tail_ng * 64 * sizeof(float));
+        if (e == hipSuccess && plan->d_tail_bias) e = hipMemset(plan->d_tail_bias, 0, (size_t)plan->tail_N * sizeof(float));
+        if (e != hipSuccess) return hip_fail("hipMemset(synthetic weights)", e);
+    }
+    plan->have_weights = ready;
+    plan->have_tail_weights = ready && plan->tail_N > 0;
+    return TDC_OK;
+}
+
+static bool log_tuning() {
+    static const bool on = std::getenv("TDC_LOG_TUNING") != nullptr;
+    return on;
+}
+
 static int tune_tile(const tdc_conv_desc &d, int tail_N, int tail_has_bias, int tail_relu, int classes, tdc_tile &best_out) {
     const std::array<int, 16> key{d.batch, d.C, d.N, d.H, d.W, d.KH, d.KW, d.stride, d.pad, d.dilation,
                                   d.has_bias, d.relu, tail_N, tail_has_bias, tail_relu, classes};
@@ -216,13 +240,7 @@ static int tune_tile(const tdc_conv_desc &d, int tail_N, int tail_has_bias, int 
         tdc_conv_plan *plan = nullptr;
         st = tdc_conv_plan_create_with_tail(&d, tail_N, tail_has_bias, tail_relu, &cands[i].tile, &plan);
         if (st != TDC_OK) break;
-        e = hipMemset(plan->d_wpk, 0x3c, packed_weight_floats(plan->geo) * sizeof(float));
-        if (e == hipSuccess && plan->d_bias) e = hipMemset(plan->d_bias, 0, (size_t)d.N * sizeof(float));
-        if (e == hipSuccess && plan->d_tail_w)
-            e = hipMemset(plan->d_tail_w, 0x3c, (size_t)((tail_N + 15) / 16) * plan->geo.tail_ng * 64 * sizeof(float));
-        if (e == hipSuccess && plan->d_tail_bias) e = hipMemset(plan->d_tail_bias, 0, (size_t)tail_N * sizeof(float));
-        if (e != hipSuccess) st = hip_fail("hipMemset(tuning weights)", e);
-        plan->have_weights = plan->have_tail_weights = true;
+        st = synthetic_weights(plan, true);
         double us = 1e30;
         for (int rep = 0; rep < 4 && st == TDC_OK; ++rep) {   // the first repetition warms up
             float ms = 0.0f;
@@ -239,6 +257,10 @@ static int tune_tile(const tdc_conv_desc &d, int tail_N, int tail_has_bias, int 
     if (d_in) (void)hipFree(d_in);
     if (d_out) (void)hipFree(d_out);
     if (st != TDC_OK) return st;
+    if (log_tuning())
+        std::fprintf(stderr, "tdc tune: conv %dx%d C%d N%d %dx%d s%d tail %d: %zu classes timed, best %.2f us (model's pick %s)\n",
+                     d.KH, d.KW, d.C, d.N, d.H, d.W, d.stride, tail_N, cands.size(), best_us,
+                     std::memcmp(&best_out, &cands[0].tile, sizeof(tdc_tile)) == 0 ? "kept" : "replaced");
     std::lock_guard<std::mutex> lock(g_tune_mutex);
     g_tuned[key] = best_out;
     return TDC_OK;
@@ -471,7 +493,17 @@ int tdc_conv_forward_strided(tdc_conv_plan *plan, const float *d_in, int64_t in_
 
 int tdc_conv_time_many(tdc_conv_plan *const *plans, const float *const *d_ins, float *const *d_outs, int32_t n,
                        int32_t iters, int32_t use_graph, float *total_ms_out) {
-    if (!plans || !d_ins || !d_outs || !total_ms_out || n < 1 || iters < 1) return fail(TDC_ERR_INVALID, "bad argument");
+    return time_plans(plans, d_ins, d_outs, n, 1, iters, use_graph, total_ms_out);
+}
+
+}  // extern "C"
+
+// hipEvents around `iters` repetitions of `passes` passes over the list; with `use_graph` the `passes` passes are
+// one HIP graph that is replayed `iters` times.
+static int time_plans(tdc_conv_plan *const *plans, const float *const *d_ins, float *const *d_outs, int n, int passes,
+                      int iters, int use_graph, float *total_ms_out) {
+    if (!plans || !d_ins || !d_outs || !total_ms_out || n < 1 || iters < 1 || passes < 1)
+        return fail(TDC_ERR_INVALID, "bad argument");
     for (int i = 0; i < n; ++i)
         if (!plans[i] || !d_ins[i] || !d_outs[i]) return fail(TDC_ERR_INVALID, "null plan or buffer in list");
     hipStream_t s = nullptr;
@@ -480,7 +512,8 @@ int tdc_conv_time_many(tdc_conv_plan *const *plans, const float *const *d_ins, f
     hipGraphExec_t exec = nullptr;
     int st = TDC_OK;
     auto one_pass = [&]() {
-        for (int i = 0; i < n && st == TDC_OK; ++i) st = tdc_conv_forward(plans[i], d_ins[i], nullptr, d_outs[i], s);
+        for (int k = 0; k < passes; ++k)
+            for (int i = 0; i < n && st == TDC_OK; ++i) st = tdc_conv_forward(plans[i], d_ins[i], nullptr, d_outs[i], s);
     };
     const char *what = "hipStreamCreate";
     hipError_t e = hipDeviceSynchronize();
@@ -519,6 +552,8 @@ int tdc_conv_time_many(tdc_conv_plan *const *plans, const float *const *d_ins, f
     if (e != hipSuccess) return hip_fail(what, e);
     return TDC_OK;
 }
+
+extern "C" {
 
 int tdc_conv_time(tdc_conv_plan *plan, const float *d_in, const float *d_residual, float *d_out, int32_t iters,
                   int32_t use_graph, float *total_ms_out) {
@@ -575,6 +610,66 @@ void tdc_conv_plan_destroy(tdc_conv_plan *plan) {
 
 // ---- TKConv ---------------------------------------------------------------
 
+// Core + last factor: one fused launch or two?  Times both on the operator's own intermediates (synthetic
+// weights) and drops the fused plan when the two launches are not slower.  Remembered per problem.
+static std::map<std::array<int, 13>, bool> g_fusion_pays;
+
+static int tkconv_measure_fusion(tdc_tkconv *op) {
+    const tdc_tkconv_desc &d = op->desc;
+    const std::array<int, 13> key{d.batch, d.C, d.R1, d.R2, d.N, d.H, d.W, d.K, d.stride, d.pad, d.dilation, d.has_bias, d.relu};
+    bool known = false, pays = false;
+    {
+        std::lock_guard<std::mutex> lock(g_tune_mutex);
+        auto hit = g_fusion_pays.find(key);
+        if (hit != g_fusion_pays.end()) {
+            known = true;
+            pays = hit->second;
+        }
+    }
+    if (!known) {
+        const size_t out_floats = (size_t)d.batch * d.N * (op->f2_floats / ((size_t)d.batch * d.R2));
+        float *d_out = nullptr;
+        hipError_t e = hipMalloc((void **)&d_out, out_floats * sizeof(float));
+        if (e == hipSuccess) e = hipMemset(op->d_f1, 0x3c, op->f1_floats * sizeof(float));
+        if (e != hipSuccess) {
+            if (d_out) (void)hipFree(d_out);
+            return hip_fail("hipMalloc(fusion timing)", e);
+        }
+        int st = synthetic_weights(op->core, true);
+        if (st == TDC_OK) st = synthetic_weights(op->last, true);
+        if (st == TDC_OK) st = synthetic_weights(op->core_last, true);
+        tdc_conv_plan *two[2] = {op->core, op->last};
+        const float *ins[2] = {op->d_f1, op->d_f2};
+        float *outs[2] = {op->d_f2, d_out};
+        tdc_conv_plan *one[1] = {op->core_last};
+        double us_two = 1e30, us_one = 1e30;
+        for (int rep = 0; rep < 4 && st == TDC_OK; ++rep) {   // the first repetition warms up
+            float ms = 0.0f;
+            // ten passes per graph: a graph launch costs more than one of these kernels
+            st = time_plans(two, ins, outs, 2, 10, 2, 1, &ms);
+            if (st == TDC_OK && rep > 0) us_two = std::min(us_two, (double)ms * 1e3 / 20);
+            if (st == TDC_OK) st = time_plans(one, ins, outs + 1, 1, 10, 2, 1, &ms);
+            if (st == TDC_OK && rep > 0) us_one = std::min(us_one, (double)ms * 1e3 / 20);
+        }
+        (void)hipFree(d_out);
+        synthetic_weights(op->core, false);
+        synthetic_weights(op->last, false);
+        synthetic_weights(op->core_last, false);
+        if (st != TDC_OK) return st;
+        pays = us_one < us_two;
+        if (log_tuning())
+            std::fprintf(stderr, "tdc tune: tkconv C%d R%d,%d N%d %dx%d K%d s%d: core+last fused %.2f us, separate %.2f us\n",
+                         d.C, d.R1, d.R2, d.N, d.H, d.W, d.K, d.stride, us_one, us_two);
+        std::lock_guard<std::mutex> lock(g_tune_mutex);
+        g_fusion_pays[key] = pays;
+    }
+    if (!pays) {
+        tdc_conv_plan_destroy(op->core_last);
+        op->core_last = nullptr;
+    }
+    return TDC_OK;
+}
+
 int tdc_tkconv_create(const tdc_tkconv_desc *desc, tdc_tkconv **op_out) {
     if (!desc || !op_out) return fail(TDC_ERR_INVALID, "null argument");
     *op_out = nullptr;
@@ -615,10 +710,14 @@ int tdc_tkconv_create(const tdc_tkconv_desc *desc, tdc_tkconv **op_out) {
     // forward_features and core_forward.
     if (!std::getenv("TDC_EXPERIMENT_NO_FUSED_TAIL")) {
         tdc_tile_info fused{};
-        if (model_select(d2, fused, nullptr, desc->N) &&
-            fused.pred_us < op->core->info.pred_us + op->last->info.pred_us) {
+        const double separate_us = op->core->info.pred_us + op->last->info.pred_us;
+        const bool measure = g_autotune.load() > 0;
+        // With measured selection on, a fused kernel predicted within 30 % of the two launches is built and the
+        // two alternatives are timed; otherwise the prediction decides.
+        if (model_select(d2, fused, nullptr, desc->N) && fused.pred_us < (measure ? 1.3 : 1.0) * separate_us) {
             st = tdc_conv_plan_create_with_tail(&d2, desc->N, desc->has_bias, desc->relu, nullptr, &op->core_last);
             if (st != TDC_OK) { cleanup(); return st; }
+            if (measure && (st = tkconv_measure_fusion(op.get())) != TDC_OK) { cleanup(); return st; }
         }
     }
     *op_out = op.release();

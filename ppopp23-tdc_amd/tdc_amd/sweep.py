@@ -74,6 +74,8 @@ def main(argv=None):
     ap.add_argument("--offset", type=int, default=0, help="first candidate of the thinned list")
     ap.add_argument("--net", choices=("resnet18", "densenet121"), default=None,
                     help="sweep the distinct convolution shapes of a whole network instead of the core-conv layers")
+    ap.add_argument("--shapes", nargs="*", default=None, metavar="C,N,H,W,K,stride,pad",
+                    help="sweep these convolution shapes instead")
     ap.add_argument("--hw", type=int, nargs="*", default=list(SWEEP_HW))
     a = ap.parse_args(argv)
     if not torch.cuda.is_available():
@@ -84,7 +86,11 @@ def main(argv=None):
     total = 0.0
     n = 0
     t0 = time.time()
-    if a.net:
+    if a.shapes:
+        shapes = [tuple(int(v) for v in sh.split(",")) for sh in a.shapes]
+        if any(len(sh) != 7 for sh in shapes):
+            sys.exit("--shapes: every shape is C,N,H,W,K,stride,pad")
+    elif a.net:
         from . import nets
         if a.net == "resnet18":
             net = nets.build_tucker_resnet18(nets.resnet18_params())
