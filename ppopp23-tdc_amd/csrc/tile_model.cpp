@@ -246,16 +246,16 @@ namespace {
 // (2080Ti-evaluation/TDC-LAYERS-MODELING/model.py:265-266,278).
 struct ModelConst {
     double launch_us = 1.474;           // device time of an empty kernel in a back-to-back stream
-    double setup_clk = 1007;          // kernel arguments and index arithmetic before the first copy is issued
+    double setup_clk = 1208;          // kernel arguments and index arithmetic before the first copy is issued
     double copy_latency_clk = 920.5;   // first byte of a global->LDS copy (L2 / memory-side cache)
-    double copy_bytes_per_clk = 33.65;   // sustained global->LDS rate of one CU
+    double copy_bytes_per_clk = 34.32;   // sustained global->LDS rate of one CU
     double l2_bytes_per_clk = 9627;   // whole-chip L2->CU rate when every CU copies at once
-    double lds_bytes_per_clk = 21.79;   // LDS traffic of the split-K reduction
-    double sync_clk = 224.8;            // one workgroup barrier
-    double store_bytes_per_clk = 2.718;  // per CU, short runs per channel
-    double kstep_issue_clk = 2.743;      // vector-ALU / LDS-issue cycles per operand read, not hidden under MFMAs
+    double lds_bytes_per_clk = 22.23;   // LDS traffic of the split-K reduction
+    double sync_clk = 229.3;            // one workgroup barrier
+    double store_bytes_per_clk = 2.772;  // per CU, short runs per channel
+    double kstep_issue_clk = 2.798;      // vector-ALU / LDS-issue cycles per operand read, not hidden under MFMAs
     double pass_overhead_clk = 578.7;   // per wave and pass: copy issue, pointer set-up, pipeline fill
-    double wave_setup_clk = 772.2;      // prologue cycles added per extra wave sharing a SIMD
+    double wave_setup_clk = 540.5;      // prologue cycles added per extra wave sharing a SIMD
     double ksplit_clk = 4604;         // split across workgroups: write-through, ticket round trip, read-back
     double copy_issue_clk = 118.2;      // a wave is held this long by every global->LDS copy instruction it issues
     double lds_read_clk = 2.88;        // LDS busy cycles per conflict-free operand read of one wave
