@@ -282,7 +282,8 @@ int tdc_model_set_constants(const double *values, int32_t count);
  * blocking and tile width) and keeps the fastest; the answer is remembered per problem for the life of the process.
  * The counterpart of the reference's measured oracle pick (2080Ti-evaluation/TDC-LAYERS-ORACLE/
  * gen_from_occupancy.py:51-66: the fastest row of the occupancy sweep), restricted to what the model cannot tell
- * apart.  0 (the default) = the model's pick alone, no device work at plan creation. */
+ * apart.  0 (the default) = the model's pick alone, no device work at plan creation.  The environment variable
+ * TDC_AUTOTUNE=k sets the initial value when the library is loaded. */
 int tdc_set_autotune(int32_t classes);
 int tdc_get_autotune(void);
 

@@ -174,7 +174,12 @@ int tdc_model_set_constants(const double *values, int32_t count) {
 // reference's measure-every-tile oracle (2080Ti-evaluation/TDC-LAYERS-ORACLE/gen_from_occupancy.py:51-66) cut
 // down to the candidates the model cannot tell apart.  Results are remembered per problem for the life of the
 // process.
-static std::atomic<int> g_autotune{0};
+static int autotune_from_env() {
+    const char *e = std::getenv("TDC_AUTOTUNE");
+    const int v = e ? std::atoi(e) : 0;
+    return v < 0 ? 0 : (v > 256 ? 256 : v);
+}
+static std::atomic<int> g_autotune{autotune_from_env()};   // TDC_AUTOTUNE=k in the environment = tdc_set_autotune(k) at load
 static std::mutex g_tune_mutex;
 static std::map<std::array<int, 16>, tdc_tile> g_tuned;
 
