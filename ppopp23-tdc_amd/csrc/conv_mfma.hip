@@ -87,7 +87,13 @@ struct Mfma<16> {
     static __device__ __forceinline__ int ksub(int lane) { return lane >> 4; }
 };
 
-enum : int { TAPS_GENERIC = 0, TAPS_1x1 = 1, TAPS_3x3 = 9 };
+// TAPS_WINO: 3x3 / stride 1 as Winograd F(2x2,3x3).  A pixel lane holds one 2x2 output tile; per four input
+// channels a wave reads the 4x4 input patch of its tile from the SAME zero-haloed LDS window the direct path
+// uses, transforms it in registers (V = B^T d B, 32 additions), and feeds 16 MFMAs — one per position of the
+// transformed domain, against weights U = G g G^T prepared on the host — where the direct path needs 36 for
+// the same four pixels.  The 16 accumulators of a lane are combined at the end (Y = A^T M A, in registers:
+// every lane holds all 16 positions of its tile) into the 2x2 outputs.
+enum : int { TAPS_GENERIC = 0, TAPS_1x1 = 1, TAPS_3x3 = 9, TAPS_WINO = 16 };
 
 constexpr int OOB_OFFSET = 0x7ffffff0;  // beyond any buffer: the load returns zero
 
@@ -221,7 +227,8 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
     const int wm = fdiv(wave_nk, p.fd_wn);
     const int wn = wave_nk - wm * p.WN;
 
-    const int PT = MF * NB * p.WN;  // pixel lanes of the workgroup (>= TH*TW)
+    // pixel lanes of the workgroup (>= TH*TW); a Winograd lane stands for 2x2 pixels
+    const int PT = (TAPS == TAPS_WINO ? 4 : 1) * MF * NB * p.WN;
     const int MT = MF * MB * p.WM;
     // Workgroups are handed to the eight compute dies (XCDs, each with its own L2) round-robin by launch
     // index.  The launch is one-dimensional and the index is re-read as (die, slot), so that each die
@@ -324,6 +331,26 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
         boff[nb] = jy * p.stride * p.RS + jx * p.stride + (ix0 - ix0a) + M::ksub(lane) * p.CS;
     }
 
+    // Winograd: LDS offset of the top-left element of this lane's 4x4 input patch, and whether the lane's tile
+    // exists (lanes past the workgroup tile re-read its last row of tiles and are never stored).
+    int wino_off = 0, wino_ty = 0, wino_tx = 0;
+    bool wino_live = false;
+    if constexpr (TAPS == TAPS_WINO) {
+        const int j = wn * 16 + (lane & 15);
+        const int tht = p.TH >> 1;
+        int ty = fdiv(j, p.fd_wtw);
+        wino_tx = j - ty * (p.TW >> 1);
+        wino_live = ty < tht && !loader;
+        ty = min(ty, tht - 1);
+        wino_ty = ty;
+        wino_off = 2 * ty * p.RS + 2 * wino_tx + (ix0 - ix0a) + (lane >> 4) * p.CS;
+    }
+    f4_t wacc[TAPS == TAPS_WINO ? 16 : 1];
+    if constexpr (TAPS == TAPS_WINO) {
+#pragma unroll
+        for (int x = 0; x < 16; ++x) wacc[x] = (f4_t){0.0f, 0.0f, 0.0f, 0.0f};
+    }
+
     acc_t acc[MB][NB];
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
@@ -403,7 +430,74 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
         for (int mb = 0; mb < MB; ++mb)
             sw[mb] = stage + p.in_stage_floats + (((wm * MB + mb) * ncg_pass + wk * ncgw) * taps) * 64 + lane;
 
-        if constexpr (TAPS == TAPS_3x3) {
+        if constexpr (TAPS == TAPS_WINO) {
+            // One group = four input channels: 16 raw patch values per lane (8 two-word LDS reads), the 16 A
+            // operands (four 128-bit reads), the register transform, 16 MFMAs.  Two register sets ping-pong as
+            // in the direct loops: patch and weights of group g+1 are read, and the patch transformed, between the
+            // MFMAs of group g.
+            static_assert(TAPS != TAPS_WINO || (MF == 16 && MB == 1 && NB == 1), "Winograd path: one 16x16 block per wave");
+            const float *praw = sin + wino_off;
+            const float *pw = stage + p.in_stage_floats + ((wm * ncg_pass + wk * ncgw) * 16) * 64 + lane * 4;
+            const int RS = p.RS;
+            const int gstep = KC * p.CS;
+            float v0[16], v1[16];
+            f4_t u0[4], u1[4];
+            auto load_group = [&](int g, float(&v)[16], f4_t(&u)[4]) {
+                const float *b = praw + g * gstep;
+                float d[4][4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) d[r][c] = b[r * RS + c];
+#pragma unroll
+                for (int q = 0; q < 4; ++q) u[q] = *reinterpret_cast<const f4_t *>(pw + (g * 16 + q * 4) * 64);
+                float tr[4][4];   // B^T d: rows
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    tr[0][c] = d[0][c] - d[2][c];
+                    tr[1][c] = d[1][c] + d[2][c];
+                    tr[2][c] = d[2][c] - d[1][c];
+                    tr[3][c] = d[1][c] - d[3][c];
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {   // (B^T d) B: columns
+                    v[i * 4 + 0] = tr[i][0] - tr[i][2];
+                    v[i * 4 + 1] = tr[i][1] + tr[i][2];
+                    v[i * 4 + 2] = tr[i][2] - tr[i][1];
+                    v[i * 4 + 3] = tr[i][1] - tr[i][3];
+                }
+            };
+            auto mfma_group = [&](const float(&v)[16], const f4_t(&u)[4]) {
+#pragma unroll
+                for (int x = 0; x < 16; ++x)
+                    wacc[x] = __builtin_amdgcn_mfma_f32_16x16x4f32(u[x >> 2][x & 3], v[x], wacc[x], 0, 0, 0);
+            };
+            auto interleave = [&]() {
+#pragma unroll
+                for (int x = 0; x < 12; ++x) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // LDS read
+                }
+#pragma unroll
+                for (int x = 0; x < 4; ++x) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x002, 8, 0);  // the transform's vector ALU work
+                }
+            };
+            load_group(0, v0, u0);
+            for (int g = 0; g + 1 < ncgw; g += 2) {
+                __builtin_amdgcn_sched_barrier(0);
+                load_group(g + 1, v1, u1);
+                mfma_group(v0, u0);
+                interleave();
+                __builtin_amdgcn_sched_barrier(0);
+                load_group(min(g + 2, ncgw - 1), v0, u0);
+                mfma_group(v1, u1);
+                interleave();
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (ncgw & 1) mfma_group(v0, u0);
+        } else if constexpr (TAPS == TAPS_3x3) {
             // dilation 1: the column tap is an immediate offset of the LDS read, the row tap one of
             // three per-lane row addresses.  Two register sets ping-pong: the operands of channel
             // group g+1 are read from LDS before the MFMAs of group g are issued, so the matrix pipe
@@ -557,7 +651,32 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
     }
     // Epilogue.  `each_output(sink)` walks this thread's share of the workgroup's output tile and
     // hands (channel, pixel offset in the image, accumulated value) to the sink.
-    if (p.WK > 1) {
+    if constexpr (TAPS == TAPS_WINO) {
+        // Output transform Y = A^T M A, A^T = [1 1 1 0; 0 1 -1 -1], per accumulator register (= output channel):
+        // all 16 positions of a tile sit in the same lane.  The 2x2 results are parked in LDS as
+        // [wk][channel][pixel of the workgroup tile]; the walk below adds the WK slices in index order and stores
+        // runs of consecutive pixels.
+        __syncthreads();
+        if (wino_live) {
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                float sr[4][2];   // M A: per row i of M
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    sr[i][0] = wacc[i * 4 + 0][v] + wacc[i * 4 + 1][v] + wacc[i * 4 + 2][v];
+                    sr[i][1] = wacc[i * 4 + 1][v] - wacc[i * 4 + 2][v] - wacc[i * 4 + 3][v];
+                }
+                const int ml = wm * 16 + 4 * (lane >> 4) + v;
+                float *dst = lds + (wk * MT + ml) * PT + (2 * wino_ty) * p.TW + 2 * wino_tx;
+#pragma unroll
+                for (int c = 0; c < 2; ++c) {
+                    dst[c] = sr[0][c] + sr[1][c] + sr[2][c];
+                    dst[p.TW + c] = sr[1][c] - sr[2][c] - sr[3][c];
+                }
+            }
+        }
+        __syncthreads();
+    } else if (p.WK > 1) {
         // Split-K across waves: park every wave's partial tile in LDS
         // ([wk][channel][pixel lane]); the walk below adds the WK slices in index order.
         __syncthreads();
@@ -578,7 +697,7 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
         __syncthreads();
     }
     auto each_output = [&](auto &&sink, bool want_value) {
-        if (p.WK == 1) {
+        if (p.WK == 1 && TAPS != TAPS_WINO) {
             // Straight from the accumulators: each store instruction writes runs of
             // consecutive pixels of one output channel.
 #pragma unroll
@@ -803,6 +922,10 @@ static int taps_mode(int KH, int KW, int dil) {
 
 const void *conv_kernel_for(const tdc_tile &t, int KH, int KW, int dilation, bool extras) {
     kernel_fn fn = nullptr;
+    if (t.wino) {
+        if (extras || KH != 3 || KW != 3 || dilation != 1 || t.mf != 16 || t.mb != 1 || t.nb != 1) return nullptr;
+        return reinterpret_cast<const void *>(static_cast<kernel_fn>(tdc_conv_mfma_kernel<16, 1, 1, TAPS_WINO, 8, false>));
+    }
     switch (taps_mode(KH, KW, dilation)) {
         case TAPS_3x3: fn = extras ? pick_mf<TAPS_3x3, true>(t.mf, t.mb, t.nb) : pick_mf<TAPS_3x3, false>(t.mf, t.mb, t.nb); break;
         case TAPS_1x1: fn = extras ? pick_mf<TAPS_1x1, true>(t.mf, t.mb, t.nb) : pick_mf<TAPS_1x1, false>(t.mf, t.mb, t.nb); break;

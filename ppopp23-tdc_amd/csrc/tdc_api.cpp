@@ -216,11 +216,11 @@ static int tune_tile(const tdc_conv_desc &d, int tail_N, int tail_has_bias, int 
         }
     }
     // the model's favourite per class (waves and register blocks, tile width), classes in order of promise
-    std::map<std::array<int, 7>, tdc_tile_info> per_class;
+    std::map<std::array<int, 8>, tdc_tile_info> per_class;
     for (const tdc_tile &t : model_enumerate(d, tail_N)) {
         tdc_tile_info info;
         if (!model_evaluate(d, t, info, nullptr, tail_N)) continue;
-        const std::array<int, 7> cls{t.mf, t.mb, t.nb, t.wm, t.wn, t.wk, t.tw};
+        const std::array<int, 8> cls{t.mf, t.mb, t.nb, t.wm, t.wn, t.wk, t.tw, t.wino};
         auto it = per_class.find(cls);
         if (it == per_class.end() || info.pred_us < it->second.pred_us) per_class[cls] = info;
     }
@@ -481,6 +481,7 @@ int tdc_conv_forward_strided(tdc_conv_plan *plan, const float *d_in, int64_t in_
     kp.fd_tw = make_fastdiv(g.TW);
     kp.fd_ntx = make_fastdiv(g.ntx);
     kp.fd_pt = make_fastdiv(g.PT);
+    kp.fd_wtw = make_fastdiv(g.wino ? g.TWt : 1);
     kp.fd_wk = make_fastdiv(plan->tile.wk);
     kp.fd_wn = make_fastdiv(plan->tile.wn);
     kp.fd_ks = make_fastdiv(g.ks);

@@ -34,6 +34,9 @@ struct Geometry {
     int Ho = 0, Wo = 0, P = 0;       // output height/width (of the kernel's view), Ho*Wo
     int kc = 0;                      // input channels consumed per MFMA (2 or 4)
     int taps = 0;                    // KH*KW
+    int ktaps = 0;                   // K-steps per channel group: taps, or 16 for Winograd F(2x2,3x3)
+    int wino = 0;                    // Winograd: pixel lanes hold 2x2 output tiles
+    int TWt = 0, THt = 0;            // Winograd: the workgroup tile in 2x2 tiles (TW = 2*TWt, TH = 2*THt)
     int PT = 0, MT = 0;              // pixel lanes / output channels per workgroup
     int TW = 0, TH = 0;              // output tile
     int ntx = 0, nty = 0;            // tiles across / down
@@ -128,6 +131,7 @@ struct ConvKParams {
     FastDiv fd_npx;            // 16-pixel blocks per tile
     FastDiv fd_csv, fd_rsv;      // LDS channel slot / row, in copy elements
     FastDiv fd_tw, fd_ntx, fd_pt;
+    FastDiv fd_wtw;            // Winograd: 2x2 tiles per row of the workgroup tile
     FastDiv fd_wk, fd_wn, fd_ks;
     unsigned wpk_bytes;
     unsigned in_image_bytes;   // C*H*W*4: reads at or past it return zero

@@ -114,7 +114,7 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
     if (t.mb < 1 || t.mb > 2 || t.nb < 1 || t.nb > 2) return fail("tile.mb / tile.nb must be 1 or 2");
     if (t.wm < 1 || t.wn < 1 || t.wk < 1) return fail("tile.wm / wn / wk must be >= 1");
     g = Geometry();
-    g.max_waves_kernel = (t.mb == 2 && t.nb == 2) ? 8 : 16;
+    g.max_waves_kernel = ((t.mb == 2 && t.nb == 2) || t.wino == 1) ? 8 : 16;   // 256 registers per lane for those
     if (t.wl < 0 || t.wl > 8) return fail("tile.wl must be in [0, 8]");
     if ((long long)t.wm * t.wn * t.wk + t.wl > g.max_waves_kernel) return fail("too many waves per workgroup for this tile");
     g.waves = t.wm * t.wn * t.wk + t.wl;
@@ -129,11 +129,30 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
     g.P = g.Ho * g.Wo;
     g.kc = (t.mf == 32) ? 2 : 4;
     g.taps = d.KH * d.KW;
-    g.PT = t.mf * t.nb * t.wn;
+    g.ktaps = g.taps;
     g.MT = t.mf * t.mb * t.wm;
-    if (t.tw < 1 || t.tw > g.PT || t.tw > g.Wo) return fail("tile.tw must be in [1, min(Wo, pixel lanes)]");
-    g.TW = t.tw;
-    g.TH = std::min(g.PT / t.tw, g.Ho);
+    if (t.wino != 0 && t.wino != 1) return fail("tile.wino must be 0 or 1");
+    g.wino = t.wino;
+    if (t.wino) {
+        // Winograd F(2x2,3x3): a pixel lane holds one 2x2 output tile; the workgroup tile is THt x TWt such tiles.
+        if (d.KH != 3 || d.KW != 3 || d.stride != 1 || d.dilation != 1) return fail("tile.wino needs a 3x3 / stride 1 / dilation 1 convolution");
+        if (t.mf != 16 || t.mb != 1 || t.nb != 1) return fail("tile.wino needs mf = 16, mb = nb = 1");
+        if (tail_N > 0) return fail("tile.wino cannot carry a fused tail");
+        const int lanes = 16 * t.wn;
+        const int Wt = ceil_div(g.Wo, 2), Ht = ceil_div(g.Ho, 2);
+        if (t.tw < 1 || t.tw > lanes || t.tw > Wt) return fail("tile.tw must be in [1, min(ceil(Wo/2), tile lanes)]");
+        g.ktaps = 16;
+        g.TWt = t.tw;
+        g.THt = std::min(lanes / t.tw, Ht);
+        g.TW = 2 * g.TWt;
+        g.TH = 2 * g.THt;
+        g.PT = 4 * lanes;   // pixels the workgroup's lanes stand for
+    } else {
+        g.PT = t.mf * t.nb * t.wn;
+        if (t.tw < 1 || t.tw > g.PT || t.tw > g.Wo) return fail("tile.tw must be in [1, min(Wo, pixel lanes)]");
+        g.TW = t.tw;
+        g.TH = std::min(g.PT / t.tw, g.Ho);
+    }
     g.ntx = ceil_div(g.Wo, g.TW);
     g.nty = ceil_div(g.Ho, g.TH);
     // (the kernel divides the tile index by ntx with a 32-bit multiply-high)
@@ -170,16 +189,19 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
     } else {
         g.RS = g.ncols;
     }
-    g.CS = pad_channel_stride(g.nrows * g.RS, t.mf, g.VW, g.PT, g.TW, g.TH, g.RS, d.stride, &g.b_ways);
+    // (Winograd: lane l reads the 4x4 input patch of tile l, two floats to the right and two rows down per tile)
+    g.CS = t.wino ? pad_channel_stride(g.nrows * g.RS, 16, g.VW, 16 * t.wn, g.TWt, g.THt, g.RS, 2, &g.b_ways)
+                  : pad_channel_stride(g.nrows * g.RS, t.mf, g.VW, g.PT, g.TW, g.TH, g.RS, d.stride, &g.b_ways);
     // Copies are issued in whole blocks of 64 elements (1 KiB with 16-byte elements): both parts of
     // a stage are rounded up to that, the slack receiving zeros.
     g.in_stage_floats = round_up(t.cch * g.CS, 256);
-    g.wslab_floats = (t.wm * t.mb) * (t.cch / g.kc) * g.taps * 64;
+    g.wslab_floats = (t.wm * t.mb) * (t.cch / g.kc) * g.ktaps * 64;
     g.aff_floats = (d.KH == 1 && d.KW == 1 && d.pad == 0) ? round_up(2 * t.cch, 256) : 0;
     g.stage_floats = g.in_stage_floats + round_up(g.wslab_floats, 256) + g.aff_floats;
     g.nstage = g.cps > 1 ? 2 : 1;
     const long long stage_bytes = (long long)g.nstage * g.stage_floats * 4;
-    const long long red_bytes = t.wk > 1 ? (long long)t.wk * g.MT * g.PT * 4 : 0;
+    // (the Winograd path always parks its output tiles in LDS, also without a split over waves)
+    const long long red_bytes = (t.wk > 1 || t.wino) ? (long long)t.wk * g.MT * g.PT * 4 : 0;
     long long lds = std::max(stage_bytes, red_bytes);
     if (tail_N > 0) {
         // A fused 1x1 tail needs every output channel of the convolution in one workgroup; its tile is parked
@@ -222,6 +244,31 @@ void pack_weights(const tdc_conv_desc &d, const tdc_tile &t, const Geometry &g, 
     const int ncg = t.cch / g.kc;
     const int taps = g.taps;
     float *dst = packed;
+    if (g.wino) {
+        // Winograd F(2x2,3x3): U = G g G^T per (output channel, input channel), G = [1 0 0; .5 .5 .5; .5 -.5 .5; 0 0 1].
+        // Per (channel tile, pass, M block, channel group): [q = 0..3][64 lanes][e = 0..3] holding U[q][e] of
+        // (n = l % 16, c = l / 16), so that one 128-bit LDS read fetches the A operands of four of the 16 MFMAs.
+        static const double G[4][3] = {{1, 0, 0}, {0.5, 0.5, 0.5}, {0.5, -0.5, 0.5}, {0, 0, 1}};
+        for (int by = 0; by < g.grid_y; ++by)
+            for (int chunk = 0; chunk < g.nchunks; ++chunk)
+                for (int mbl = 0; mbl < mbw; ++mbl)
+                    for (int cg = 0; cg < ncg; ++cg)
+                        for (int q = 0; q < 4; ++q)
+                            for (int l = 0; l < 64; ++l) {
+                                const int n = by * g.MT + mbl * 16 + l % 16;
+                                const int c = chunk * t.cch + cg * 4 + l / 16;
+                                for (int e = 0; e < 4; ++e) {
+                                    double u = 0.0;
+                                    if (n < d.N && c < d.C) {
+                                        const float *gk = w + ((size_t)n * d.C + c) * 9;
+                                        for (int r = 0; r < 3; ++r)
+                                            for (int s = 0; s < 3; ++s) u += G[q][r] * (double)gk[r * 3 + s] * G[e][s];
+                                    }
+                                    *dst++ = (float)u;
+                                }
+                            }
+        return;
+    }
     for (int by = 0; by < g.grid_y; ++by)
         for (int chunk = 0; chunk < g.nchunks; ++chunk)
             for (int mbl = 0; mbl < mbw; ++mbl)
@@ -259,9 +306,10 @@ struct ModelConst {
     double ksplit_clk = 4604;         // split across workgroups: write-through, ticket round trip, read-back
     double copy_issue_clk = 118.2;      // a wave is held this long by every global->LDS copy instruction it issues
     double lds_read_clk = 2.88;        // LDS busy cycles per conflict-free operand read of one wave
+    double wino_kstep_clk = 12.0;      // Winograd: vector-ALU cycles of the input transform per MFMA (2 per MFMA, plus addressing)
 };
 ModelConst MC;
-constexpr int kNumModelConst = 14;
+constexpr int kNumModelConst = 15;
 
 double *mc_field(int i) {
     switch (i) {
@@ -279,6 +327,7 @@ double *mc_field(int i) {
         case 11: return &MC.ksplit_clk;
         case 12: return &MC.copy_issue_clk;
         case 13: return &MC.lds_read_clk;
+        case 14: return &MC.wino_kstep_clk;
         default: return nullptr;
     }
 }
@@ -288,6 +337,7 @@ int kernel_vgprs(const tdc_tile &t, int taps_mode) {
     const int nacc = (t.mf == 32) ? 16 : 4;
     int regs = nacc * t.mb * t.nb + 6 * (t.mb + t.nb) + 24;
     if (taps_mode == 9) regs += 6 * t.nb;
+    if (t.wino) regs = 136;   // 64 accumulators, two sets of 16 B and 16 A operands, the raw patch
     return round_up(regs, 8);
 }
 
@@ -336,10 +386,11 @@ bool model_evaluate(const tdc_conv_desc &d, const tdc_tile &t, tdc_tile_info &in
     // --- per-workgroup costs (clock cycles of one CU) ------------------------
     const long long n_wg = (long long)g.grid_x * g.grid_y * g.grid_z;
     const double mfma_clk = (t.mf == 32) ? 64.0 : 32.0;
-    const double ksteps_pass = (double)(g.cpw / g.kc) * g.taps;
+    const double ksteps_pass = (double)(g.cpw / g.kc) * g.ktaps;
     // One wave's matrix-core time per pass; the LDS reads of a K-step (one A and
     // one B word per lane per block row/column) must fit under it.
-    const double mfma_pass = ksteps_pass * t.mb * t.nb * mfma_clk;
+    // (Winograd: the register transform of the input patch shares the wave's issue slots with its MFMAs)
+    const double mfma_pass = ksteps_pass * t.mb * t.nb * (mfma_clk + (t.wino ? MC.wino_kstep_clk : 0.0));
     const double copy_bytes_pass = (double)g.stage_floats * 4.0;
     const double red_bytes = t.wk > 1 ? (double)t.wk * g.MT * g.PT * 4.0 * 2.0 : 0.0;
     const double out_bytes = (double)g.MT * g.PT * 4.0;
@@ -417,6 +468,50 @@ std::vector<tdc_tile> model_enumerate(const tdc_conv_desc &d, int tail_N) {
     static const int wks[] = {1, 2, 4, 8, 16};
     static const int wms[] = {1, 2, 4};
     static const int wns[] = {1, 2, 4};
+    // Winograd candidates for 3x3 / stride 1 convolutions with enough pixels to fill tile lanes
+    if (d.KH == 3 && d.KW == 3 && d.stride == 1 && d.dilation == 1 && tail_N == 0 && !std::getenv("TDC_EXPERIMENT_NO_WINOGRAD")) {
+        const int Wt = ceil_div(Wo, 2), Ht = ceil_div(Ho, 2);
+        for (int wm : wms)
+            for (int wn : wns)
+                for (int wk : wks) {
+                    if (wm * wn * wk > 8) continue;
+                    if (16 * wm > round_up(d.N, 16)) continue;
+                    const int lanes = 16 * wn;
+                    if (lanes > round_up(Wt * Ht, 16)) continue;
+                    std::vector<int> tws;
+                    for (int tw = 1; tw <= std::min(Wt, lanes); ++tw) {
+                        const bool pow2 = (tw & (tw - 1)) == 0;
+                        const bool widest = (tw == std::min(Wt, lanes));
+                        if (!(widest || (pow2 && tw >= 2) || (Wt % tw == 0 && tw >= 2))) continue;
+                        const int th = std::min(lanes / tw, Ht);
+                        const double util = (double)(Wt * Ht) / ((double)ceil_div(Wt, tw) * ceil_div(Ht, th) * lanes);
+                        if (util < 0.7 && !widest) continue;
+                        tws.push_back(tw);
+                    }
+                    const int granule = 4 * wk;
+                    std::vector<int> cchs;
+                    for (int div : {1, 2, 4, 8}) {
+                        const int cch = round_up(ceil_div(d.C, div), granule);
+                        if (std::find(cchs.begin(), cchs.end(), cch) == cchs.end()) cchs.push_back(cch);
+                    }
+                    for (int fixed : {16, 32})
+                        if (fixed % granule == 0 && fixed < round_up(d.C, granule) &&
+                            std::find(cchs.begin(), cchs.end(), fixed) == cchs.end())
+                            cchs.push_back(fixed);
+                    const long long max_wgs = 4LL * machine().cus;
+                    for (int tw : tws)
+                        for (int cch : cchs)
+                            for (int ks : {1, 2, 4})
+                                for (int wl : {0, 2, 4}) {
+                                    tdc_tile t{16, 1, 1, wm, wn, wk, cch, tw, ks, wl, 1};
+                                    Geometry g;
+                                    if (!make_geometry(d, t, g, nullptr, 0)) continue;
+                                    if (ks > 1 && (long long)g.grid_x * g.grid_y * g.grid_z > max_wgs) continue;
+                                    if (wl > 0 && g.cps < 2) continue;
+                                    out.push_back(t);
+                                }
+                }
+    }
     for (int mf : mfs) {
         const int kc = (mf == 32) ? 2 : 4;
         for (int mb = 1; mb <= 2; ++mb)
@@ -460,7 +555,7 @@ std::vector<tdc_tile> model_enumerate(const tdc_conv_desc &d, int tail_N) {
                                 for (int cch : cchs)
                                     for (int ks : {1, 2, 4, 8})
                                         for (int wl : {0, 1, 2, 4}) {
-                                            tdc_tile t{mf, mb, nb, wm, wn, wk, cch, tw, ks, wl};
+                                            tdc_tile t{mf, mb, nb, wm, wn, wk, cch, tw, ks, wl, 0};
                                             Geometry g;
                                             if (!make_geometry(d, t, g, nullptr, tail_N)) continue;
                                             if (ks > 1 && (long long)g.grid_x * g.grid_y * g.grid_z > max_wgs) continue;
@@ -499,7 +594,7 @@ bool model_select(const tdc_conv_desc &d, tdc_tile_info &best, std::string *why,
     }
     if (!have && why) {
         // say why the plainest tile cannot be launched: that is the limit the shape runs into
-        const tdc_tile plain{16, 1, 1, 1, 1, 1, 4, 1, 1, 0};
+        const tdc_tile plain{16, 1, 1, 1, 1, 1, 4, 1, 1, 0, 0};
         Geometry g;
         std::string reason;
         *why = make_geometry(d, plain, g, &reason, tail_N) ? "no launchable tile for this shape"

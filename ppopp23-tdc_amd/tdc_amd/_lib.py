@@ -44,16 +44,16 @@ class ConvDesc(Structure):
 
 
 class Tile(Structure):
-    _fields_ = [(n, c_int32) for n in ("mf", "mb", "nb", "wm", "wn", "wk", "cch", "tw", "ks", "wl")]
+    _fields_ = [(n, c_int32) for n in ("mf", "mb", "nb", "wm", "wn", "wk", "cch", "tw", "ks", "wl", "wino")]
 
-    def __init__(self, mf=0, mb=0, nb=0, wm=0, wn=0, wk=0, cch=0, tw=0, ks=1, wl=0):
-        super().__init__(mf, mb, nb, wm, wn, wk, cch, tw, ks, wl)
+    def __init__(self, mf=0, mb=0, nb=0, wm=0, wn=0, wk=0, cch=0, tw=0, ks=1, wl=0, wino=0):
+        super().__init__(mf, mb, nb, wm, wn, wk, cch, tw, ks, wl, wino)
 
     def astuple(self):
-        return (self.mf, self.mb, self.nb, self.wm, self.wn, self.wk, self.cch, self.tw, self.ks, self.wl)
+        return (self.mf, self.mb, self.nb, self.wm, self.wn, self.wk, self.cch, self.tw, self.ks, self.wl, self.wino)
 
     def __repr__(self):
-        return "Tile(mf=%d, mb=%d, nb=%d, wm=%d, wn=%d, wk=%d, cch=%d, tw=%d, ks=%d, wl=%d)" % self.astuple()
+        return "Tile(mf=%d, mb=%d, nb=%d, wm=%d, wn=%d, wk=%d, cch=%d, tw=%d, ks=%d, wl=%d, wino=%d)" % self.astuple()
 
 
 class TileInfo(Structure):
@@ -168,7 +168,7 @@ def model_evaluate(desc: ConvDesc, tile: Tile) -> TileInfo:
 
 MODEL_CONSTANT_NAMES = ("launch_us", "setup_clk", "copy_latency_clk", "copy_bytes_per_clk", "l2_bytes_per_clk",
                         "lds_bytes_per_clk", "sync_clk", "store_bytes_per_clk", "kstep_issue_clk", "pass_overhead_clk",
-                        "wave_setup_clk", "ksplit_clk", "copy_issue_clk", "lds_read_clk")
+                        "wave_setup_clk", "ksplit_clk", "copy_issue_clk", "lds_read_clk", "wino_kstep_clk")
 
 
 def model_select_with_tail(desc: ConvDesc, tail_N: int):

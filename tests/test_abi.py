@@ -36,11 +36,11 @@ def test_version_and_error_string():
 
 def test_struct_layouts_match_the_header():
     assert ctypes.sizeof(_lib.ConvDesc) == 12 * 4
-    assert ctypes.sizeof(_lib.Tile) == 10 * 4
+    assert ctypes.sizeof(_lib.Tile) == 11 * 4
     assert ctypes.sizeof(_lib.TKConvDesc) == 13 * 4
-    # tile (10 ints) + 10 ints + 5 doubles
-    assert ctypes.sizeof(_lib.TileInfo) == 10 * 4 + 10 * 4 + 5 * 8
-    assert _lib.TileInfo.flops.offset == 80
+    # tile (11 ints) + 10 ints + 4 bytes of padding + 5 doubles
+    assert ctypes.sizeof(_lib.TileInfo) == 11 * 4 + 10 * 4 + 4 + 5 * 8
+    assert _lib.TileInfo.flops.offset == 88
 
 
 def test_invalid_descriptors_are_rejected_with_a_reason():

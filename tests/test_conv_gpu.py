@@ -72,6 +72,46 @@ def test_every_tile_3x3(shape):
         assert_close(run_conv(x, w, pad=1, tile=t), want, f"{shape} {t}")
 
 
+@pytest.mark.parametrize("shape,pad", [((1, 8, 16, 8, 8), 1), ((2, 13, 20, 9, 11), 1), ((1, 7, 5, 5, 7), 0),
+                                       ((1, 16, 16, 12, 12), 2), ((1, 40, 24, 14, 14), 1), ((1, 3, 2, 2, 2), 1),
+                                       ((1, 4, 4, 1, 9), 1)])
+def test_every_winograd_tile(shape, pad):
+    """The Winograd F(2x2,3x3) path (tile.wino = 1) with every launchable tile: odd image sizes (the last tile row
+    and column are half outside), paddings 0..2, several passes, splits over waves and workgroups, loader waves."""
+    B, C, N, H, W = shape
+    x, w = case(1500 + C * N + H, B, C, N, H, W, 3)
+    want = ref.conv2d_c(x.numpy(), w.numpy(), pad=pad)
+    tiles = [t for t in tdc_amd.model_enumerate(tdc_amd.conv_desc(B, C, N, H, W, 3, 3, 1, pad)) if t.wino]
+    assert tiles
+    for t in tiles[::max(1, len(tiles) // 100)]:
+        announce("winograd", shape, pad, t)
+        assert_close(run_conv(x, w, pad=pad, tile=t), want, f"{shape} pad {pad} {t}")
+
+
+def test_winograd_epilogue_exactness_and_determinism():
+    """Winograd tiles on a benchmark layer: bias + residual + ReLU, the same bits on every launch, and the
+    reference's integer known-answer test stays exact (the transformed weights 1, 3/2, 1/2, 9/4, 3/4, 1/4 and all
+    partial sums are exactly representable)."""
+    tiles = [tdc_amd.Tile(16, 1, 1, 1, 2, 2, 32, 14, 1, 4, 1), tdc_amd.Tile(16, 1, 1, 2, 1, 4, 16, 7, 2, 0, 1)]
+    x, w = ref.make_core_case(56, 64, 64)
+    g = seeded(77)
+    bias = torch.randn(64, generator=g)
+    resid = torch.randn(1, 64, 56, 56, generator=g)
+    want = (ref.conv2d_torch(x, w, pad=1) + bias.view(1, -1, 1, 1) + resid).clamp_min(0).numpy()
+    rng = np.random.default_rng(8)
+    xi = torch.from_numpy(rng.integers(0, 10, size=(1, 64, 56, 56)).astype(np.float32))
+    s = np.pad(xi.numpy().sum(axis=1)[0].astype(np.float64), 1)
+    box = sum(s[r:r + 56, c:c + 56] for r in range(3) for c in range(3))
+    for t in tiles:
+        announce("winograd epilogue", t)
+        a = run_conv(x, w, bias, resid, pad=1, relu=True, tile=t)
+        b = run_conv(x, w, bias, resid, pad=1, relu=True, tile=t)
+        assert_close(a, want, f"winograd epilogue {t}")
+        assert np.array_equal(a, b)
+        got = run_conv(xi, torch.ones(64, 64, 3, 3), pad=1, tile=t)
+        assert np.abs(got - box[None, None]).sum() == 0.0
+
+
 @pytest.mark.parametrize("shape", [(1, 16, 8, 5, 5), (1, 7, 5, 9, 4), (2, 64, 48, 7, 7), (1, 100, 36, 14, 14)])
 def test_every_tile_1x1(shape):
     B, C, N, H, W = shape
@@ -315,7 +355,7 @@ def test_fused_1x1_tail(shape):
     desc = tdc_amd.conv_desc(B, C, N, H, W, K, K, stride, K // 2, 1, True, True)
     ok = []
     for t in tdc_amd.model_enumerate(desc):
-        if t.ks == 1 and t.mf * t.mb * t.wm >= N:
+        if t.ks == 1 and t.mf * t.mb * t.wm >= N and not t.wino:    # (the Winograd path carries no tail)
             ok.append(t)
     assert ok
     xd, rd = x.cuda(), resid.cuda()

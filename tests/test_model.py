@@ -22,14 +22,35 @@ def test_every_candidate_is_launchable_and_covers_the_output(hw, r1, r2):
     for t in tiles[:: max(1, len(tiles) // 60)]:
         i = tdc_amd.model_evaluate(d, t)
         lanes = t.mf * t.nb * t.wn
-        assert 1 <= i.th and i.th * t.tw <= lanes
-        ntx, nty = math.ceil(hw / t.tw), math.ceil(hw / i.th)
-        assert i.grid_x == ntx * nty and ntx * t.tw >= hw and nty * i.th >= hw      # tiles cover the image
+        # a Winograd lane stands for a 2x2-pixel tile and tw counts those
+        tw_px, lane_px = (2 * t.tw, 4) if t.wino else (t.tw, 1)
+        assert 1 <= i.th and i.th * tw_px <= lanes * lane_px
+        ntx, nty = math.ceil(hw / tw_px), math.ceil(hw / i.th)
+        assert i.grid_x == ntx * nty and ntx * tw_px >= hw and nty * i.th >= hw     # tiles cover the image
         assert i.grid_y * t.mf * t.mb * t.wm >= r2                                   # ... and all channels
         assert i.nchunks * t.cch >= r1 and t.cch % ((2 if t.mf == 32 else 4) * t.wk) == 0
         assert i.block_threads == 64 * (t.wm * t.wn * t.wk + t.wl) <= 1024      # computing waves + loader waves
         assert 0 < i.lds_bytes <= LDS_BYTES
         assert i.wg_per_cu >= 1 and i.pred_us > 0
+
+
+def test_winograd_tiles_only_where_the_algorithm_applies():
+    """tile.wino needs a 3x3 / stride 1 / dilation 1 convolution and one 16x16 block per wave; the model hands the
+    large 56x56 layers to it and keeps the small ones on the direct path."""
+    w = tdc_amd.Tile(16, 1, 1, 1, 2, 2, 32, 14, 1, 0, 1)
+    assert tdc_amd.model_evaluate(conv3(128, 128, 56), w).th == 4           # 2 tile rows of 14 tiles = 4 x 28 pixels
+    for d, t in [(conv3(64, 64, 56, stride=2), w),
+                 (tdc_amd.conv_desc(1, 64, 64, 56, 56, 1, 1, 1, 0), w),
+                 (tdc_amd.conv_desc(1, 64, 64, 56, 56, 3, 3, 1, 2, 2), w),      # dilation 2
+                 (conv3(128, 128, 56), tdc_amd.Tile(32, 1, 1, 1, 2, 2, 32, 14, 1, 0, 1)),
+                 (conv3(128, 128, 56), tdc_amd.Tile(16, 1, 2, 1, 2, 2, 32, 14, 1, 0, 1)),
+                 (conv3(128, 128, 56), tdc_amd.Tile(16, 1, 1, 1, 2, 2, 32, 29, 1, 0, 1)),   # wider than the image in tiles
+                 (conv3(128, 128, 56), tdc_amd.Tile(16, 1, 1, 2, 4, 2, 32, 14, 1, 0, 1))]:   # 16 waves: over the budget of 8
+        with pytest.raises(tdc_amd.TdcError):
+            tdc_amd.model_evaluate(d, t)
+    assert tdc_amd.model_select(conv3(128, 128, 56)).tile.wino == 1
+    assert tdc_amd.model_select(conv3(32, 32, 14)).tile.wino == 0
+    assert not any(t.wino for t in tdc_amd.model_enumerate(conv3(64, 64, 56, stride=2)))
 
 
 def test_algorithmic_work_and_roofline_of_config1():
