@@ -306,7 +306,7 @@ struct ModelConst {
     double ksplit_clk = 4604;         // split across workgroups: write-through, ticket round trip, read-back
     double copy_issue_clk = 118.2;      // a wave is held this long by every global->LDS copy instruction it issues
     double lds_read_clk = 2.88;        // LDS busy cycles per conflict-free operand read of one wave
-    double wino_kstep_clk = 12.0;      // Winograd: vector-ALU cycles of the input transform per MFMA (2 per MFMA, plus addressing)
+    double wino_kstep_clk = 14.4;      // Winograd: vector-ALU cycles of the input transform per MFMA (2 per MFMA, plus addressing)
 };
 ModelConst MC;
 constexpr int kNumModelConst = 15;

@@ -60,7 +60,7 @@ def sweep_shape(C, N, H, W, K=3, stride=1, pad=1, batch=1, iters=20, every=1, lo
             log.write(",".join(f"{v:.3f}" if isinstance(v, float) else str(v) for v in row) + "\n")
             log.flush()
     best = min(rows, key=lambda r: r[-1])
-    mine = next(r for r in rows if r[6:16] == pick.tile.astuple())
+    mine = next(r for r in rows if r[6:17] == pick.tile.astuple())
     return {"shape": (C, N, H, W, K, stride), "best": best, "model": mine, "loss": mine[-1] / best[-1] - 1,
             "roof_us": pick.roof_us, "n": len(rows)}
 
