@@ -842,6 +842,49 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
         return;
     }
     if (p.KS == 1) {
+        if constexpr (TAPS == TAPS_WINO) {
+            // The parked tile rows are runs of TW (even) consecutive pixels: where image width and the output
+            // address allow it, every thread finishes four (or two) consecutive pixels of one channel with one wide
+            // LDS read per slice and one wide store.
+            const unsigned long long addr_bits =
+                reinterpret_cast<unsigned long long>(p.out) | reinterpret_cast<unsigned long long>(p.resid);
+            const long long stride_bits = p.out_bstride | p.resid_bstride;
+            auto walk = [&](auto vec_tag) {
+                using vec_t = decltype(vec_tag);
+                constexpr int V = sizeof(vec_t) / sizeof(float);
+                const int total_v = (MT * PT) / V;
+                for (int q = tid; q < total_v; q += nthreads) {
+                    const int idx = q * V;
+                    const int ml = fdiv(idx, p.fd_pt);
+                    const int j = idx - ml * PT;
+                    const int jy = fdiv(j, p.fd_tw);
+                    const int jx = j - jy * p.TW;
+                    const int n = m0 + ml;
+                    const int oy = oy0 + jy, ox = ox0 + jx;
+                    if (n < p.N && jy < p.TH && oy < p.Ho && ox < p.Wo) {
+                        vec_t val = *reinterpret_cast<const vec_t *>(lds + idx);
+                        for (int k = 1; k < p.WK; ++k) val += *reinterpret_cast<const vec_t *>(lds + k * (MT * PT) + idx);
+                        const long long o = (long long)n * p.P + oy * p.Wo + ox;
+                        if (p.bias) val += p.bias[n];
+                        if (resid) val += *reinterpret_cast<const vec_t *>(resid + o);
+                        if (p.relu) {
+#pragma unroll
+                            for (int e = 0; e < V; ++e) val[e] = fmaxf(val[e], 0.0f);
+                        }
+                        *reinterpret_cast<vec_t *>(out + o) = val;
+                    }
+                }
+            };
+            typedef float f2_t __attribute__((ext_vector_type(2)));
+            if (((p.TW | p.Wo) & 3) == 0 && (stride_bits & 3) == 0 && (addr_bits & 15ull) == 0) {
+                walk(f4_t{});
+                return;
+            }
+            if ((p.Wo & 1) == 0 && (stride_bits & 1) == 0 && (addr_bits & 7ull) == 0) {
+                walk(f2_t{});
+                return;
+            }
+        }
         each_output(finish, true);
         return;
     }
