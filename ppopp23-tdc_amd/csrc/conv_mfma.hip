@@ -967,7 +967,7 @@ const void *conv_kernel_for(const tdc_tile &t, int KH, int KW, int dilation, boo
     kernel_fn fn = nullptr;
     if (t.wino) {
         if (extras || KH != 3 || KW != 3 || dilation != 1 || t.mf != 16 || t.mb != 1 || t.nb != 1) return nullptr;
-        return reinterpret_cast<const void *>(static_cast<kernel_fn>(tdc_conv_mfma_kernel<16, 1, 1, TAPS_WINO, 8, false>));
+        return reinterpret_cast<const void *>(static_cast<kernel_fn>(tdc_conv_mfma_kernel<16, 1, 1, TAPS_WINO, 12, false>));
     }
     switch (taps_mode(KH, KW, dilation)) {
         case TAPS_3x3: fn = extras ? pick_mf<TAPS_3x3, true>(t.mf, t.mb, t.nb) : pick_mf<TAPS_3x3, false>(t.mf, t.mb, t.nb); break;

@@ -114,7 +114,8 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
     if (t.mb < 1 || t.mb > 2 || t.nb < 1 || t.nb > 2) return fail("tile.mb / tile.nb must be 1 or 2");
     if (t.wm < 1 || t.wn < 1 || t.wk < 1) return fail("tile.wm / wn / wk must be >= 1");
     g = Geometry();
-    g.max_waves_kernel = ((t.mb == 2 && t.nb == 2) || t.wino == 1) ? 8 : 16;   // 256 registers per lane for those
+    // (256 registers per lane for the 2x2 block grid, 168 for the Winograd path)
+    g.max_waves_kernel = (t.mb == 2 && t.nb == 2) ? 8 : t.wino == 1 ? 12 : 16;
     if (t.wl < 0 || t.wl > 8) return fail("tile.wl must be in [0, 8]");
     if ((long long)t.wm * t.wn * t.wk + t.wl > g.max_waves_kernel) return fail("too many waves per workgroup for this tile");
     g.waves = t.wm * t.wn * t.wk + t.wl;
@@ -296,17 +297,17 @@ struct ModelConst {
     double setup_clk = 1208;          // kernel arguments and index arithmetic before the first copy is issued
     double copy_latency_clk = 920.5;   // first byte of a global->LDS copy (L2 / memory-side cache)
     double copy_bytes_per_clk = 34.32;   // sustained global->LDS rate of one CU
-    double l2_bytes_per_clk = 9627;   // whole-chip L2->CU rate when every CU copies at once
-    double lds_bytes_per_clk = 22.23;   // LDS traffic of the split-K reduction
-    double sync_clk = 229.3;            // one workgroup barrier
-    double store_bytes_per_clk = 2.772;  // per CU, short runs per channel
+    double l2_bytes_per_clk = 8183;   // whole-chip L2->CU rate when every CU copies at once
+    double lds_bytes_per_clk = 22.41;   // LDS traffic of the split-K reduction
+    double sync_clk = 275.2;            // one workgroup barrier
+    double store_bytes_per_clk = 3.326;  // per CU, short runs per channel
     double kstep_issue_clk = 2.798;      // vector-ALU / LDS-issue cycles per operand read, not hidden under MFMAs
     double pass_overhead_clk = 578.7;   // per wave and pass: copy issue, pointer set-up, pipeline fill
     double wave_setup_clk = 540.5;      // prologue cycles added per extra wave sharing a SIMD
     double ksplit_clk = 4604;         // split across workgroups: write-through, ticket round trip, read-back
     double copy_issue_clk = 118.2;      // a wave is held this long by every global->LDS copy instruction it issues
     double lds_read_clk = 2.88;        // LDS busy cycles per conflict-free operand read of one wave
-    double wino_kstep_clk = 14.4;      // Winograd: vector-ALU cycles of the input transform per MFMA (2 per MFMA, plus addressing)
+    double wino_kstep_clk = 2.142;      // Winograd: cycles per MFMA that the input transform adds on top of the operand reads
 };
 ModelConst MC;
 constexpr int kNumModelConst = 15;
