@@ -273,7 +273,8 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
 
     // The weight copies of the first pass need no per-lane arithmetic: start them before anything else.
     const int lane16 = lane * 16;
-    issue_weights<EXT>(p, w_rsrc, lds, lane16, (int)(w_byte_base + (unsigned)chunk0 * w_pass_bytes), wave, nwaves, chunk0);
+    if constexpr (TAPS != TAPS_WINO)   // (the Winograd path reads its weights from global memory into registers)
+        issue_weights<EXT>(p, w_rsrc, lds, lane16, (int)(w_byte_base + (unsigned)chunk0 * w_pass_bytes), wave, nwaves, chunk0);
 
     // Offsets of this lane's elements in its wave's first MAXPRE input blocks (pass 0), for the steady dealing
     // (positions past the stage decode to a channel >= CCH and so to the out-of-range offset).  With loader
@@ -315,7 +316,7 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
         // Copy issue competes for the SIMD with other waves' MFMA streams and loses by default (measured:
         // ~330 cycles per copy instruction instead of ~115); it is short, so let it go first.
         __builtin_amdgcn_s_setprio(3);
-        issue_weights<EXT>(p, w_rsrc, stage, lane16, w_byte0, dw, dn, chunk);
+        if constexpr (TAPS != TAPS_WINO) issue_weights<EXT>(p, w_rsrc, stage, lane16, w_byte0, dw, dn, chunk);
         issue_inputs(p, in_rsrc, stage, pre, true, chunk, iy0, ix0a, dw, dn, lane);
         __builtin_amdgcn_s_setprio(0);
     };
@@ -437,7 +438,9 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
             // MFMAs of group g.
             static_assert(TAPS != TAPS_WINO || (MF == 16 && MB == 1 && NB == 1), "Winograd path: one 16x16 block per wave");
             const float *praw = sin + wino_off;
-            const float *pw = stage + p.in_stage_floats + ((wm * ncg_pass + wk * ncgw) * 16) * 64 + lane * 4;
+            // A operands: straight from the packed weights in global memory (L2), 16 bytes per lane and quarter,
+            // one group ahead like the patch reads; the scalar operand carries everything but the lane.
+            const int w_soff = (int)(w_byte_base + (unsigned)chunk * w_pass_bytes) + ((wm * ncg_pass + wk * ncgw) * 16) * 256;
             const int RS = p.RS;
             const int gstep = KC * p.CS;
             float v0[16], v1[16];
@@ -450,7 +453,10 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
 #pragma unroll
                     for (int c = 0; c < 4; ++c) d[r][c] = b[r * RS + c];
 #pragma unroll
-                for (int q = 0; q < 4; ++q) u[q] = *reinterpret_cast<const f4_t *>(pw + (g * 16 + q * 4) * 64);
+                for (int q = 0; q < 4; ++q) {
+                    const auto raw = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, lane16, w_soff + (g * 16 + q * 4) * 256, 0);
+                    u[q] = __builtin_bit_cast(f4_t, raw);
+                }
                 float tr[4][4];   // B^T d: rows
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
@@ -474,7 +480,12 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
             };
             auto interleave = [&]() {
 #pragma unroll
-                for (int x = 0; x < 12; ++x) {
+                for (int x = 0; x < 4; ++x) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+                    __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // weight load
+                }
+#pragma unroll
+                for (int x = 0; x < 8; ++x) {
                     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
                     __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // LDS read
                 }

@@ -198,7 +198,8 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
     g.in_stage_floats = round_up(t.cch * g.CS, 256);
     g.wslab_floats = (t.wm * t.mb) * (t.cch / g.kc) * g.ktaps * 64;
     g.aff_floats = (d.KH == 1 && d.KW == 1 && d.pad == 0) ? round_up(2 * t.cch, 256) : 0;
-    g.stage_floats = g.in_stage_floats + round_up(g.wslab_floats, 256) + g.aff_floats;
+    // (the Winograd path reads its weights straight from global memory into registers: the LDS holds input only)
+    g.stage_floats = g.in_stage_floats + (t.wino ? 0 : round_up(g.wslab_floats, 256)) + g.aff_floats;
     g.nstage = g.cps > 1 ? 2 : 1;
     const long long stage_bytes = (long long)g.nstage * g.stage_floats * 4;
     // (the Winograd path always parks its output tiles in LDS, also without a split over waves)
@@ -399,7 +400,7 @@ bool model_evaluate(const tdc_conv_desc &d, const tdc_tile &t, tdc_tile_info &in
     // Copy instructions of one pass (64 elements each) and how long issuing them holds a wave: the first
     // pass is dealt to every wave; later ones to the loader waves if there are any, else to everybody.
     const int ncomp = t.wm * t.wn * t.wk;
-    const double n_instr = (double)g.in_stage_floats / (64.0 * g.VW) + std::ceil(g.wslab_floats / 256.0);
+    const double n_instr = (double)g.in_stage_floats / (64.0 * g.VW) + (t.wino ? 0.0 : std::ceil(g.wslab_floats / 256.0));
     const double issue_first = std::ceil(n_instr / g.waves) * MC.copy_issue_clk;
     const double issue_steady = std::ceil(n_instr / (t.wl ? t.wl : g.waves)) * MC.copy_issue_clk;
     const int comp_waves_per_simd = ceil_div(ncomp, m.simds_per_cu);
