@@ -395,7 +395,10 @@ bool model_evaluate(const tdc_conv_desc &d, const tdc_tile &t, tdc_tile_info &in
     const double mfma_pass = ksteps_pass * t.mb * t.nb * (mfma_clk + (t.wino ? MC.wino_kstep_clk : 0.0));
     const double copy_bytes_pass = (double)g.stage_floats * 4.0;
     const double red_bytes = t.wk > 1 ? (double)t.wk * g.MT * g.PT * 4.0 * 2.0 : 0.0;
-    const double out_bytes = (double)g.MT * g.PT * 4.0;
+    // (the Winograd epilogue stores four pixels per instruction where tile and image width are multiples of four,
+    //  two where the image width is even: cheaper per byte than single-pixel stores)
+    const double store_width = !t.wino ? 1.0 : ((g.TW | g.Wo) % 4 == 0) ? 0.6 : (g.Wo % 2 == 0) ? 0.85 : 1.0;
+    const double out_bytes = (double)g.MT * g.PT * 4.0 * store_width;
 
     // Copy instructions of one pass (64 elements each) and how long issuing them holds a wave: the first
     // pass is dealt to every wave; later ones to the loader waves if there are any, else to everybody.
