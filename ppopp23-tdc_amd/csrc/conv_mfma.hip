@@ -364,6 +364,19 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
     const int ncg_pass = p.CCH / KC;  // channel groups per pass
     const int ncgw = p.CPW / KC;      // ... of which this wave takes [wk*ncgw, (wk+1)*ncgw)
 
+    // Winograd: the A operands come from global memory and do not depend on the staged input, so the first group
+    // of every pass is requested before the wait and the barrier of that pass and is in registers when they end.
+    f4_t wu0[TAPS == TAPS_WINO ? 4 : 1];
+    auto wino_load_a = [&](int chunk, int g, f4_t(&u)[4]) {
+        const int soff = (int)(w_byte_base + (unsigned)chunk * w_pass_bytes) + ((wm * ncg_pass + wk * ncgw + g) * 16) * 256;
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+            u[q] = __builtin_bit_cast(f4_t, __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, lane16, soff + q * 1024, 0));
+    };
+    if constexpr (TAPS == TAPS_WINO) {
+        if (!loader) wino_load_a(chunk0, 0, wu0);
+    }
+
     for (int chunk = chunk0; chunk < chunk1; ++chunk) {
         // My copies of this pass have landed; after the barrier everybody's have, and
         // everybody is done reading the stage the next pass is about to overwrite.
@@ -440,23 +453,17 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
             const float *praw = sin + wino_off;
             // A operands: straight from the packed weights in global memory (L2), 16 bytes per lane and quarter,
             // one group ahead like the patch reads; the scalar operand carries everything but the lane.
-            const int w_soff = (int)(w_byte_base + (unsigned)chunk * w_pass_bytes) + ((wm * ncg_pass + wk * ncgw) * 16) * 256;
             const int RS = p.RS;
             const int gstep = KC * p.CS;
             float v0[16], v1[16];
-            f4_t u0[4], u1[4];
-            auto load_group = [&](int g, float(&v)[16], f4_t(&u)[4]) {
+            f4_t u1[4];
+            auto load_patch = [&](int g, float(&v)[16]) {
                 const float *b = praw + g * gstep;
                 float d[4][4];
 #pragma unroll
                 for (int r = 0; r < 4; ++r)
 #pragma unroll
                     for (int c = 0; c < 4; ++c) d[r][c] = b[r * RS + c];
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const auto raw = __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, lane16, w_soff + (g * 16 + q * 4) * 256, 0);
-                    u[q] = __builtin_bit_cast(f4_t, raw);
-                }
                 float tr[4][4];   // B^T d: rows
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
@@ -495,19 +502,22 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
                     __builtin_amdgcn_sched_group_barrier(0x002, 8, 0);  // the transform's vector ALU work
                 }
             };
-            load_group(0, v0, u0);
+            load_patch(0, v0);   // (its A operands are already on their way, or here)
             for (int g = 0; g + 1 < ncgw; g += 2) {
                 __builtin_amdgcn_sched_barrier(0);
-                load_group(g + 1, v1, u1);
-                mfma_group(v0, u0);
+                wino_load_a(chunk, g + 1, u1);
+                load_patch(g + 1, v1);
+                mfma_group(v0, wu0);
                 interleave();
                 __builtin_amdgcn_sched_barrier(0);
-                load_group(min(g + 2, ncgw - 1), v0, u0);
+                wino_load_a(chunk, min(g + 2, ncgw - 1), wu0);
+                load_patch(min(g + 2, ncgw - 1), v0);
                 mfma_group(v1, u1);
                 interleave();
                 __builtin_amdgcn_sched_barrier(0);
             }
-            if (ncgw & 1) mfma_group(v0, u0);
+            if (ncgw & 1) mfma_group(v0, wu0);
+            if (chunk + 1 < chunk1) wino_load_a(chunk + 1, 0, wu0);
         } else if constexpr (TAPS == TAPS_3x3) {
             // dilation 1: the column tap is an immediate offset of the LDS read, the row tap one of
             // three per-lane row addresses.  Two register sets ping-pong: the operands of channel
