@@ -56,7 +56,7 @@ def main():
                     help="profiling aid: run only the end-to-end Tucker ResNet-18 forward, `steps` times, and exit")
     ap.add_argument("--e2e-net", choices=["resnet18", "densenet121"], default="resnet18",
                     help="which Tucker network --only-e2e runs (batch 1)")
-    ap.add_argument("--tile", default=None, metavar="mf,mb,nb,wm,wn,wk,cch,tw,ks,wl,wino",
+    ap.add_argument("--tile", default=None, metavar="mf,mb,nb,wm,wn,wk,cch,tw,ks,wl,alg",
                     help="with --only-dominant: force this tile instead of selecting one")
     ap.add_argument("--tune", type=int, default=16, metavar="CLASSES",
                     help="measured tile selection at plan creation: time the model's favourite tile of this many tile "
@@ -103,7 +103,7 @@ def main():
         forced = None
         if a.tile:
             v = [int(t) for t in a.tile.split(",")]
-            forced = tdc_amd.Tile(*v[:8], ks=v[8], wl=v[9], wino=v[10] if len(v) > 10 else 0)
+            forced = tdc_amd.Tile(*v[:8], ks=v[8], wl=v[9], alg=v[10] if len(v) > 10 else 0)
         plan = Conv2dPlan(1, 128, 128, 56, 56, 3, 3, 1, 1, tile=forced).set_weights(w)
         xd, out = x.cuda(), torch.empty(1, 128, 56, 56, device="cuda")
         # the same back-to-back launches as the timed region of the full run (one graph of `steps` launches)

@@ -80,9 +80,13 @@ typedef struct tdc_tile {
                      added in index order by the last workgroup to arrive             */
     int32_t wl;   /* extra wavefronts that only issue the global->LDS copies of the
                      next pass while the wm*wn*wk others compute (0 = every wave does both) */
-    int32_t wino; /* 1 = Winograd F(2x2,3x3) for 3x3 / stride 1 / dilation 1 convolutions: the pixel
-                     lanes hold 2x2-pixel output tiles (tw counts those tiles), 16 MFMAs per four input
-                     channels and 16 tiles instead of 36; mf = 16, mb = nb = 1.  0 = direct convolution */
+    int32_t alg;  /* 0 = direct convolution, weights staged in LDS next to the input.
+                     1 = Winograd F(2x2,3x3) for 3x3 / stride 1 / dilation 1 convolutions: the pixel lanes hold
+                         2x2-pixel output tiles (tw counts those tiles), 16 MFMAs per four input channels and 16
+                         tiles instead of 36; weights read from global memory into registers; mf = 16, mb = nb = 1.
+                     2 = direct 3x3 / dilation 1 convolution with the weights read from global memory straight
+                         into registers (the LDS holds input only, so a pass can take more input channels);
+                         mb = nb = 1, an even number of channel groups per wave and pass */
 } tdc_tile;
 
 typedef struct tdc_tile_info {

@@ -93,7 +93,9 @@ struct Mfma<16> {
 // transformed domain, against weights U = G g G^T prepared on the host — where the direct path needs 36 for
 // the same four pixels.  The 16 accumulators of a lane are combined at the end (Y = A^T M A, in registers:
 // every lane holds all 16 positions of its tile) into the 2x2 outputs.
-enum : int { TAPS_GENERIC = 0, TAPS_1x1 = 1, TAPS_3x3 = 9, TAPS_WINO = 16 };
+// TAPS_3x3G: the direct 3x3 loop with its weights read from global memory straight into registers (like the
+// Winograd path) instead of being staged in LDS: the LDS then holds input only and a pass can take all input channels.
+enum : int { TAPS_GENERIC = 0, TAPS_1x1 = 1, TAPS_3x3 = 9, TAPS_3x3G = 10, TAPS_WINO = 16 };
 
 constexpr int OOB_OFFSET = 0x7ffffff0;  // beyond any buffer: the load returns zero
 
@@ -273,7 +275,7 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
 
     // The weight copies of the first pass need no per-lane arithmetic: start them before anything else.
     const int lane16 = lane * 16;
-    if constexpr (TAPS != TAPS_WINO)   // (the Winograd path reads its weights from global memory into registers)
+    if constexpr (TAPS != TAPS_WINO && TAPS != TAPS_3x3G)   // (those paths read their weights from global memory into registers)
         issue_weights<EXT>(p, w_rsrc, lds, lane16, (int)(w_byte_base + (unsigned)chunk0 * w_pass_bytes), wave, nwaves, chunk0);
 
     // Offsets of this lane's elements in its wave's first MAXPRE input blocks (pass 0), for the steady dealing
@@ -316,7 +318,7 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
         // Copy issue competes for the SIMD with other waves' MFMA streams and loses by default (measured:
         // ~330 cycles per copy instruction instead of ~115); it is short, so let it go first.
         __builtin_amdgcn_s_setprio(3);
-        if constexpr (TAPS != TAPS_WINO) issue_weights<EXT>(p, w_rsrc, stage, lane16, w_byte0, dw, dn, chunk);
+        if constexpr (TAPS != TAPS_WINO && TAPS != TAPS_3x3G) issue_weights<EXT>(p, w_rsrc, stage, lane16, w_byte0, dw, dn, chunk);
         issue_inputs(p, in_rsrc, stage, pre, true, chunk, iy0, ix0a, dw, dn, lane);
         __builtin_amdgcn_s_setprio(0);
     };
@@ -360,7 +362,7 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
 #pragma unroll
             for (int v = 0; v < NACC; ++v) acc[mb][nb][v] = 0.0f;
 
-    const int taps = (TAPS == TAPS_GENERIC) ? p.KH * p.KW : TAPS;
+    const int taps = (TAPS == TAPS_GENERIC) ? p.KH * p.KW : (TAPS == TAPS_3x3G) ? 9 : TAPS;
     const int ncg_pass = p.CCH / KC;  // channel groups per pass
     const int ncgw = p.CPW / KC;      // ... of which this wave takes [wk*ncgw, (wk+1)*ncgw)
 
@@ -375,6 +377,31 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
     };
     if constexpr (TAPS == TAPS_WINO) {
         if (!loader) wino_load_a(chunk0, 0, wu0);
+    }
+    // Direct 3x3 with weights from global memory: a group is a PAIR of channel groups (18 K-steps per block, long
+    // enough to cover the L2 latency one group ahead); per channel group and 16/32-row block the packed weights hold
+    // [taps 0-3][lane][4] [taps 4-7][lane][4] [tap 8][lane]: two 128-bit loads and one 32-bit load per lane.
+    float ga0[TAPS == TAPS_3x3G ? 18 : 1][MB];
+    auto g3_load_a = [&](int chunk, int pair, float(&a)[18][MB]) {
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int soff = (int)(w_byte_base + (unsigned)chunk * w_pass_bytes) +
+                                 (((wm * MB + mb) * ncg_pass + wk * ncgw + pair * 2 + h) * 9) * 256;
+                const f4_t q0 = __builtin_bit_cast(f4_t, __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, lane16, soff, 0));
+                const f4_t q1 = __builtin_bit_cast(f4_t, __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, lane16, soff + 1024, 0));
+                const float t8 = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(w_rsrc, lane * 4, soff + 2048, 0));
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    a[h * 9 + t][mb] = q0[t];
+                    a[h * 9 + 4 + t][mb] = q1[t];
+                }
+                a[h * 9 + 8][mb] = t8;
+            }
+    };
+    if constexpr (TAPS == TAPS_3x3G) {
+        if (!loader) g3_load_a(chunk0, 0, ga0);
     }
 
     for (int chunk = chunk0; chunk < chunk1; ++chunk) {
@@ -518,6 +545,60 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
             }
             if (ncgw & 1) mfma_group(v0, wu0);
             if (chunk + 1 < chunk1) wino_load_a(chunk + 1, 0, wu0);
+        } else if constexpr (TAPS == TAPS_3x3G) {
+            const int npairs = ncgw >> 1;   // (the host only offers this path for an even number of channel groups)
+            float a1[18][MB], b0[18][NB], b1[18][NB];
+            auto load_b = [&](int pair, float(&b)[18][NB]) {
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const float *lgrp = sin + (pair * 2 + h) * KC * p.CS;
+#pragma unroll
+                    for (int r = 0; r < 3; ++r)
+#pragma unroll
+                        for (int nb = 0; nb < NB; ++nb) {
+                            const float *lrow = lgrp + boff[nb] + r * p.RS;
+#pragma unroll
+                            for (int c = 0; c < 3; ++c) b[h * 9 + r * 3 + c][nb] = lrow[c];
+                        }
+                }
+            };
+            auto mfma_pair = [&](const float(&a)[18][MB], const float(&b)[18][NB]) {
+#pragma unroll
+                for (int t = 0; t < 18; ++t)
+#pragma unroll
+                    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                        for (int nb = 0; nb < NB; ++nb) acc[mb][nb] = M::run(a[t][mb], b[t][nb], acc[mb][nb]);
+            };
+            auto interleave = [&]() {
+#pragma unroll
+                for (int t = 0; t < 6; ++t) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, MB * NB, 0);  // MFMA
+                    __builtin_amdgcn_sched_group_barrier(0x020, MB, 0);       // weight loads
+                    __builtin_amdgcn_sched_group_barrier(0x100, NB, 0);       // LDS reads
+                }
+#pragma unroll
+                for (int t = 6; t < 18; ++t) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, MB * NB, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x100, NB, 0);
+                }
+            };
+            load_b(0, b0);   // (the weights of the first pair are already on their way, or here)
+            for (int pp = 0; pp + 1 < npairs; pp += 2) {
+                __builtin_amdgcn_sched_barrier(0);
+                g3_load_a(chunk, pp + 1, a1);
+                load_b(pp + 1, b1);
+                mfma_pair(ga0, b0);
+                interleave();
+                __builtin_amdgcn_sched_barrier(0);
+                g3_load_a(chunk, min(pp + 2, npairs - 1), ga0);
+                load_b(min(pp + 2, npairs - 1), b0);
+                mfma_pair(a1, b1);
+                interleave();
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (npairs & 1) mfma_pair(ga0, b0);
+            if (chunk + 1 < chunk1) g3_load_a(chunk + 1, 0, ga0);
         } else if constexpr (TAPS == TAPS_3x3) {
             // dilation 1: the column tap is an immediate offset of the LDS read, the row tap one of
             // three per-lane row addresses.  Two register sets ping-pong: the operands of channel
@@ -986,9 +1067,15 @@ static int taps_mode(int KH, int KW, int dil) {
 
 const void *conv_kernel_for(const tdc_tile &t, int KH, int KW, int dilation, bool extras) {
     kernel_fn fn = nullptr;
-    if (t.wino) {
+    if (t.alg == 1) {
         if (extras || KH != 3 || KW != 3 || dilation != 1 || t.mf != 16 || t.mb != 1 || t.nb != 1) return nullptr;
         return reinterpret_cast<const void *>(static_cast<kernel_fn>(tdc_conv_mfma_kernel<16, 1, 1, TAPS_WINO, 12, false>));
+    }
+    if (t.alg == 2) {
+        if (extras || KH != 3 || KW != 3 || dilation != 1 || t.mb != 1 || t.nb != 1) return nullptr;
+        if (t.mf == 16) return reinterpret_cast<const void *>(static_cast<kernel_fn>(tdc_conv_mfma_kernel<16, 1, 1, TAPS_3x3G, 16, false>));
+        if (t.mf == 32) return reinterpret_cast<const void *>(static_cast<kernel_fn>(tdc_conv_mfma_kernel<32, 1, 1, TAPS_3x3G, 16, false>));
+        return nullptr;
     }
     switch (taps_mode(KH, KW, dilation)) {
         case TAPS_3x3: fn = extras ? pick_mf<TAPS_3x3, true>(t.mf, t.mb, t.nb) : pick_mf<TAPS_3x3, false>(t.mf, t.mb, t.nb); break;

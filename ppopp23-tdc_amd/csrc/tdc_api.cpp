@@ -220,7 +220,7 @@ static int tune_tile(const tdc_conv_desc &d, int tail_N, int tail_has_bias, int 
     for (const tdc_tile &t : model_enumerate(d, tail_N)) {
         tdc_tile_info info;
         if (!model_evaluate(d, t, info, nullptr, tail_N)) continue;
-        const std::array<int, 8> cls{t.mf, t.mb, t.nb, t.wm, t.wn, t.wk, t.tw, t.wino};
+        const std::array<int, 8> cls{t.mf, t.mb, t.nb, t.wm, t.wn, t.wk, t.tw, t.alg};
         auto it = per_class.find(cls);
         if (it == per_class.end() || info.pred_us < it->second.pred_us) per_class[cls] = info;
     }

@@ -115,7 +115,7 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
     if (t.wm < 1 || t.wn < 1 || t.wk < 1) return fail("tile.wm / wn / wk must be >= 1");
     g = Geometry();
     // (256 registers per lane for the 2x2 block grid, 168 for the Winograd path)
-    g.max_waves_kernel = (t.mb == 2 && t.nb == 2) ? 8 : t.wino == 1 ? 12 : 16;
+    g.max_waves_kernel = (t.mb == 2 && t.nb == 2) ? 8 : t.alg == 1 ? 12 : 16;
     if (t.wl < 0 || t.wl > 8) return fail("tile.wl must be in [0, 8]");
     if ((long long)t.wm * t.wn * t.wk + t.wl > g.max_waves_kernel) return fail("too many waves per workgroup for this tile");
     g.waves = t.wm * t.wn * t.wk + t.wl;
@@ -132,13 +132,20 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
     g.taps = d.KH * d.KW;
     g.ktaps = g.taps;
     g.MT = t.mf * t.mb * t.wm;
-    if (t.wino != 0 && t.wino != 1) return fail("tile.wino must be 0 or 1");
-    g.wino = t.wino;
-    if (t.wino) {
+    if (t.alg < 0 || t.alg > 2) return fail("tile.alg must be 0, 1 or 2");
+    g.wino = t.alg == 1;
+    if (t.alg == 2) {
+        // direct 3x3 convolution with the weights read from global memory into registers, a pair of channel groups at a time
+        if (d.KH != 3 || d.KW != 3 || d.dilation != 1) return fail("tile.alg = 2 needs a 3x3 / dilation 1 convolution");
+        if (t.mb != 1 || t.nb != 1) return fail("tile.alg = 2 needs mb = nb = 1");
+        if (tail_N > 0) return fail("tile.alg = 2 cannot carry a fused tail");
+        if (t.cch % (2 * g.kc * t.wk) != 0) return fail("tile.alg = 2 needs an even number of channel groups per wave and pass");
+    }
+    if (t.alg == 1) {
         // Winograd F(2x2,3x3): a pixel lane holds one 2x2 output tile; the workgroup tile is THt x TWt such tiles.
-        if (d.KH != 3 || d.KW != 3 || d.stride != 1 || d.dilation != 1) return fail("tile.wino needs a 3x3 / stride 1 / dilation 1 convolution");
-        if (t.mf != 16 || t.mb != 1 || t.nb != 1) return fail("tile.wino needs mf = 16, mb = nb = 1");
-        if (tail_N > 0) return fail("tile.wino cannot carry a fused tail");
+        if (d.KH != 3 || d.KW != 3 || d.stride != 1 || d.dilation != 1) return fail("tile.alg needs a 3x3 / stride 1 / dilation 1 convolution");
+        if (t.mf != 16 || t.mb != 1 || t.nb != 1) return fail("tile.alg needs mf = 16, mb = nb = 1");
+        if (tail_N > 0) return fail("tile.alg cannot carry a fused tail");
         const int lanes = 16 * t.wn;
         const int Wt = ceil_div(g.Wo, 2), Ht = ceil_div(g.Ho, 2);
         if (t.tw < 1 || t.tw > lanes || t.tw > Wt) return fail("tile.tw must be in [1, min(ceil(Wo/2), tile lanes)]");
@@ -191,7 +198,7 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
         g.RS = g.ncols;
     }
     // (Winograd: lane l reads the 4x4 input patch of tile l, two floats to the right and two rows down per tile)
-    g.CS = t.wino ? pad_channel_stride(g.nrows * g.RS, 16, g.VW, 16 * t.wn, g.TWt, g.THt, g.RS, 2, &g.b_ways)
+    g.CS = t.alg == 1 ? pad_channel_stride(g.nrows * g.RS, 16, g.VW, 16 * t.wn, g.TWt, g.THt, g.RS, 2, &g.b_ways)
                   : pad_channel_stride(g.nrows * g.RS, t.mf, g.VW, g.PT, g.TW, g.TH, g.RS, d.stride, &g.b_ways);
     // Copies are issued in whole blocks of 64 elements (1 KiB with 16-byte elements): both parts of
     // a stage are rounded up to that, the slack receiving zeros.
@@ -199,11 +206,11 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
     g.wslab_floats = (t.wm * t.mb) * (t.cch / g.kc) * g.ktaps * 64;
     g.aff_floats = (d.KH == 1 && d.KW == 1 && d.pad == 0) ? round_up(2 * t.cch, 256) : 0;
     // (the Winograd path reads its weights straight from global memory into registers: the LDS holds input only)
-    g.stage_floats = g.in_stage_floats + (t.wino ? 0 : round_up(g.wslab_floats, 256)) + g.aff_floats;
+    g.stage_floats = g.in_stage_floats + (t.alg ? 0 : round_up(g.wslab_floats, 256)) + g.aff_floats;   // (wino = 2 likewise)
     g.nstage = g.cps > 1 ? 2 : 1;
     const long long stage_bytes = (long long)g.nstage * g.stage_floats * 4;
     // (the Winograd path always parks its output tiles in LDS, also without a split over waves)
-    const long long red_bytes = (t.wk > 1 || t.wino) ? (long long)t.wk * g.MT * g.PT * 4 : 0;
+    const long long red_bytes = (t.wk > 1 || t.alg == 1) ? (long long)t.wk * g.MT * g.PT * 4 : 0;
     long long lds = std::max(stage_bytes, red_bytes);
     if (tail_N > 0) {
         // A fused 1x1 tail needs every output channel of the convolution in one workgroup; its tile is parked
@@ -246,6 +253,21 @@ void pack_weights(const tdc_conv_desc &d, const tdc_tile &t, const Geometry &g, 
     const int ncg = t.cch / g.kc;
     const int taps = g.taps;
     float *dst = packed;
+    if (t.alg == 2) {
+        // per (channel tile, pass, M block, channel group): [taps 0-3][lane][4] [taps 4-7][lane][4] [tap 8][lane]
+        for (int by = 0; by < g.grid_y; ++by)
+            for (int chunk = 0; chunk < g.nchunks; ++chunk)
+                for (int mbl = 0; mbl < mbw; ++mbl)
+                    for (int cg = 0; cg < ncg; ++cg, dst += 9 * 64)
+                        for (int tap = 0; tap < 9; ++tap)
+                            for (int l = 0; l < 64; ++l) {
+                                const int n = by * g.MT + mbl * t.mf + l % t.mf;
+                                const int c = chunk * t.cch + cg * g.kc + l / t.mf;
+                                const float v = (n < d.N && c < d.C) ? w[((size_t)n * d.C + c) * 9 + tap] : 0.0f;
+                                dst[tap < 8 ? (tap / 4) * 256 + l * 4 + tap % 4 : 512 + l] = v;
+                            }
+        return;
+    }
     if (g.wino) {
         // Winograd F(2x2,3x3): U = G g G^T per (output channel, input channel), G = [1 0 0; .5 .5 .5; .5 -.5 .5; 0 0 1].
         // Per (channel tile, pass, M block, channel group): [q = 0..3][64 lanes][e = 0..3] holding U[q][e] of
@@ -339,7 +361,8 @@ int kernel_vgprs(const tdc_tile &t, int taps_mode) {
     const int nacc = (t.mf == 32) ? 16 : 4;
     int regs = nacc * t.mb * t.nb + 6 * (t.mb + t.nb) + 24;
     if (taps_mode == 9) regs += 6 * t.nb;
-    if (t.wino) regs = 136;   // 64 accumulators, two sets of 16 B and 16 A operands, the raw patch
+    if (t.alg == 1) regs = 136;   // 64 accumulators, two sets of 16 B and 16 A operands, the raw patch
+    if (t.alg == 2) regs = 104;   // two sets of 18 A and 18 B operands
     return round_up(regs, 8);
 }
 
@@ -392,18 +415,18 @@ bool model_evaluate(const tdc_conv_desc &d, const tdc_tile &t, tdc_tile_info &in
     // One wave's matrix-core time per pass; the LDS reads of a K-step (one A and
     // one B word per lane per block row/column) must fit under it.
     // (Winograd: the register transform of the input patch shares the wave's issue slots with its MFMAs)
-    const double mfma_pass = ksteps_pass * t.mb * t.nb * (mfma_clk + (t.wino ? MC.wino_kstep_clk : 0.0));
+    const double mfma_pass = ksteps_pass * t.mb * t.nb * (mfma_clk + (t.alg == 1 ? MC.wino_kstep_clk : 0.0));
     const double copy_bytes_pass = (double)g.stage_floats * 4.0;
     const double red_bytes = t.wk > 1 ? (double)t.wk * g.MT * g.PT * 4.0 * 2.0 : 0.0;
     // (the Winograd epilogue stores four pixels per instruction where tile and image width are multiples of four,
     //  two where the image width is even: cheaper per byte than single-pixel stores)
-    const double store_width = !t.wino ? 1.0 : ((g.TW | g.Wo) % 4 == 0) ? 0.6 : (g.Wo % 2 == 0) ? 0.85 : 1.0;
+    const double store_width = t.alg != 1 ? 1.0 : ((g.TW | g.Wo) % 4 == 0) ? 0.6 : (g.Wo % 2 == 0) ? 0.85 : 1.0;
     const double out_bytes = (double)g.MT * g.PT * 4.0 * store_width;
 
     // Copy instructions of one pass (64 elements each) and how long issuing them holds a wave: the first
     // pass is dealt to every wave; later ones to the loader waves if there are any, else to everybody.
     const int ncomp = t.wm * t.wn * t.wk;
-    const double n_instr = (double)g.in_stage_floats / (64.0 * g.VW) + (t.wino ? 0.0 : std::ceil(g.wslab_floats / 256.0));
+    const double n_instr = (double)g.in_stage_floats / (64.0 * g.VW) + (t.alg ? 0.0 : std::ceil(g.wslab_floats / 256.0));
     const double issue_first = std::ceil(n_instr / g.waves) * MC.copy_issue_clk;
     const double issue_steady = std::ceil(n_instr / (t.wl ? t.wl : g.waves)) * MC.copy_issue_clk;
     const int comp_waves_per_simd = ceil_div(ncomp, m.simds_per_cu);
@@ -414,10 +437,12 @@ bool model_evaluate(const tdc_conv_desc &d, const tdc_tile &t, tdc_tile_info &in
         const double waves_simd = (double)comp_waves_per_simd * r;
         // A wave alone on its SIMD stalls on every operand read and while it issues copies; with several
         // waves per SIMD those gaps are filled by the others until the matrix pipe itself is the limit.
-        const double stall = ksteps_pass * (t.mb + t.nb * g.b_ways) * MC.kstep_issue_clk + MC.pass_overhead_clk;
+        // (wino = 2: the A operands do not come from the LDS)
+        const double a_reads = t.alg == 2 ? 0.25 * t.mb : (double)t.mb;
+        const double stall = ksteps_pass * (a_reads + t.nb * g.b_ways) * MC.kstep_issue_clk + MC.pass_overhead_clk;
         const double alone = mfma_pass + stall;
         // ... or the LDS: every operand read keeps it busy for lds_read_clk cycles, a conflicting one longer.
-        const double lds_busy = ksteps_pass * (t.mb + t.nb * g.b_ways) * MC.lds_read_clk * ncomp * r;
+        const double lds_busy = ksteps_pass * ((t.alg == 2 ? 0.0 : (double)t.mb) + t.nb * g.b_ways) * MC.lds_read_clk * ncomp * r;
         const double pipe = std::max(mfma_pass * waves_simd, lds_busy) + MC.pass_overhead_clk;
         const double compute = std::max(alone, pipe) + MC.sync_clk;
         const double compute_issuing = std::max(alone + issue_steady, pipe) + MC.sync_clk;
@@ -517,6 +542,8 @@ std::vector<tdc_tile> model_enumerate(const tdc_conv_desc &d, int tail_N) {
                                 }
                 }
     }
+    const bool global_weights = d.KH == 3 && d.KW == 3 && d.dilation == 1 && tail_N == 0 &&
+                                !std::getenv("TDC_EXPERIMENT_NO_GLOBAL_WEIGHTS");
     for (int mf : mfs) {
         const int kc = (mf == 32) ? 2 : 4;
         for (int mb = 1; mb <= 2; ++mb)
@@ -566,6 +593,11 @@ std::vector<tdc_tile> model_enumerate(const tdc_conv_desc &d, int tail_N) {
                                             if (ks > 1 && (long long)g.grid_x * g.grid_y * g.grid_z > max_wgs) continue;
                                             if (wl > 0 && g.cps < 2) continue;  // loaders only work from the second pass on
                                             out.push_back(t);
+                                            // the same tile with its weights read from global memory
+                                            if (global_weights && mb == 1 && nb == 1) {
+                                                t.alg = 2;
+                                                if (make_geometry(d, t, g, nullptr, 0)) out.push_back(t);
+                                            }
                                         }
                         }
     }

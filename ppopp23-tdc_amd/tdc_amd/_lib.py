@@ -44,16 +44,16 @@ class ConvDesc(Structure):
 
 
 class Tile(Structure):
-    _fields_ = [(n, c_int32) for n in ("mf", "mb", "nb", "wm", "wn", "wk", "cch", "tw", "ks", "wl", "wino")]
+    _fields_ = [(n, c_int32) for n in ("mf", "mb", "nb", "wm", "wn", "wk", "cch", "tw", "ks", "wl", "alg")]
 
-    def __init__(self, mf=0, mb=0, nb=0, wm=0, wn=0, wk=0, cch=0, tw=0, ks=1, wl=0, wino=0):
-        super().__init__(mf, mb, nb, wm, wn, wk, cch, tw, ks, wl, wino)
+    def __init__(self, mf=0, mb=0, nb=0, wm=0, wn=0, wk=0, cch=0, tw=0, ks=1, wl=0, alg=0):
+        super().__init__(mf, mb, nb, wm, wn, wk, cch, tw, ks, wl, alg)
 
     def astuple(self):
-        return (self.mf, self.mb, self.nb, self.wm, self.wn, self.wk, self.cch, self.tw, self.ks, self.wl, self.wino)
+        return (self.mf, self.mb, self.nb, self.wm, self.wn, self.wk, self.cch, self.tw, self.ks, self.wl, self.alg)
 
     def __repr__(self):
-        return "Tile(mf=%d, mb=%d, nb=%d, wm=%d, wn=%d, wk=%d, cch=%d, tw=%d, ks=%d, wl=%d, wino=%d)" % self.astuple()
+        return "Tile(mf=%d, mb=%d, nb=%d, wm=%d, wn=%d, wk=%d, cch=%d, tw=%d, ks=%d, wl=%d, alg=%d)" % self.astuple()
 
 
 class TileInfo(Structure):

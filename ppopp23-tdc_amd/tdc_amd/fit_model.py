@@ -26,7 +26,7 @@ def load(paths):
         for r in csv.DictReader(open(path)):
             key = tuple(int(r[k]) for k in ("C", "N", "H", "W", "K", "stride"))
             tile = _lib.Tile(*[int(r[k]) for k in ("mf", "mb", "nb", "wm", "wn", "wk", "cch", "tw")],
-                             ks=int(r.get("ks") or 1), wl=int(r.get("wl") or 0), wino=int(r.get("wino") or 0))
+                             ks=int(r.get("ks") or 1), wl=int(r.get("wl") or 0), alg=int(r.get("alg") or r.get("wino") or 0))
             layers[key].append((tile, float(r["time_us"])))
     return layers
 

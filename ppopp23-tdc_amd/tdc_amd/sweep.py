@@ -1,7 +1,7 @@
 """Measured tile sweep and model-loss report.
 
 For every shape, time every launchable tile through the C ABI, record
-``C,N,H,W,K,stride,mf,mb,nb,wm,wn,wk,cch,tw,ks,wl,wino,pred_us,time_us`` rows, and report how
+``C,N,H,W,K,stride,mf,mb,nb,wm,wn,wk,cch,tw,ks,wl,alg,pred_us,time_us`` rows, and report how
 much slower the analytic model's pick is than the measured best
 (``loss = t(model pick) / t(best) - 1``).  This is the gfx950 counterpart of the
 reference's brute-force occupancy/timing sweep
@@ -82,7 +82,7 @@ def main(argv=None):
         sys.exit("tdc_amd.sweep needs a GPU")
     log = open(a.out, "w") if a.out else None
     if log:
-        log.write("C,N,H,W,K,stride,mf,mb,nb,wm,wn,wk,cch,tw,ks,wl,wino,pred_us,time_us\n")
+        log.write("C,N,H,W,K,stride,mf,mb,nb,wm,wn,wk,cch,tw,ks,wl,alg,pred_us,time_us\n")
     total = 0.0
     n = 0
     t0 = time.time()

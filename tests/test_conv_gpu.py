@@ -76,16 +76,31 @@ def test_every_tile_3x3(shape):
                                        ((1, 16, 16, 12, 12), 2), ((1, 40, 24, 14, 14), 1), ((1, 3, 2, 2, 2), 1),
                                        ((1, 4, 4, 1, 9), 1)])
 def test_every_winograd_tile(shape, pad):
-    """The Winograd F(2x2,3x3) path (tile.wino = 1) with every launchable tile: odd image sizes (the last tile row
+    """The Winograd F(2x2,3x3) path (tile.alg = 1) with every launchable tile: odd image sizes (the last tile row
     and column are half outside), paddings 0..2, several passes, splits over waves and workgroups, loader waves."""
     B, C, N, H, W = shape
     x, w = case(1500 + C * N + H, B, C, N, H, W, 3)
     want = ref.conv2d_c(x.numpy(), w.numpy(), pad=pad)
-    tiles = [t for t in tdc_amd.model_enumerate(tdc_amd.conv_desc(B, C, N, H, W, 3, 3, 1, pad)) if t.wino]
+    tiles = [t for t in tdc_amd.model_enumerate(tdc_amd.conv_desc(B, C, N, H, W, 3, 3, 1, pad)) if t.alg == 1]
     assert tiles
     for t in tiles[::max(1, len(tiles) // 100)]:
         announce("winograd", shape, pad, t)
         assert_close(run_conv(x, w, pad=pad, tile=t), want, f"{shape} pad {pad} {t}")
+
+
+@pytest.mark.parametrize("shape,stride,pad", [((1, 8, 16, 8, 8), 1, 1), ((2, 13, 20, 9, 11), 1, 1), ((1, 40, 24, 13, 13), 2, 1),
+                                              ((1, 16, 16, 12, 12), 1, 2), ((1, 128, 48, 7, 7), 1, 1)])
+def test_every_global_weight_tile(shape, stride, pad):
+    """The direct 3x3 path that reads its weights from global memory into registers (tile.alg = 2), every launchable
+    tile: both MFMA shapes, stride 2, ragged channel counts (zero-filled channel groups), several passes."""
+    B, C, N, H, W = shape
+    x, w = case(1700 + C * N + H, B, C, N, H, W, 3)
+    want = ref.conv2d_c(x.numpy(), w.numpy(), stride=stride, pad=pad)
+    tiles = [t for t in tdc_amd.model_enumerate(tdc_amd.conv_desc(B, C, N, H, W, 3, 3, stride, pad)) if t.alg == 2]
+    assert tiles and {t.mf for t in tiles} == {16, 32}
+    for t in tiles[::max(1, len(tiles) // 100)]:
+        announce("global weights", shape, stride, pad, t)
+        assert_close(run_conv(x, w, stride=stride, pad=pad, tile=t), want, f"{shape} s{stride} p{pad} {t}")
 
 
 def test_winograd_epilogue_exactness_and_determinism():
@@ -355,7 +370,7 @@ def test_fused_1x1_tail(shape):
     desc = tdc_amd.conv_desc(B, C, N, H, W, K, K, stride, K // 2, 1, True, True)
     ok = []
     for t in tdc_amd.model_enumerate(desc):
-        if t.ks == 1 and t.mf * t.mb * t.wm >= N and not t.wino:    # (the Winograd path carries no tail)
+        if t.ks == 1 and t.mf * t.mb * t.wm >= N and not t.alg:    # (the Winograd path carries no tail)
             ok.append(t)
     assert ok
     xd, rd = x.cuda(), resid.cuda()

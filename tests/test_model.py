@@ -23,7 +23,7 @@ def test_every_candidate_is_launchable_and_covers_the_output(hw, r1, r2):
         i = tdc_amd.model_evaluate(d, t)
         lanes = t.mf * t.nb * t.wn
         # a Winograd lane stands for a 2x2-pixel tile and tw counts those
-        tw_px, lane_px = (2 * t.tw, 4) if t.wino else (t.tw, 1)
+        tw_px, lane_px = (2 * t.tw, 4) if t.alg == 1 else (t.tw, 1)
         assert 1 <= i.th and i.th * tw_px <= lanes * lane_px
         ntx, nty = math.ceil(hw / tw_px), math.ceil(hw / i.th)
         assert i.grid_x == ntx * nty and ntx * tw_px >= hw and nty * i.th >= hw     # tiles cover the image
@@ -35,7 +35,7 @@ def test_every_candidate_is_launchable_and_covers_the_output(hw, r1, r2):
 
 
 def test_winograd_tiles_only_where_the_algorithm_applies():
-    """tile.wino needs a 3x3 / stride 1 / dilation 1 convolution and one 16x16 block per wave; the model hands the
+    """tile.alg needs a 3x3 / stride 1 / dilation 1 convolution and one 16x16 block per wave; the model hands the
     large 56x56 layers to it and keeps the small ones on the direct path."""
     w = tdc_amd.Tile(16, 1, 1, 1, 2, 2, 32, 14, 1, 0, 1)
     assert tdc_amd.model_evaluate(conv3(128, 128, 56), w).th == 4           # 2 tile rows of 14 tiles = 4 x 28 pixels
@@ -48,9 +48,18 @@ def test_winograd_tiles_only_where_the_algorithm_applies():
                  (conv3(128, 128, 56), tdc_amd.Tile(16, 1, 1, 2, 4, 2, 32, 14, 1, 0, 1))]:   # 16 waves: over the budget of 8
         with pytest.raises(tdc_amd.TdcError):
             tdc_amd.model_evaluate(d, t)
-    assert tdc_amd.model_select(conv3(128, 128, 56)).tile.wino == 1
-    assert tdc_amd.model_select(conv3(32, 32, 14)).tile.wino == 0
-    assert not any(t.wino for t in tdc_amd.model_enumerate(conv3(64, 64, 56, stride=2)))
+    # alg = 2 (weights from global memory): 3x3 only, one block per wave, an even number of channel groups per wave
+    assert tdc_amd.model_evaluate(conv3(64, 64, 28), tdc_amd.Tile(16, 1, 1, 1, 1, 4, 64, 7, 1, 0, 2)).lds_bytes < \
+        tdc_amd.model_evaluate(conv3(64, 64, 28), tdc_amd.Tile(16, 1, 1, 1, 1, 4, 64, 7, 1, 0, 0)).lds_bytes
+    for d, t in [(tdc_amd.conv_desc(1, 64, 64, 56, 56, 1, 1, 1, 0), tdc_amd.Tile(16, 1, 1, 1, 1, 4, 64, 7, 1, 0, 2)),
+                 (conv3(64, 64, 28), tdc_amd.Tile(16, 2, 1, 1, 1, 4, 64, 7, 1, 0, 2)),
+                 (conv3(64, 64, 28), tdc_amd.Tile(16, 1, 1, 1, 1, 4, 16, 7, 1, 0, 2)),      # one channel group per wave
+                 (conv3(64, 64, 28), tdc_amd.Tile(16, 1, 1, 1, 1, 4, 64, 7, 1, 0, 3))]:
+        with pytest.raises(tdc_amd.TdcError):
+            tdc_amd.model_evaluate(d, t)
+    assert tdc_amd.model_select(conv3(128, 128, 56)).tile.alg == 1
+    assert tdc_amd.model_select(conv3(32, 32, 14)).tile.alg != 1
+    assert not any(t.alg == 1 for t in tdc_amd.model_enumerate(conv3(64, 64, 56, stride=2)))
 
 
 def test_algorithmic_work_and_roofline_of_config1():
