@@ -317,23 +317,24 @@ namespace {
 // (2080Ti-evaluation/TDC-LAYERS-MODELING/model.py:265-266,278).
 struct ModelConst {
     double launch_us = 1.474;           // device time of an empty kernel in a back-to-back stream
-    double setup_clk = 1208;          // kernel arguments and index arithmetic before the first copy is issued
-    double copy_latency_clk = 920.5;   // first byte of a global->LDS copy (L2 / memory-side cache)
-    double copy_bytes_per_clk = 34.32;   // sustained global->LDS rate of one CU
-    double l2_bytes_per_clk = 8183;   // whole-chip L2->CU rate when every CU copies at once
-    double lds_bytes_per_clk = 22.41;   // LDS traffic of the split-K reduction
+    double setup_clk = 1740;          // kernel arguments and index arithmetic before the first copy is issued
+    double copy_latency_clk = 665.1;   // first byte of a global->LDS copy (L2 / memory-side cache)
+    double copy_bytes_per_clk = 41.18;   // sustained global->LDS rate of one CU
+    double l2_bytes_per_clk = 8347;   // whole-chip L2->CU rate when every CU copies at once
+    double lds_bytes_per_clk = 22.86;   // LDS traffic of the split-K reduction
     double sync_clk = 275.2;            // one workgroup barrier
-    double store_bytes_per_clk = 3.326;  // per CU, short runs per channel
-    double kstep_issue_clk = 2.798;      // vector-ALU / LDS-issue cycles per operand read, not hidden under MFMAs
-    double pass_overhead_clk = 578.7;   // per wave and pass: copy issue, pointer set-up, pipeline fill
+    double store_bytes_per_clk = 2.827;  // per CU, short runs per channel
+    double kstep_issue_clk = 6.044;      // vector-ALU / LDS-issue cycles per operand read, not hidden under MFMAs
+    double pass_overhead_clk = 491.9;   // per wave and pass: copy issue, pointer set-up, pipeline fill
     double wave_setup_clk = 540.5;      // prologue cycles added per extra wave sharing a SIMD
     double ksplit_clk = 4604;         // split across workgroups: write-through, ticket round trip, read-back
-    double copy_issue_clk = 118.2;      // a wave is held this long by every global->LDS copy instruction it issues
+    double copy_issue_clk = 100.5;      // a wave is held this long by every global->LDS copy instruction it issues
     double lds_read_clk = 2.88;        // LDS busy cycles per conflict-free operand read of one wave
-    double wino_kstep_clk = 2.142;      // Winograd: cycles per MFMA that the input transform adds on top of the operand reads
+    double wino_kstep_clk = 13.99;      // Winograd: cycles per MFMA that the input transform adds on top of the operand reads
+    double gw_latency_clk = 1457;       // alg 2: the first weights come from L2 into registers after the input copy is under way
 };
 ModelConst MC;
-constexpr int kNumModelConst = 15;
+constexpr int kNumModelConst = 16;
 
 double *mc_field(int i) {
     switch (i) {
@@ -352,6 +353,7 @@ double *mc_field(int i) {
         case 12: return &MC.copy_issue_clk;
         case 13: return &MC.lds_read_clk;
         case 14: return &MC.wino_kstep_clk;
+        case 15: return &MC.gw_latency_clk;
         default: return nullptr;
     }
 }
@@ -452,7 +454,7 @@ bool model_evaluate(const tdc_conv_desc &d, const tdc_tile &t, tdc_tile_info &in
         const double copy = copy_bytes_pass * r / rate;
         // First pass is exposed; afterwards the copy of pass i+1 runs under the MFMAs of pass i.
         double clk = MC.setup_clk + MC.wave_setup_clk * ((double)wg_waves_per_simd * r - 1.0) + issue_first +
-                     MC.copy_latency_clk + copy;
+                     MC.copy_latency_clk + copy + (t.alg == 2 ? MC.gw_latency_clk : 0.0);
         clk += compute;  // last pass: nothing left to hide
         if (g.cps > 1) {
             const double pass = t.wl ? std::max(compute, std::max(issue_steady, copy) + MC.copy_latency_clk)
