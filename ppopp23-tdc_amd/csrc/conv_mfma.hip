@@ -23,6 +23,13 @@
 // B: the pixel lanes of a tile row read consecutive words, shifted by the tap)
 // and MB*NB MFMAs.
 //
+// Three inner loops share this frame (tile.alg):
+//   0  direct convolution as described, for every filter size (3x3 and 1x1 loops are specialised);
+//   1  Winograd F(2x2,3x3) for 3x3 / stride 1: a lane holds a 2x2 output tile, transforms its 4x4 input patch in
+//      registers and feeds 16 MFMAs per four input channels instead of 36;
+//   2  the direct 3x3 loop with its A operands read from global memory (L2) straight into registers.
+// In 1 and 2 the weights never pass through the LDS, which then stages input only, in longer passes.
+//
 // Differences from the reference kernel (template_benchmark_cudnn.template:365-402):
 //   * lanes index PIXELS, output channels live in the MFMA accumulator rows; the
 //     reference maps lane -> channel and broadcasts one LDS word to the warp;
