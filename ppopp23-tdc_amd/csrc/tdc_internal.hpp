@@ -79,6 +79,8 @@ bool model_set_constants(const double *in, int n);
 // OIHW [N,C,KH,KW] -> [channel tile][pass][M block in tile][channel group in pass][tap][64 lanes]
 // in MFMA A-operand order: lane l of an entry holds
 // w[tile*MT + mblk*mf + l%mf][pass*cch + cg*kc + l/mf][tap], zero outside N x C.
+// tile.alg = 2 regroups the nine taps of a channel group as [taps 0-3][lane][4] [taps 4-7][lane][4] [tap 8][lane];
+// tile.alg = 1 stores the 16 Winograd-domain values U = G g G^T of every (n, c) as [quarter][lane][4].
 size_t packed_weight_floats(const Geometry &g);
 void pack_weights(const tdc_conv_desc &d, const tdc_tile &t, const Geometry &g, const float *w_oihw, float *packed);
 
