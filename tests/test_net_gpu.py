@@ -90,6 +90,25 @@ def test_resnet18_batch2_small_resolution():
     net.close()
 
 
+def test_resnet18_with_measured_tile_selection():
+    """The same network with every tile choice (and every core + last fusion) measured at build time: the picks
+    may be Winograd or global-weight tiles, the logits must not move beyond the tolerance."""
+    import tdc_amd
+    p = nets.resnet18_params(seed=18)
+    x = torch.randn(1, 3, 224, 224, generator=torch.Generator().manual_seed(18))
+    want = nets_ref.tucker_resnet18_forward(p, x)
+    prev = tdc_amd.set_autotune(8)
+    try:
+        net = nets.build_tucker_resnet18(p, batch=1)
+    finally:
+        tdc_amd.set_autotune(prev)
+    print("kernels per forward:", net.num_kernels, flush=True)
+    got = net(x.cuda())
+    torch.cuda.synchronize()
+    scale_close(got.cpu().numpy().reshape(1, 1000), want.numpy(), "logits, measured selection")
+    net.close()
+
+
 @pytest.mark.parametrize("batch,res", [(1, 224), (8, 64)])
 def test_tucker_densenet121(batch, res):
     """Benchmark configuration 5 (batch 1 at 224x224; batch 8 at a reduced resolution to keep the CPU side short)."""
