@@ -103,6 +103,34 @@ def test_every_global_weight_tile(shape, stride, pad):
         assert_close(run_conv(x, w, stride=stride, pad=pad, tile=t), want, f"{shape} s{stride} p{pad} {t}")
 
 
+@pytest.mark.parametrize("W,c0", [(16, 0), (16, 3), (14, 3), (13, 1)])
+def test_winograd_into_channel_slices(W, c0):
+    """A Winograd tile reading from, adding a residual from, and writing into channel slices of wider buffers (the
+    strided entry point): the wide epilogue stores must respect the batch strides and fall back to narrower stores
+    when width or slice offset break their alignment."""
+    from ctypes import c_void_p
+    B, C, N, H = 2, 16, 24, 12
+    x, w = case(1900 + W + c0, B, C, N, H, W, 3)
+    g = seeded(1901)
+    bias = torch.randn(N, generator=g)
+    resid = torch.randn(B, N, H, W, generator=g)
+    want = (ref.conv2d_torch(x, w, pad=1) + bias.view(1, -1, 1, 1) + resid).clamp_min(0)
+    tile = tdc_amd.Tile(16, 1, 1, 1, 1, 2, 8, min(8, (W + 1) // 2), 1, 0, 1)
+    plan = tdc_amd.Conv2dPlan(B, C, N, H, W, 3, 3, 1, 1, 1, True, True, tile=tile).set_weights(w, bias)
+    xin = torch.zeros(B, C + 5, H, W, device="cuda"); xin[:, 2:2 + C] = x.cuda()
+    rbuf = torch.zeros(B, N + 7, H, W, device="cuda"); rbuf[:, c0:c0 + N] = resid.cuda()
+    obuf = torch.full((B, N + 9, H, W), 7.0, device="cuda")
+    P = H * W
+    tdc_amd._lib.check(tdc_amd.lib().tdc_conv_forward_strided(
+        plan._h, c_void_p(xin[:, 2:].data_ptr()), (C + 5) * P, c_void_p(rbuf[:, c0:].data_ptr()), (N + 7) * P,
+        c_void_p(obuf[:, c0:].data_ptr()), (N + 9) * P, c_void_p(torch.cuda.current_stream().cuda_stream)))
+    torch.cuda.synchronize()
+    got = obuf.cpu()
+    assert_close(got[:, c0:c0 + N].numpy(), want.numpy(), f"winograd slices W={W} c0={c0}")
+    assert (got[:, :c0] == 7.0).all() and (got[:, c0 + N:] == 7.0).all()      # nothing written outside the slice
+    plan.close()
+
+
 def test_winograd_epilogue_exactness_and_determinism():
     """Winograd tiles on a benchmark layer: bias + residual + ReLU, the same bits on every launch, and the
     reference's integer known-answer test stays exact (the transformed weights 1, 3/2, 1/2, 9/4, 3/4, 1/4 and all
