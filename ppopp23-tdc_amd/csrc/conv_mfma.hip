@@ -1045,6 +1045,121 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
 }
 
 // ---------------------------------------------------------------------------
+// 1x1 convolution with many input channels over few pixels (tile.alg = 3): no LDS stage, no passes, no barrier
+// before the reduction.  One workgroup owns a 16-channel x 16-pixel block of the output; its WK waves split the
+// input channels, NQ runs of 16 channels each.  A wave requests ALL its operands up front, straight into
+// registers (per run: one 128-bit load of packed weights, four 32-bit loads of the input, and two 128-bit loads of
+// the input affine if there is one), then issues its 4*NQ MFMAs as the data arrives and leaves its 16x16 partial
+// in LDS for wave 0 to add up in a fixed order.  Within a run lane (k, n) takes channels 16q + 4k + s over the four
+// K-steps s, so that its weights and its scale/shift pairs are contiguous.
+// Channels past C read as zero (range-checked vector offsets) and meet zero weights; pixel lanes past the image
+// re-read its last pixel and are never stored.
+// ---------------------------------------------------------------------------
+// (eight runs per wave: 72 registers of operands, 136 with the affine; that variant is built for at most 8 waves)
+template <int NQ, bool AFF>
+__global__ void __launch_bounds__(NQ == 8 ? 512 : 1024) tdc_conv1x1_stream_kernel(const ConvKParams p) {
+    extern __shared__ __align__(16) float lds[];
+    if constexpr (TDC_TOUCH_KERNARGS) {
+        static_assert(sizeof(ConvKParams) <= 8 * 64, "touch more lines");
+        const auto kargs = __builtin_amdgcn_kernarg_segment_ptr();
+        unsigned t0, t1, t2, t3, t4, t5, t6, t7;
+        asm volatile(
+            "s_load_dword %0, %8, 0x0\n\ts_load_dword %1, %8, 0x40\n\ts_load_dword %2, %8, 0x80\n\t"
+            "s_load_dword %3, %8, 0xc0\n\ts_load_dword %4, %8, 0x100\n\ts_load_dword %5, %8, 0x140\n\t"
+            "s_load_dword %6, %8, 0x180\n\ts_load_dword %7, %8, 0x1c0\n\ts_waitcnt lgkmcnt(0)"
+            : "=&s"(t0), "=&s"(t1), "=&s"(t2), "=&s"(t3), "=&s"(t4), "=&s"(t5), "=&s"(t6), "=&s"(t7)
+            : "s"(kargs)
+            : "memory");
+    }
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // = this wave's slice of the input channels
+    // same die-aware decoding of the one-dimensional launch as the staged kernel
+    const int logical = (int)(blockIdx.x & 7u) * p.xcd_chunk + (int)(blockIdx.x >> 3);
+    if (logical >= p.n_wg) return;
+    const int q1 = fdiv(logical, p.fd_g1);
+    const int r1 = logical - q1 * p.fd_g1.d;
+    const int img = fdiv(q1, p.fd_g2);
+    const int r2 = q1 - img * p.fd_g2.d;
+    const int bx = p.channel_major ? r1 : r2;  // pixel block
+    const int by = p.channel_major ? r2 : r1;  // channel block
+    const float *__restrict__ in = p.in + (long long)img * p.in_bstride;
+    float *__restrict__ out = p.out + (long long)img * p.out_bstride;
+    const float *__restrict__ resid = p.resid ? p.resid + (long long)img * p.resid_bstride : nullptr;
+    const __amdgpu_buffer_rsrc_t in_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(in), (short)0, (int)p.in_image_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t w_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.wpk), (short)0, (int)p.wpk_bytes, 0x00020000);
+
+    const int k = lane >> 4, n = lane & 15;
+    const int px = bx * 16 + n;
+    const int pxr = min(px, p.P - 1);
+    const int c0 = wave * (16 * NQ) + 4 * k;   // this lane's first channel
+    const unsigned HW4 = (unsigned)p.W * 4u;   // bytes between channels (the image is one row of H*W pixels)
+
+    f4_t a[NQ], sc[NQ], sh[NQ];
+    float b[NQ][4];
+    const int a_soff = (by * (p.CCH >> 4) + wave * NQ) * 1024;
+    const unsigned b_voff = (unsigned)c0 * HW4 + (unsigned)pxr * 4u;
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) {
+        a[q] = __builtin_bit_cast(f4_t, __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, lane * 16, a_soff + q * 1024, 0));
+#pragma unroll
+        for (int s4 = 0; s4 < 4; ++s4)   // (the whole offset goes through the range-checked vector operand)
+            b[q][s4] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(in_rsrc, (int)(b_voff + (unsigned)(16 * q + s4) * HW4), 0, 0));
+        if constexpr (AFF) {
+            const __amdgpu_buffer_rsrc_t aff_rsrc =
+                __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.in_aff), (short)0, p.CCH * 8, 0x00020000);
+            sc[q] = __builtin_bit_cast(f4_t, __builtin_amdgcn_raw_buffer_load_b128(aff_rsrc, (c0 + 16 * q) * 4, 0, 0));
+            sh[q] = __builtin_bit_cast(f4_t, __builtin_amdgcn_raw_buffer_load_b128(aff_rsrc, (p.CCH + c0 + 16 * q) * 4, 0, 0));
+        }
+        __builtin_amdgcn_sched_barrier(0);   // requests in the order the MFMAs consume them
+    }
+    // (every request is issued before the first MFMA: the scheduler must not sink loads into the MFMA sequence)
+    __builtin_amdgcn_sched_barrier(0);
+    // two accumulator chains: consecutive MFMAs do not wait for each other's result
+    f4_t acc0 = (f4_t){0.0f, 0.0f, 0.0f, 0.0f}, acc1 = (f4_t){0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) {
+#pragma unroll
+        for (int s4 = 0; s4 < 4; ++s4) {
+            float v = b[q][s4];
+            if constexpr (AFF) {
+                v = v * sc[q][s4] + sh[q][s4];
+                if (p.in_relu) v = fmaxf(v, 0.0f);
+            }
+            if (s4 & 1) acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(a[q][s4], v, acc1, 0, 0, 0);
+            else acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(a[q][s4], v, acc0, 0, 0, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);   // run by run, as the data arrives
+    }
+    f4_t acc = acc0 + acc1;
+    // lane l holds rows 4*(l/16) .. +3 (output channels) of column l%16 (pixel)
+    if (p.WK > 1) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) lds[(wave * 4 + i) * 64 + lane] = acc[i];
+        __syncthreads();
+        if (wave != 0) return;
+        acc = (f4_t){0.0f, 0.0f, 0.0f, 0.0f};
+        for (int w = 0; w < p.WK; ++w)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[i] += lds[(w * 4 + i) * 64 + lane];
+    }
+    if (px >= p.P) return;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int ch = by * 16 + 4 * k + i;
+        if (ch >= p.N) continue;
+        float val = acc[i];
+        if (p.bias) val += p.bias[ch];
+        const long long o = (long long)ch * p.P + px;
+        if (resid) val += resid[o];
+        if (p.relu) val = fmaxf(val, 0.0f);
+        out[o] = val;
+    }
+}
+
+// ---------------------------------------------------------------------------
 // Instantiation table.  A 2x2 block grid of MFMAs per wave is built for at
 // most 8 waves per workgroup (256 registers per lane); everything else for 16.
 // ---------------------------------------------------------------------------
@@ -1072,8 +1187,27 @@ static int taps_mode(int KH, int KW, int dil) {
     return TAPS_GENERIC;
 }
 
+template <bool AFF>
+static kernel_fn pick_stream(int nq) {
+    switch (nq) {
+        case 1: return tdc_conv1x1_stream_kernel<1, AFF>;
+        case 2: return tdc_conv1x1_stream_kernel<2, AFF>;
+        case 4: return tdc_conv1x1_stream_kernel<4, AFF>;
+        case 8: return tdc_conv1x1_stream_kernel<8, AFF>;
+        default: return nullptr;
+    }
+}
+
 const void *conv_kernel_for(const tdc_tile &t, int KH, int KW, int dilation, bool extras) {
     kernel_fn fn = nullptr;
+    if (t.alg == 3) {
+        // (`extras` here can only mean the input affine: the host refuses a fused tail for this path)
+        if (KH != 1 || KW != 1 || t.mf != 16 || t.mb != 1 || t.nb != 1 || t.wm != 1 || t.wn != 1 || t.wk < 1) return nullptr;
+        if (t.cch % (16 * t.wk) != 0) return nullptr;
+        const int nq = t.cch / (16 * t.wk);
+        if (t.wk > (nq == 8 ? 8 : 16)) return nullptr;
+        return reinterpret_cast<const void *>(extras ? pick_stream<true>(nq) : pick_stream<false>(nq));
+    }
     if (t.alg == 1) {
         if (extras || KH != 3 || KW != 3 || dilation != 1 || t.mf != 16 || t.mb != 1 || t.nb != 1) return nullptr;
         return reinterpret_cast<const void *>(static_cast<kernel_fn>(tdc_conv_mfma_kernel<16, 1, 1, TAPS_WINO, 12, false>));

@@ -132,8 +132,22 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
     g.taps = d.KH * d.KW;
     g.ktaps = g.taps;
     g.MT = t.mf * t.mb * t.wm;
-    if (t.alg < 0 || t.alg > 2) return fail("tile.alg must be 0, 1 or 2");
+    if (t.alg < 0 || t.alg > 3) return fail("tile.alg must be 0, 1, 2 or 3");
     g.wino = t.alg == 1;
+    if (t.alg == 3) {
+        // 1x1 convolution streamed from global memory: a 16x16 output block per workgroup, the input channels split
+        // over wk waves in runs of 16, everything in one pass
+        if (!flat) return fail("tile.alg = 3 needs a 1x1 / stride 1 / pad 0 convolution");
+        if (t.mf != 16 || t.mb != 1 || t.nb != 1 || t.wm != 1 || t.wn != 1) return fail("tile.alg = 3 needs mf = 16 and one block per workgroup");
+        if (t.ks != 1 || t.wl != 0) return fail("tile.alg = 3 has no split across workgroups and no loader waves");
+        if (tail_N > 0) return fail("tile.alg = 3 cannot carry a fused tail");
+        const int runs = (t.cch % (16 * t.wk) == 0) ? t.cch / (16 * t.wk) : 0;
+        if (runs != 1 && runs != 2 && runs != 4 && runs != 8) return fail("tile.alg = 3 needs cch = 16 * wk * {1, 2, 4, 8}");
+        if (runs == 8 && t.wk > 8) return fail("tile.alg = 3 with eight runs per wave is built for at most 8 waves");
+        if (t.cch < d.C) return fail("tile.alg = 3 takes all input channels in one pass");
+        if (t.tw != std::min(16, g.Wo)) return fail("tile.alg = 3 needs tw = min(16, pixels)");
+        if ((long long)t.cch * g.We * 4 >= (1LL << 31)) return fail("image too large for tile.alg = 3");
+    }
     if (t.alg == 2) {
         // direct 3x3 convolution with the weights read from global memory into registers, a pair of channel groups at a time
         if (d.KH != 3 || d.KW != 3 || d.dilation != 1) return fail("tile.alg = 2 needs a 3x3 / dilation 1 convolution");
@@ -175,7 +189,7 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
     if (g.grid_y > 65535) return fail("grid too large");
     const int granule = g.kc * t.wk;
     if (t.cch < granule || t.cch % granule != 0) return fail("tile.cch must be a positive multiple of kc*wk");
-    if (t.cch > round_up(d.C, granule)) return fail("tile.cch exceeds the (padded) channel count");
+    if (t.alg != 3 && t.cch > round_up(d.C, granule)) return fail("tile.cch exceeds the (padded) channel count");
     g.cpw = t.cch / t.wk;
     g.nchunks = ceil_div(d.C, t.cch);
     g.c_pad = g.nchunks * t.cch;
@@ -207,6 +221,7 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
     g.aff_floats = (d.KH == 1 && d.KW == 1 && d.pad == 0) ? round_up(2 * t.cch, 256) : 0;
     // (the Winograd path reads its weights straight from global memory into registers: the LDS holds input only)
     g.stage_floats = g.in_stage_floats + (t.alg ? 0 : round_up(g.wslab_floats, 256)) + g.aff_floats;   // (wino = 2 likewise)
+    if (t.alg == 3) g.in_stage_floats = g.aff_floats = g.stage_floats = 0;   // nothing is staged
     g.nstage = g.cps > 1 ? 2 : 1;
     const long long stage_bytes = (long long)g.nstage * g.stage_floats * 4;
     // (the Winograd path always parks its output tiles in LDS, also without a split over waves)
@@ -266,6 +281,19 @@ void pack_weights(const tdc_conv_desc &d, const tdc_tile &t, const Geometry &g, 
                                 const float v = (n < d.N && c < d.C) ? w[((size_t)n * d.C + c) * 9 + tap] : 0.0f;
                                 dst[tap < 8 ? (tap / 4) * 256 + l * 4 + tap % 4 : 512 + l] = v;
                             }
+        return;
+    }
+    if (t.alg == 3) {
+        // per (channel block, run of 16 input channels): [lane][s], lane (n = l % 16, k = l / 16) holding
+        // w[block*16 + n][16*run + 4*k + s]
+        const int runs = t.cch / 16;
+        for (int by = 0; by < g.grid_y; ++by)
+            for (int r = 0; r < runs; ++r)
+                for (int l = 0; l < 64; ++l)
+                    for (int e = 0; e < 4; ++e) {
+                        const int n = by * 16 + l % 16, c = 16 * r + 4 * (l / 16) + e;
+                        *dst++ = (n < d.N && c < d.C) ? w[(size_t)n * d.C + c] : 0.0f;
+                    }
         return;
     }
     if (g.wino) {
@@ -332,9 +360,11 @@ struct ModelConst {
     double lds_read_clk = 2.88;        // LDS busy cycles per conflict-free operand read of one wave
     double wino_kstep_clk = 13.99;      // Winograd: cycles per MFMA that the input transform adds on top of the operand reads
     double gw_latency_clk = 1457;       // alg 2: the first weights come from L2 into registers after the input copy is under way
+    double stream_setup_clk = 250;      // alg 3: index arithmetic before the requests go out (no copy tables, no stages)
+    double stream_latency_clk = 645;    // alg 3: round trip of the first request, global memory -> registers
 };
 ModelConst MC;
-constexpr int kNumModelConst = 16;
+constexpr int kNumModelConst = 18;
 
 double *mc_field(int i) {
     switch (i) {
@@ -354,6 +384,8 @@ double *mc_field(int i) {
         case 13: return &MC.lds_read_clk;
         case 14: return &MC.wino_kstep_clk;
         case 15: return &MC.gw_latency_clk;
+        case 16: return &MC.stream_setup_clk;
+        case 17: return &MC.stream_latency_clk;
         default: return nullptr;
     }
 }
@@ -365,6 +397,7 @@ int kernel_vgprs(const tdc_tile &t, int taps_mode) {
     if (taps_mode == 9) regs += 6 * t.nb;
     if (t.alg == 1) regs = 136;   // 64 accumulators, two sets of 16 B and 16 A operands, the raw patch
     if (t.alg == 2) regs = 104;   // two sets of 18 A and 18 B operands
+    if (t.alg == 3) regs = 40 + 16 * (t.cch / (16 * t.wk));   // per run of 16 channels: 4 A, 4 B, 8 scale/shift
     return round_up(regs, 8);
 }
 
@@ -391,7 +424,8 @@ bool model_evaluate(const tdc_conv_desc &d, const tdc_tile &t, tdc_tile_info &in
     const int wg_waves_per_simd = ceil_div(g.waves, m.simds_per_cu);
     const int wg_by_vgpr = waves_simd_vgpr / wg_waves_per_simd;
     const int wg_by_lds = m.lds_bytes_per_cu / std::max(g.lds_bytes, 1);
-    int wg_per_cu = std::min(std::min(wg_by_vgpr, wg_by_lds), 8);
+    // (the staged kernels are never resident more than eight times per CU; the streamed one has no stage to hold)
+    int wg_per_cu = std::min(std::min(wg_by_vgpr, wg_by_lds), t.alg == 3 ? 32 : 8);
     if (wg_per_cu < 1) {
         if (why) *why = "tile does not fit one compute unit";
         return false;
@@ -434,6 +468,23 @@ bool model_evaluate(const tdc_conv_desc &d, const tdc_tile &t, tdc_tile_info &in
     const int comp_waves_per_simd = ceil_div(ncomp, m.simds_per_cu);
 
     auto wg_time = [&](int r, long long concurrent_wgs) {
+        if (t.alg == 3) {
+            // every wave requests its whole share up front and works through it as it arrives: one round trip, the
+            // bytes at the CU's (or the chip's) fill rate, two chains of dependent MFMAs, the reduction over the waves
+            const double chip_share =
+                MC.l2_bytes_per_clk / std::max<double>(1.0, (double)std::min<long long>(concurrent_wgs, m.cus));
+            const double rate = std::min(MC.copy_bytes_per_clk, chip_share);
+            const double bytes = (double)t.cch * (64.0 + 64.0) * r;   // weights and input of one 16x16 block
+            const double runs = (double)t.cch / (16.0 * t.wk);
+            const double waves_simd = std::ceil((double)g.waves * r / m.simds_per_cu);
+            // (fitted to 71 timed tiles of 23 shapes: the requests of all resident waves overlap, so only the bytes,
+            //  a little per extra wave and half an MFMA time per K-step show; the stores are hidden)
+            double clk = MC.stream_setup_clk + MC.stream_latency_clk + 20.0 * (waves_simd - 1.0) + bytes / (0.87 * rate) +
+                         runs * 4.0 * 0.5 * mfma_clk * waves_simd;
+            if (t.wk > 1) clk += 1.5 * MC.sync_clk;
+            clk += out_bytes * r / 64.0;
+            return clk;
+        }
         // r workgroups share one CU: matrix time and the issue cycles of the operand reads add up per
         // SIMD; copies share the CU's fill rate and, chip-wide, the L2.
         const double waves_simd = (double)comp_waves_per_simd * r;
@@ -500,6 +551,18 @@ std::vector<tdc_tile> model_enumerate(const tdc_conv_desc &d, int tail_N) {
     static const int wks[] = {1, 2, 4, 8, 16};
     static const int wms[] = {1, 2, 4};
     static const int wns[] = {1, 2, 4};
+    // streamed 1x1 candidates: the input channels in runs of 16, 1, 2, 4 or 8 runs per wave
+    if (flat && tail_N == 0 && !std::getenv("TDC_EXPERIMENT_NO_STREAMED_1X1")) {
+        const int runs = ceil_div(d.C, 16);
+        for (int per_wave : {8, 4, 2, 1}) {
+            if (per_wave > runs) continue;   // (more than half of such a wave's channels would be padding)
+            const int wk = ceil_div(runs, per_wave);
+            if (wk > 16) continue;
+            tdc_tile t{16, 1, 1, 1, 1, wk, 16 * per_wave * wk, std::min(16, Wo), 1, 0, 3};
+            Geometry g;
+            if (make_geometry(d, t, g, nullptr, 0)) out.push_back(t);
+        }
+    }
     // Winograd candidates for 3x3 / stride 1 convolutions with enough pixels to fill tile lanes
     if (d.KH == 3 && d.KW == 3 && d.stride == 1 && d.dilation == 1 && tail_N == 0 && !std::getenv("TDC_EXPERIMENT_NO_WINOGRAD")) {
         const int Wt = ceil_div(Wo, 2), Ht = ceil_div(Ho, 2);

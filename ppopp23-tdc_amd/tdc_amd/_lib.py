@@ -168,7 +168,8 @@ def model_evaluate(desc: ConvDesc, tile: Tile) -> TileInfo:
 
 MODEL_CONSTANT_NAMES = ("launch_us", "setup_clk", "copy_latency_clk", "copy_bytes_per_clk", "l2_bytes_per_clk",
                         "lds_bytes_per_clk", "sync_clk", "store_bytes_per_clk", "kstep_issue_clk", "pass_overhead_clk",
-                        "wave_setup_clk", "ksplit_clk", "copy_issue_clk", "lds_read_clk", "wino_kstep_clk", "gw_latency_clk")
+                        "wave_setup_clk", "ksplit_clk", "copy_issue_clk", "lds_read_clk", "wino_kstep_clk", "gw_latency_clk",
+                        "stream_setup_clk", "stream_latency_clk")
 
 
 def model_select_with_tail(desc: ConvDesc, tail_N: int):

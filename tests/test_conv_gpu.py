@@ -103,6 +103,52 @@ def test_every_global_weight_tile(shape, stride, pad):
         assert_close(run_conv(x, w, stride=stride, pad=pad, tile=t), want, f"{shape} s{stride} p{pad} {t}")
 
 
+@pytest.mark.parametrize("shape", [(1, 64, 16, 7, 7), (2, 100, 40, 5, 6), (1, 288, 128, 14, 14), (1, 1024, 128, 7, 7),
+                                   (1, 512, 1000, 1, 1), (3, 19, 5, 3, 3), (1, 256, 64, 20, 20)])
+def test_every_streamed_1x1_tile(shape):
+    """The 1x1 path that streams both operands from global memory into registers (tile.alg = 3): every launchable
+    tile (1, 2, 4 or 8 runs of 16 channels per wave, 1 to 16 waves), ragged channel and pixel counts, a single pixel,
+    batches; plain, with bias + residual + ReLU written into a channel slice of a wider buffer, and with the input
+    affine (+ReLU) in front."""
+    from ctypes import c_void_p
+    B, C, N, H, W = shape
+    x, w = case(2300 + C + N + H, B, C, N, H, W, 1)
+    g = seeded(2301)
+    bias = torch.randn(N, generator=g)
+    resid = torch.randn(B, N, H, W, generator=g)
+    scale = torch.rand(C, generator=g) * 2 - 0.5
+    shift = torch.randn(C, generator=g) * 0.3
+    want_plain = ref.conv2d_c(x.numpy(), w.numpy())
+    want_full = (ref.conv2d_torch(x, w) + bias.view(1, -1, 1, 1) + resid).clamp_min(0).numpy()
+    xt = (x * scale.view(1, C, 1, 1) + shift.view(1, C, 1, 1)).clamp_min(0)
+    want_aff = ref.conv2d_c(xt.numpy(), w.numpy(), bias.numpy(), relu=True)
+    tiles = [t for t in tdc_amd.model_enumerate(tdc_amd.conv_desc(B, C, N, H, W, 1, 1, 1, 0)) if t.alg == 3]
+    assert tiles
+    P = H * W
+    for t in tiles:
+        announce("streamed 1x1", shape, t)
+        assert_close(run_conv(x, w, tile=t), want_plain, f"{shape} {t}")
+        # bias + residual + ReLU, input and output as channel slices of wider buffers
+        plan = tdc_amd.Conv2dPlan(B, C, N, H, W, 1, 1, 1, 0, 1, True, True, tile=t).set_weights(w, bias)
+        xin = torch.zeros(B, C + 3, H, W, device="cuda"); xin[:, 1:1 + C] = x.cuda()
+        rbuf = torch.zeros(B, N + 2, H, W, device="cuda"); rbuf[:, 2:] = resid.cuda()
+        obuf = torch.full((B, N + 5, H, W), 7.0, device="cuda")
+        tdc_amd._lib.check(tdc_amd.lib().tdc_conv_forward_strided(
+            plan._h, c_void_p(xin[:, 1:].data_ptr()), (C + 3) * P, c_void_p(rbuf[:, 2:].data_ptr()), (N + 2) * P,
+            c_void_p(obuf[:, 4:].data_ptr()), (N + 5) * P, c_void_p(torch.cuda.current_stream().cuda_stream)))
+        torch.cuda.synchronize()
+        got = obuf.cpu()
+        assert_close(got[:, 4:4 + N].numpy(), want_full, f"slices {shape} {t}")
+        assert (got[:, :4] == 7.0).all() and (got[:, 4 + N:] == 7.0).all()
+        # the input affine in front
+        plan.set_input_affine(scale, shift, relu=True)
+        out = torch.full((B, N, H, W), float("nan"), device="cuda")
+        plan.forward(x.cuda(), out=out)
+        torch.cuda.synchronize()
+        plan.close()
+        assert_close(out.cpu().numpy(), want_aff, f"input affine {shape} {t}")
+
+
 @pytest.mark.parametrize("W,c0", [(16, 0), (16, 3), (14, 3), (13, 1)])
 def test_winograd_into_channel_slices(W, c0):
     """A Winograd tile reading from, adding a residual from, and writing into channel slices of wider buffers (the
