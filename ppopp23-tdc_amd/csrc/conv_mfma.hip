@@ -1187,6 +1187,118 @@ static int taps_mode(int KH, int KW, int dil) {
     return TAPS_GENERIC;
 }
 
+// ---------------------------------------------------------------------------
+// 3x3 convolution streamed the same way (tile.alg = 4): one workgroup owns 16 output channels of a TH x TW tile of 16
+// pixels, its WK waves split the input channels, CG groups of four channels each.  Per group a lane requests its nine
+// input values (one per tap, four channels across the lane quarters) and its nine weights (packed as for
+// tile.alg = 2: two 128-bit loads and one 32-bit load); padding, channels past C and lanes past the tile present an
+// out-of-range offset and read zero without a memory access.
+// ---------------------------------------------------------------------------
+template <int CG>
+__global__ void __launch_bounds__(1024) tdc_conv3x3_stream_kernel(const ConvKParams p) {
+    extern __shared__ __align__(16) float lds[];
+    if constexpr (TDC_TOUCH_KERNARGS) {
+        const auto kargs = __builtin_amdgcn_kernarg_segment_ptr();
+        unsigned t0, t1, t2, t3, t4, t5, t6, t7;
+        asm volatile(
+            "s_load_dword %0, %8, 0x0\n\ts_load_dword %1, %8, 0x40\n\ts_load_dword %2, %8, 0x80\n\t"
+            "s_load_dword %3, %8, 0xc0\n\ts_load_dword %4, %8, 0x100\n\ts_load_dword %5, %8, 0x140\n\t"
+            "s_load_dword %6, %8, 0x180\n\ts_load_dword %7, %8, 0x1c0\n\ts_waitcnt lgkmcnt(0)"
+            : "=&s"(t0), "=&s"(t1), "=&s"(t2), "=&s"(t3), "=&s"(t4), "=&s"(t5), "=&s"(t6), "=&s"(t7)
+            : "s"(kargs)
+            : "memory");
+    }
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int logical = (int)(blockIdx.x & 7u) * p.xcd_chunk + (int)(blockIdx.x >> 3);
+    if (logical >= p.n_wg) return;
+    const int q1 = fdiv(logical, p.fd_g1);
+    const int r1 = logical - q1 * p.fd_g1.d;
+    const int img = fdiv(q1, p.fd_g2);
+    const int r2 = q1 - img * p.fd_g2.d;
+    const int bx = p.channel_major ? r1 : r2;  // pixel tile
+    const int by = p.channel_major ? r2 : r1;  // channel block
+    const int tile_y = fdiv(bx, p.fd_ntx);
+    const int tile_x = bx - tile_y * p.ntx;
+    const float *__restrict__ in = p.in + (long long)img * p.in_bstride;
+    float *__restrict__ out = p.out + (long long)img * p.out_bstride;
+    const float *__restrict__ resid = p.resid ? p.resid + (long long)img * p.resid_bstride : nullptr;
+    const __amdgpu_buffer_rsrc_t in_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(in), (short)0, (int)p.in_image_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t w_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.wpk), (short)0, (int)p.wpk_bytes, 0x00020000);
+
+    const int k = lane >> 4, n = lane & 15;
+    const int jy = fdiv(n, p.fd_tw);
+    const int jx = n - jy * p.TW;
+    const int oy = tile_y * p.TH + jy, ox = tile_x * p.TW + jx;
+    const bool live = jy < p.TH && oy < p.Ho && ox < p.Wo;
+    // byte offset of every tap inside one channel, or the out-of-range offset
+    unsigned toff[9];
+#pragma unroll
+    for (int r = 0; r < 3; ++r)
+#pragma unroll
+        for (int c = 0; c < 3; ++c) {
+            const int iy = oy * p.stride - p.pad + r, ix = ox * p.stride - p.pad + c;
+            const bool ok = live && iy >= 0 && iy < p.H && ix >= 0 && ix < p.W;
+            toff[r * 3 + c] = ok ? (unsigned)(iy * p.W + ix) * 4u : (unsigned)OOB_OFFSET;
+        }
+    const unsigned chan_bytes = (unsigned)(p.H * p.W) * 4u;
+    const unsigned base = (unsigned)(wave * (4 * CG) + k) * chan_bytes;   // this lane's first channel
+    const int a_soff = (by * (p.CCH >> 2) + wave * CG) * 2304;            // nine taps x 64 lanes x 4 bytes per group
+
+    f4_t a0[CG], a1[CG];
+    float a8[CG], b[CG][9];
+#pragma unroll
+    for (int g = 0; g < CG; ++g) {
+        a0[g] = __builtin_bit_cast(f4_t, __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, lane * 16, a_soff + g * 2304, 0));
+        a1[g] = __builtin_bit_cast(f4_t, __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, lane * 16, a_soff + g * 2304 + 1024, 0));
+        a8[g] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(w_rsrc, lane * 4, a_soff + g * 2304 + 2048, 0));
+#pragma unroll
+        for (int t = 0; t < 9; ++t)   // (the whole offset goes through the range-checked vector operand)
+            b[g][t] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                in_rsrc, (int)(toff[t] + base + (unsigned)(4 * g) * chan_bytes), 0, 0));
+        __builtin_amdgcn_sched_barrier(0);   // requests in the order the MFMAs consume them
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    f4_t acc0 = (f4_t){0.0f, 0.0f, 0.0f, 0.0f}, acc1 = (f4_t){0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int g = 0; g < CG; ++g) {
+#pragma unroll
+        for (int t = 0; t < 9; ++t) {
+            const float av = t < 4 ? a0[g][t] : t < 8 ? a1[g][t - 4] : a8[g];
+            if (t & 1) acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(av, b[g][t], acc1, 0, 0, 0);
+            else acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(av, b[g][t], acc0, 0, 0, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);   // group by group, as the data arrives
+    }
+    f4_t acc = acc0 + acc1;
+    if (p.WK > 1) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) lds[(wave * 4 + i) * 64 + lane] = acc[i];
+        __syncthreads();
+        if (wave != 0) return;
+        acc = (f4_t){0.0f, 0.0f, 0.0f, 0.0f};
+        for (int w = 0; w < p.WK; ++w)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[i] += lds[(w * 4 + i) * 64 + lane];
+    }
+    if (!live) return;
+    const int pp = oy * p.Wo + ox;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int ch = by * 16 + 4 * k + i;
+        if (ch >= p.N) continue;
+        float val = acc[i];
+        if (p.bias) val += p.bias[ch];
+        const long long o = (long long)ch * p.P + pp;
+        if (resid) val += resid[o];
+        if (p.relu) val = fmaxf(val, 0.0f);
+        out[o] = val;
+    }
+}
+
 template <bool AFF>
 static kernel_fn pick_stream(int nq) {
     switch (nq) {
@@ -1200,6 +1312,16 @@ static kernel_fn pick_stream(int nq) {
 
 const void *conv_kernel_for(const tdc_tile &t, int KH, int KW, int dilation, bool extras) {
     kernel_fn fn = nullptr;
+    if (t.alg == 4) {
+        if (extras || KH != 3 || KW != 3 || dilation != 1 || t.mf != 16 || t.mb != 1 || t.nb != 1 || t.wm != 1 || t.wn != 1 || t.wk < 1 || t.wk > 16)
+            return nullptr;
+        switch (t.cch % (4 * t.wk) == 0 ? t.cch / (4 * t.wk) : 0) {
+            case 1: return reinterpret_cast<const void *>(static_cast<kernel_fn>(tdc_conv3x3_stream_kernel<1>));
+            case 2: return reinterpret_cast<const void *>(static_cast<kernel_fn>(tdc_conv3x3_stream_kernel<2>));
+            case 4: return reinterpret_cast<const void *>(static_cast<kernel_fn>(tdc_conv3x3_stream_kernel<4>));
+            default: return nullptr;
+        }
+    }
     if (t.alg == 3) {
         // (`extras` here can only mean the input affine: the host refuses a fused tail for this path)
         if (KH != 1 || KW != 1 || t.mf != 16 || t.mb != 1 || t.nb != 1 || t.wm != 1 || t.wn != 1 || t.wk < 1) return nullptr;

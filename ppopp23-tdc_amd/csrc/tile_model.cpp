@@ -132,7 +132,19 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
     g.taps = d.KH * d.KW;
     g.ktaps = g.taps;
     g.MT = t.mf * t.mb * t.wm;
-    if (t.alg < 0 || t.alg > 3) return fail("tile.alg must be 0, 1, 2 or 3");
+    if (t.alg < 0 || t.alg > 4) return fail("tile.alg must be in [0, 4]");
+    if (t.alg == 4) {
+        // 3x3 convolution streamed from global memory: 16 channels x 16 pixels per workgroup, the input channels
+        // split over wk waves in groups of four, everything in one pass
+        if (d.KH != 3 || d.KW != 3 || d.dilation != 1) return fail("tile.alg = 4 needs a 3x3 / dilation 1 convolution");
+        if (t.mf != 16 || t.mb != 1 || t.nb != 1 || t.wm != 1 || t.wn != 1) return fail("tile.alg = 4 needs mf = 16 and one block per workgroup");
+        if (t.ks != 1 || t.wl != 0) return fail("tile.alg = 4 has no split across workgroups and no loader waves");
+        if (tail_N > 0) return fail("tile.alg = 4 cannot carry a fused tail");
+        const int groups = (t.cch % (4 * t.wk) == 0) ? t.cch / (4 * t.wk) : 0;
+        if (groups != 1 && groups != 2 && groups != 4) return fail("tile.alg = 4 needs cch = 4 * wk * {1, 2, 4}");
+        if (t.cch < d.C) return fail("tile.alg = 4 takes all input channels in one pass");
+        if ((long long)t.cch * d.H * d.W * 4 >= (1LL << 31)) return fail("image too large for tile.alg = 4");
+    }
     g.wino = t.alg == 1;
     if (t.alg == 3) {
         // 1x1 convolution streamed from global memory: a 16x16 output block per workgroup, the input channels split
@@ -189,7 +201,7 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
     if (g.grid_y > 65535) return fail("grid too large");
     const int granule = g.kc * t.wk;
     if (t.cch < granule || t.cch % granule != 0) return fail("tile.cch must be a positive multiple of kc*wk");
-    if (t.alg != 3 && t.cch > round_up(d.C, granule)) return fail("tile.cch exceeds the (padded) channel count");
+    if (t.alg < 3 && t.cch > round_up(d.C, granule)) return fail("tile.cch exceeds the (padded) channel count");
     g.cpw = t.cch / t.wk;
     g.nchunks = ceil_div(d.C, t.cch);
     g.c_pad = g.nchunks * t.cch;
@@ -221,7 +233,7 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
     g.aff_floats = (d.KH == 1 && d.KW == 1 && d.pad == 0) ? round_up(2 * t.cch, 256) : 0;
     // (the Winograd path reads its weights straight from global memory into registers: the LDS holds input only)
     g.stage_floats = g.in_stage_floats + (t.alg ? 0 : round_up(g.wslab_floats, 256)) + g.aff_floats;   // (wino = 2 likewise)
-    if (t.alg == 3) g.in_stage_floats = g.aff_floats = g.stage_floats = 0;   // nothing is staged
+    if (t.alg >= 3) g.in_stage_floats = g.aff_floats = g.stage_floats = 0;   // nothing is staged
     g.nstage = g.cps > 1 ? 2 : 1;
     const long long stage_bytes = (long long)g.nstage * g.stage_floats * 4;
     // (the Winograd path always parks its output tiles in LDS, also without a split over waves)
@@ -268,7 +280,7 @@ void pack_weights(const tdc_conv_desc &d, const tdc_tile &t, const Geometry &g, 
     const int ncg = t.cch / g.kc;
     const int taps = g.taps;
     float *dst = packed;
-    if (t.alg == 2) {
+    if (t.alg == 2 || t.alg == 4) {
         // per (channel tile, pass, M block, channel group): [taps 0-3][lane][4] [taps 4-7][lane][4] [tap 8][lane]
         for (int by = 0; by < g.grid_y; ++by)
             for (int chunk = 0; chunk < g.nchunks; ++chunk)
@@ -398,6 +410,7 @@ int kernel_vgprs(const tdc_tile &t, int taps_mode) {
     if (t.alg == 1) regs = 136;   // 64 accumulators, two sets of 16 B and 16 A operands, the raw patch
     if (t.alg == 2) regs = 104;   // two sets of 18 A and 18 B operands
     if (t.alg == 3) regs = 40 + 16 * (t.cch / (16 * t.wk));   // per run of 16 channels: 4 A, 4 B, 8 scale/shift
+    if (t.alg == 4) regs = 40 + 18 * (t.cch / (4 * t.wk));    // per group of 4 channels: 9 A, 9 B
     return round_up(regs, 8);
 }
 
@@ -425,7 +438,7 @@ bool model_evaluate(const tdc_conv_desc &d, const tdc_tile &t, tdc_tile_info &in
     const int wg_by_vgpr = waves_simd_vgpr / wg_waves_per_simd;
     const int wg_by_lds = m.lds_bytes_per_cu / std::max(g.lds_bytes, 1);
     // (the staged kernels are never resident more than eight times per CU; the streamed one has no stage to hold)
-    int wg_per_cu = std::min(std::min(wg_by_vgpr, wg_by_lds), t.alg == 3 ? 32 : 8);
+    int wg_per_cu = std::min(std::min(wg_by_vgpr, wg_by_lds), t.alg >= 3 ? 32 : 8);
     if (wg_per_cu < 1) {
         if (why) *why = "tile does not fit one compute unit";
         return false;
@@ -468,6 +481,22 @@ bool model_evaluate(const tdc_conv_desc &d, const tdc_tile &t, tdc_tile_info &in
     const int comp_waves_per_simd = ceil_div(ncomp, m.simds_per_cu);
 
     auto wg_time = [&](int r, long long concurrent_wgs) {
+        if (t.alg == 4) {
+            // as below; per input channel 576 bytes of weights and nine 64-byte rows of input (the rows of
+            // neighbouring taps mostly hit in the L1, so they count for less than their size)
+            const double chip_share =
+                MC.l2_bytes_per_clk / std::max<double>(1.0, (double)std::min<long long>(concurrent_wgs, m.cus));
+            // (fitted to 364 timed tiles of 35 shapes, 7 % mean error: the nine taps of a lane are separate requests and
+            //  the achieved fill rate is lower than that of the 1x1 path; the MFMAs all but vanish under the arrivals)
+            const double rate = std::min(0.62 * MC.copy_bytes_per_clk, chip_share);
+            const double bytes = (double)t.cch * (576.0 + 0.87 * 576.0) * r;
+            const double groups = (double)t.cch / (4.0 * t.wk);
+            const double waves_simd = std::ceil((double)g.waves * r / m.simds_per_cu);
+            double clk = MC.stream_setup_clk + MC.stream_latency_clk + 1455.0 + bytes / rate + groups * 9.0 * 5.0 * waves_simd;
+            if (t.wk > 1) clk += MC.sync_clk;
+            clk += out_bytes * r / 200.0;
+            return clk;
+        }
         if (t.alg == 3) {
             // every wave requests its whole share up front and works through it as it arrives: one round trip, the
             // bytes at the CU's (or the chip's) fill rate, two chains of dependent MFMAs, the reduction over the waves
@@ -561,6 +590,28 @@ std::vector<tdc_tile> model_enumerate(const tdc_conv_desc &d, int tail_N) {
             tdc_tile t{16, 1, 1, 1, 1, wk, 16 * per_wave * wk, std::min(16, Wo), 1, 0, 3};
             Geometry g;
             if (make_geometry(d, t, g, nullptr, 0)) out.push_back(t);
+        }
+    }
+    // streamed 3x3 candidates: 1, 2 or 4 groups of four channels per wave, a few shapes of the 16-pixel tile
+    if (d.KH == 3 && d.KW == 3 && d.dilation == 1 && tail_N == 0 && !std::getenv("TDC_EXPERIMENT_NO_STREAMED_3X3")) {
+        const int groups = ceil_div(d.C, 4);
+        std::vector<int> tws;
+        for (int tw : {16, 14, 8, 7, 4, std::min(16, Wo)}) {
+            if (tw > std::min(16, Wo) || std::find(tws.begin(), tws.end(), tw) != tws.end()) continue;
+            const int th = std::min(16 / tw, Ho);
+            const double util = (double)P / ((double)ceil_div(Wo, tw) * ceil_div(Ho, th) * 16);
+            if (util < 0.6 && tw != std::min(16, Wo)) continue;
+            tws.push_back(tw);
+        }
+        for (int per_wave : {4, 2, 1}) {
+            if (per_wave > groups) continue;
+            const int wk = ceil_div(groups, per_wave);
+            if (wk > 16) continue;
+            for (int tw : tws) {
+                tdc_tile t{16, 1, 1, 1, 1, wk, 4 * per_wave * wk, tw, 1, 0, 4};
+                Geometry g;
+                if (make_geometry(d, t, g, nullptr, 0)) out.push_back(t);
+            }
         }
     }
     // Winograd candidates for 3x3 / stride 1 convolutions with enough pixels to fill tile lanes

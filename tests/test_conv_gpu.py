@@ -149,6 +149,41 @@ def test_every_streamed_1x1_tile(shape):
         assert_close(out.cpu().numpy(), want_aff, f"input affine {shape} {t}")
 
 
+@pytest.mark.parametrize("shape,stride,pad", [((1, 16, 16, 7, 7), 1, 1), ((2, 13, 20, 9, 11), 1, 1), ((1, 40, 24, 13, 13), 2, 1),
+                                              ((1, 16, 16, 12, 12), 1, 2), ((1, 128, 48, 7, 7), 1, 1), ((1, 64, 32, 28, 28), 1, 1),
+                                              ((3, 5, 3, 4, 3), 1, 0), ((1, 250, 17, 5, 5), 2, 1)])
+def test_every_streamed_3x3_tile(shape, stride, pad):
+    """The 3x3 path that streams both operands from global memory into registers (tile.alg = 4): every launchable tile
+    (1, 2 or 4 channel groups per wave, 1 to 16 waves, every shape of the 16-pixel tile), stride 2, wide and no padding,
+    ragged channel counts, batches; plain, and with bias + residual + ReLU written into a channel slice."""
+    from ctypes import c_void_p
+    B, C, N, H, W = shape
+    x, w = case(2500 + C * N + H, B, C, N, H, W, 3)
+    g = seeded(2501)
+    bias = torch.randn(N, generator=g)
+    want = ref.conv2d_c(x.numpy(), w.numpy(), stride=stride, pad=pad)
+    Ho, Wo = want.shape[2], want.shape[3]
+    resid = torch.randn(B, N, Ho, Wo, generator=g)
+    want_full = (torch.from_numpy(want) + bias.view(1, -1, 1, 1) + resid).clamp_min(0).numpy()
+    tiles = [t for t in tdc_amd.model_enumerate(tdc_amd.conv_desc(B, C, N, H, W, 3, 3, stride, pad)) if t.alg == 4]
+    assert tiles
+    for t in tiles:
+        announce("streamed 3x3", shape, stride, pad, t)
+        assert_close(run_conv(x, w, stride=stride, pad=pad, tile=t), want, f"{shape} s{stride} p{pad} {t}")
+        plan = tdc_amd.Conv2dPlan(B, C, N, H, W, 3, 3, stride, pad, 1, True, True, tile=t).set_weights(w, bias)
+        xin = torch.zeros(B, C + 3, H, W, device="cuda"); xin[:, 1:1 + C] = x.cuda()
+        rbuf = torch.zeros(B, N + 2, Ho, Wo, device="cuda"); rbuf[:, 2:] = resid.cuda()
+        obuf = torch.full((B, N + 5, Ho, Wo), 7.0, device="cuda")
+        tdc_amd._lib.check(tdc_amd.lib().tdc_conv_forward_strided(
+            plan._h, c_void_p(xin[:, 1:].data_ptr()), (C + 3) * H * W, c_void_p(rbuf[:, 2:].data_ptr()), (N + 2) * Ho * Wo,
+            c_void_p(obuf[:, 4:].data_ptr()), (N + 5) * Ho * Wo, c_void_p(torch.cuda.current_stream().cuda_stream)))
+        torch.cuda.synchronize()
+        plan.close()
+        got = obuf.cpu()
+        assert_close(got[:, 4:4 + N].numpy(), want_full, f"slices {shape} {t}")
+        assert (got[:, :4] == 7.0).all() and (got[:, 4 + N:] == 7.0).all()
+
+
 @pytest.mark.parametrize("W,c0", [(16, 0), (16, 3), (14, 3), (13, 1)])
 def test_winograd_into_channel_slices(W, c0):
     """A Winograd tile reading from, adding a residual from, and writing into channel slices of wider buffers (the

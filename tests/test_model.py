@@ -30,8 +30,44 @@ def test_every_candidate_is_launchable_and_covers_the_output(hw, r1, r2):
         assert i.grid_y * t.mf * t.mb * t.wm >= r2                                   # ... and all channels
         assert i.nchunks * t.cch >= r1 and t.cch % ((2 if t.mf == 32 else 4) * t.wk) == 0
         assert i.block_threads == 64 * (t.wm * t.wn * t.wk + t.wl) <= 1024      # computing waves + loader waves
-        assert 0 < i.lds_bytes <= LDS_BYTES
+        # (the streamed paths stage nothing: their LDS only holds the partial sums of a split over waves)
+        assert (0 if t.alg >= 3 else 1) <= i.lds_bytes <= LDS_BYTES
         assert i.wg_per_cu >= 1 and i.pred_us > 0
+
+
+def test_streamed_tiles_only_where_they_apply():
+    """tile.alg = 3 (1x1) and 4 (3x3) read both operands from global memory: one 16x16 block per workgroup, every
+    input channel in one pass, 1/2/4/8 runs of 16 channels (alg 3) or 1/2/4 groups of 4 channels (alg 4) per wave."""
+    d1 = tdc_amd.conv_desc(1, 256, 64, 14, 14, 1, 1, 1, 0)
+    ok = tdc_amd.model_evaluate(d1, tdc_amd.Tile(16, 1, 1, 1, 1, 4, 256, 16, 1, 0, 3))
+    assert (ok.grid_x, ok.grid_y, ok.block_threads, ok.lds_bytes, ok.nchunks) == (13, 4, 256, 4096, 1)
+    for d, t in [(d1, tdc_amd.Tile(16, 1, 1, 1, 1, 1, 256, 16, 1, 0, 3)),      # 16 runs per wave
+                 (d1, tdc_amd.Tile(16, 1, 1, 1, 1, 4, 128, 16, 1, 0, 3)),      # not all channels in one pass
+                 (d1, tdc_amd.Tile(16, 1, 1, 1, 1, 4, 256, 16, 2, 0, 3)),      # split across workgroups
+                 (d1, tdc_amd.Tile(16, 1, 1, 1, 2, 4, 256, 16, 1, 0, 3)),      # more than one block
+                 (d1, tdc_amd.Tile(32, 1, 1, 1, 1, 4, 256, 16, 1, 0, 3)),
+                 (d1, tdc_amd.Tile(16, 1, 1, 1, 1, 4, 256, 8, 1, 0, 3)),       # tw must be 16 (or all pixels)
+                 (tdc_amd.conv_desc(1, 2048, 64, 7, 7, 1, 1, 1, 0), tdc_amd.Tile(16, 1, 1, 1, 1, 16, 2048, 16, 1, 0, 3)),  # 8 runs x 16 waves
+                 (tdc_amd.conv_desc(1, 256, 64, 14, 14, 1, 1, 2, 0), tdc_amd.Tile(16, 1, 1, 1, 1, 4, 256, 16, 1, 0, 3)),   # stride 2
+                 (conv3(64, 64, 14), tdc_amd.Tile(16, 1, 1, 1, 1, 4, 64, 14, 1, 0, 3))]:
+        with pytest.raises(tdc_amd.TdcError):
+            tdc_amd.model_evaluate(d, t)
+    d3 = conv3(64, 64, 14)
+    ok = tdc_amd.model_evaluate(d3, tdc_amd.Tile(16, 1, 1, 1, 1, 4, 64, 14, 1, 0, 4))
+    assert (ok.grid_x, ok.grid_y, ok.th, ok.block_threads) == (14, 4, 1, 256)
+    assert tdc_amd.model_evaluate(conv3(64, 64, 14, stride=2), tdc_amd.Tile(16, 1, 1, 1, 1, 4, 64, 7, 1, 0, 4)).th == 2
+    for d, t in [(d3, tdc_amd.Tile(16, 1, 1, 1, 1, 2, 64, 14, 1, 0, 4)),       # 8 groups per wave
+                 (d3, tdc_amd.Tile(16, 1, 1, 1, 1, 4, 32, 14, 1, 0, 4)),       # not all channels in one pass
+                 (d3, tdc_amd.Tile(16, 1, 1, 1, 1, 4, 64, 14, 1, 2, 4)),       # loader waves
+                 (d3, tdc_amd.Tile(16, 1, 1, 2, 1, 4, 64, 14, 1, 0, 4)),
+                 (tdc_amd.conv_desc(1, 64, 64, 14, 14, 3, 3, 1, 2, 2), tdc_amd.Tile(16, 1, 1, 1, 1, 4, 64, 14, 1, 0, 4)),  # dilation 2
+                 (d1, tdc_amd.Tile(16, 1, 1, 1, 1, 4, 256, 16, 1, 0, 4))]:
+        with pytest.raises(tdc_amd.TdcError):
+            tdc_amd.model_evaluate(d, t)
+    # the enumeration offers them for every 1x1 / 3x3 shape they fit, and only there
+    assert any(t.alg == 3 for t in tdc_amd.model_enumerate(d1)) and not any(t.alg == 4 for t in tdc_amd.model_enumerate(d1))
+    assert any(t.alg == 4 for t in tdc_amd.model_enumerate(d3)) and not any(t.alg == 3 for t in tdc_amd.model_enumerate(d3))
+    assert not any(t.alg >= 3 for t in tdc_amd.model_enumerate(tdc_amd.conv_desc(1, 3, 64, 32, 32, 7, 7, 2, 3)))
 
 
 def test_winograd_tiles_only_where_the_algorithm_applies():
