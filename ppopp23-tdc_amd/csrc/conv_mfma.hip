@@ -1229,25 +1229,8 @@ __global__ void __launch_bounds__(1024) tdc_conv3x3_stream_kernel(const ConvKPar
     const __amdgpu_buffer_rsrc_t w_rsrc =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.wpk), (short)0, (int)p.wpk_bytes, 0x00020000);
 
-    const int k = lane >> 4, n = lane & 15;
-    const int jy = fdiv(n, p.fd_tw);
-    const int jx = n - jy * p.TW;
-    const int oy = tile_y * p.TH + jy, ox = tile_x * p.TW + jx;
-    const bool live = jy < p.TH && oy < p.Ho && ox < p.Wo;
-    // byte offset of every tap inside one channel, or the out-of-range offset
-    unsigned toff[9];
-#pragma unroll
-    for (int r = 0; r < 3; ++r)
-#pragma unroll
-        for (int c = 0; c < 3; ++c) {
-            const int iy = oy * p.stride - p.pad + r, ix = ox * p.stride - p.pad + c;
-            const bool ok = live && iy >= 0 && iy < p.H && ix >= 0 && ix < p.W;
-            toff[r * 3 + c] = ok ? (unsigned)(iy * p.W + ix) * 4u : (unsigned)OOB_OFFSET;
-        }
-    const unsigned chan_bytes = (unsigned)(p.H * p.W) * 4u;
-    const unsigned base = (unsigned)(wave * (4 * CG) + k) * chan_bytes;   // this lane's first channel
+    // The weights depend on nothing but the channel block and the wave: request them before any pixel arithmetic.
     const int a_soff = (by * (p.CCH >> 2) + wave * CG) * 2304;            // nine taps x 64 lanes x 4 bytes per group
-
     f4_t a0[CG], a1[CG];
     float a8[CG], b[CG][9];
 #pragma unroll
@@ -1255,6 +1238,36 @@ __global__ void __launch_bounds__(1024) tdc_conv3x3_stream_kernel(const ConvKPar
         a0[g] = __builtin_bit_cast(f4_t, __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, lane * 16, a_soff + g * 2304, 0));
         a1[g] = __builtin_bit_cast(f4_t, __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, lane * 16, a_soff + g * 2304 + 1024, 0));
         a8[g] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(w_rsrc, lane * 4, a_soff + g * 2304 + 2048, 0));
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    const int k = lane >> 4, n = lane & 15;
+    const int jy = fdiv(n, p.fd_tw);
+    const int jx = n - jy * p.TW;
+    const int oy = tile_y * p.TH + jy, ox = tile_x * p.TW + jx;
+    const bool live = jy < p.TH && oy < p.Ho && ox < p.Wo;
+    // byte offset of every tap inside one channel, or the out-of-range offset (branch-free: row and column tests apart)
+    const int iy0 = oy * p.stride - p.pad, ix0 = ox * p.stride - p.pad;
+    const unsigned off0 = (unsigned)(iy0 * p.W + ix0) * 4u;
+    const unsigned rowb = (unsigned)p.W * 4u;
+    unsigned rmask[3], cmask[3];
+#pragma unroll
+    for (int r = 0; r < 3; ++r) {
+        rmask[r] = ((unsigned)(iy0 + r) < (unsigned)p.H && live) ? 0xffffffffu : 0u;
+        cmask[r] = ((unsigned)(ix0 + r) < (unsigned)p.W) ? 0xffffffffu : 0u;
+    }
+    unsigned toff[9];
+#pragma unroll
+    for (int r = 0; r < 3; ++r)
+#pragma unroll
+        for (int c = 0; c < 3; ++c) {
+            const unsigned m = rmask[r] & cmask[c];
+            toff[r * 3 + c] = ((off0 + (unsigned)r * rowb + (unsigned)c * 4u) & m) | ((unsigned)OOB_OFFSET & ~m);
+        }
+    const unsigned chan_bytes = (unsigned)(p.H * p.W) * 4u;
+    const unsigned base = (unsigned)(wave * (4 * CG) + k) * chan_bytes;   // this lane's first channel
+#pragma unroll
+    for (int g = 0; g < CG; ++g) {
 #pragma unroll
         for (int t = 0; t < 9; ++t)   // (the whole offset goes through the range-checked vector operand)
             b[g][t] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
