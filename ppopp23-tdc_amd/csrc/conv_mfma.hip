@@ -1194,7 +1194,10 @@ static int taps_mode(int KH, int KW, int dil) {
 // tile.alg = 2: two 128-bit loads and one 32-bit load); padding, channels past C and lanes past the tile present an
 // out-of-range offset and read zero without a memory access.
 // ---------------------------------------------------------------------------
-template <int CG>
+// ROW (stride 1 and a tile of one row of 14 pixels): the 16 lanes of a quarter load the 16 consecutive input pixels
+// that the row of outputs touches, once per filter row, and the three taps of a row are lane shifts of that value
+// (three requests per group of channels instead of nine).
+template <int CG, bool ROW>
 __global__ void __launch_bounds__(1024) tdc_conv3x3_stream_kernel(const ConvKParams p) {
     extern __shared__ __align__(16) float lds[];
     if constexpr (TDC_TOUCH_KERNARGS) {
@@ -1246,33 +1249,65 @@ __global__ void __launch_bounds__(1024) tdc_conv3x3_stream_kernel(const ConvKPar
     const int jx = n - jy * p.TW;
     const int oy = tile_y * p.TH + jy, ox = tile_x * p.TW + jx;
     const bool live = jy < p.TH && oy < p.Ho && ox < p.Wo;
-    // byte offset of every tap inside one channel, or the out-of-range offset (branch-free: row and column tests apart)
     const int iy0 = oy * p.stride - p.pad, ix0 = ox * p.stride - p.pad;
-    const unsigned off0 = (unsigned)(iy0 * p.W + ix0) * 4u;
     const unsigned rowb = (unsigned)p.W * 4u;
-    unsigned rmask[3], cmask[3];
-#pragma unroll
-    for (int r = 0; r < 3; ++r) {
-        rmask[r] = ((unsigned)(iy0 + r) < (unsigned)p.H && live) ? 0xffffffffu : 0u;
-        cmask[r] = ((unsigned)(ix0 + r) < (unsigned)p.W) ? 0xffffffffu : 0u;
-    }
-    unsigned toff[9];
-#pragma unroll
-    for (int r = 0; r < 3; ++r)
-#pragma unroll
-        for (int c = 0; c < 3; ++c) {
-            const unsigned m = rmask[r] & cmask[c];
-            toff[r * 3 + c] = ((off0 + (unsigned)r * rowb + (unsigned)c * 4u) & m) | ((unsigned)OOB_OFFSET & ~m);
-        }
     const unsigned chan_bytes = (unsigned)(p.H * p.W) * 4u;
     const unsigned base = (unsigned)(wave * (4 * CG) + k) * chan_bytes;   // this lane's first channel
+    if constexpr (ROW) {
+        // lane n of a quarter: input column (tile's first column - pad + n) of the three input rows
+        const int iyr = tile_y - p.pad, ixr = tile_x * 14 - p.pad + n;
+        unsigned roff[3];
 #pragma unroll
-    for (int g = 0; g < CG; ++g) {
+        for (int r = 0; r < 3; ++r) {
+            const bool ok = (unsigned)(iyr + r) < (unsigned)p.H && (unsigned)ixr < (unsigned)p.W;
+            const unsigned m = ok ? 0xffffffffu : 0u;
+            roff[r] = ((unsigned)((iyr + r) * p.W + ixr) * 4u & m) | ((unsigned)OOB_OFFSET & ~m);
+        }
+        float rowv[CG][3];
 #pragma unroll
-        for (int t = 0; t < 9; ++t)   // (the whole offset goes through the range-checked vector operand)
-            b[g][t] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
-                in_rsrc, (int)(toff[t] + base + (unsigned)(4 * g) * chan_bytes), 0, 0));
-        __builtin_amdgcn_sched_barrier(0);   // requests in the order the MFMAs consume them
+        for (int g = 0; g < CG; ++g) {
+#pragma unroll
+            for (int r = 0; r < 3; ++r)
+                rowv[g][r] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                    in_rsrc, (int)(roff[r] + base + (unsigned)(4 * g) * chan_bytes), 0, 0));
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int g = 0; g < CG; ++g)
+#pragma unroll
+            for (int r = 0; r < 3; ++r) {
+                const int v = __builtin_bit_cast(int, rowv[g][r]);
+                b[g][r * 3 + 0] = rowv[g][r];
+                // row_shl:1 / row_shl:2 within the 16 lanes of a quarter: lane n takes the value of lane n+1 / n+2
+                b[g][r * 3 + 1] = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, v, 0x101, 0xf, 0xf, true));
+                b[g][r * 3 + 2] = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, v, 0x102, 0xf, 0xf, true));
+            }
+    } else {
+        // byte offset of every tap inside one channel, or the out-of-range offset (branch-free: row and column tests apart)
+        const unsigned off0 = (unsigned)(iy0 * p.W + ix0) * 4u;
+        unsigned rmask[3], cmask[3];
+#pragma unroll
+        for (int r = 0; r < 3; ++r) {
+            rmask[r] = ((unsigned)(iy0 + r) < (unsigned)p.H && live) ? 0xffffffffu : 0u;
+            cmask[r] = ((unsigned)(ix0 + r) < (unsigned)p.W) ? 0xffffffffu : 0u;
+        }
+        unsigned toff[9];
+#pragma unroll
+        for (int r = 0; r < 3; ++r)
+#pragma unroll
+            for (int c = 0; c < 3; ++c) {
+                const unsigned m = rmask[r] & cmask[c];
+                toff[r * 3 + c] = ((off0 + (unsigned)r * rowb + (unsigned)c * 4u) & m) | ((unsigned)OOB_OFFSET & ~m);
+            }
+#pragma unroll
+        for (int g = 0; g < CG; ++g) {
+#pragma unroll
+            for (int t = 0; t < 9; ++t)   // (the whole offset goes through the range-checked vector operand)
+                b[g][t] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                    in_rsrc, (int)(toff[t] + base + (unsigned)(4 * g) * chan_bytes), 0, 0));
+            __builtin_amdgcn_sched_barrier(0);   // requests in the order the MFMAs consume them
+        }
     }
     __builtin_amdgcn_sched_barrier(0);
     f4_t acc0 = (f4_t){0.0f, 0.0f, 0.0f, 0.0f}, acc1 = (f4_t){0.0f, 0.0f, 0.0f, 0.0f};
@@ -1323,15 +1358,17 @@ static kernel_fn pick_stream(int nq) {
     }
 }
 
-const void *conv_kernel_for(const tdc_tile &t, int KH, int KW, int dilation, bool extras) {
+const void *conv_kernel_for(const tdc_tile &t, int KH, int KW, int dilation, int stride, bool extras) {
     kernel_fn fn = nullptr;
     if (t.alg == 4) {
         if (extras || KH != 3 || KW != 3 || dilation != 1 || t.mf != 16 || t.mb != 1 || t.nb != 1 || t.wm != 1 || t.wn != 1 || t.wk < 1 || t.wk > 16)
             return nullptr;
-        switch (t.cch % (4 * t.wk) == 0 ? t.cch / (4 * t.wk) : 0) {
-            case 1: return reinterpret_cast<const void *>(static_cast<kernel_fn>(tdc_conv3x3_stream_kernel<1>));
-            case 2: return reinterpret_cast<const void *>(static_cast<kernel_fn>(tdc_conv3x3_stream_kernel<2>));
-            case 4: return reinterpret_cast<const void *>(static_cast<kernel_fn>(tdc_conv3x3_stream_kernel<4>));
+        const int groups = t.cch % (4 * t.wk) == 0 ? t.cch / (4 * t.wk) : 0;
+        const bool row = stride == 1 && t.tw == 14;
+        switch (groups) {
+            case 1: return reinterpret_cast<const void *>(row ? static_cast<kernel_fn>(tdc_conv3x3_stream_kernel<1, true>) : static_cast<kernel_fn>(tdc_conv3x3_stream_kernel<1, false>));
+            case 2: return reinterpret_cast<const void *>(row ? static_cast<kernel_fn>(tdc_conv3x3_stream_kernel<2, true>) : static_cast<kernel_fn>(tdc_conv3x3_stream_kernel<2, false>));
+            case 4: return reinterpret_cast<const void *>(row ? static_cast<kernel_fn>(tdc_conv3x3_stream_kernel<4, true>) : static_cast<kernel_fn>(tdc_conv3x3_stream_kernel<4, false>));
             default: return nullptr;
         }
     }

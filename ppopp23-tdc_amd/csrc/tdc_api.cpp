@@ -312,7 +312,7 @@ int tdc_conv_plan_create_with_tail(const tdc_conv_desc *desc, int32_t tail_N, in
     }
     p->tile = p->info.tile;
     if (!make_geometry(*desc, p->tile, p->geo, &why, tail_N)) return fail(TDC_ERR_INVALID, why);
-    p->kernel = conv_kernel_for(p->tile, desc->KH, desc->KW, desc->dilation, tail_N > 0);
+    p->kernel = conv_kernel_for(p->tile, desc->KH, desc->KW, desc->dilation, desc->stride, tail_N > 0);
     if (!p->kernel) return fail(TDC_ERR_UNSUPPORTED, "no kernel instantiated for this tile");
     int he = prepare_conv_kernel(p->kernel, p->geo);
     if (he) return hip_fail("hipFuncSetAttribute(MaxDynamicSharedMemorySize)", he);
@@ -411,7 +411,7 @@ int tdc_conv_plan_set_input_affine(tdc_conv_plan *plan, const float *scale, cons
     if (e == hipSuccess) e = hipMemcpy(plan->d_in_aff, packed.data(), n * sizeof(float), hipMemcpyHostToDevice);
     if (e != hipSuccess) return hip_fail("input affine upload", e);
     // from now on this plan needs the kernel instantiation that carries the extras
-    plan->kernel = conv_kernel_for(plan->tile, d.KH, d.KW, d.dilation, true);
+    plan->kernel = conv_kernel_for(plan->tile, d.KH, d.KW, d.dilation, d.stride, true);
     if (!plan->kernel) return fail(TDC_ERR_UNSUPPORTED, "no kernel instantiated for this tile");
     if (int he = prepare_conv_kernel(plan->kernel, plan->geo)) return hip_fail("hipFuncSetAttribute(MaxDynamicSharedMemorySize)", he);
     plan->in_relu = relu != 0;

@@ -144,7 +144,7 @@ struct ConvKParams {
 
 // The instantiated kernel for a tile and filter size (nullptr if none).
 // `extras`: the instantiation that also carries the input affine and the fused 1x1 tail.
-const void *conv_kernel_for(const tdc_tile &t, int KH, int KW, int dilation, bool extras);
+const void *conv_kernel_for(const tdc_tile &t, int KH, int KW, int dilation, int stride, bool extras);
 // One-time per-plan attribute setup (dynamic LDS above 64 KiB).  hipError_t as int.
 int prepare_conv_kernel(const void *fn, const Geometry &g);
 // Enqueue the kernel.  Returns a hipError_t as int.

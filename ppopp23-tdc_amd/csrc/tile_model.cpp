@@ -486,14 +486,18 @@ bool model_evaluate(const tdc_conv_desc &d, const tdc_tile &t, tdc_tile_info &in
             // neighbouring taps mostly hit in the L1, so they count for less than their size)
             const double chip_share =
                 MC.l2_bytes_per_clk / std::max<double>(1.0, (double)std::min<long long>(concurrent_wgs, m.cus));
-            // (fitted to 364 timed tiles of 35 shapes, 7 % mean error: the nine taps of a lane are separate requests and
-            //  the achieved fill rate is lower than that of the 1x1 path; the MFMAs all but vanish under the arrivals)
-            const double rate = std::min(0.62 * MC.copy_bytes_per_clk, chip_share);
-            const double bytes = (double)t.cch * (576.0 + 0.87 * 576.0) * r;
+            // (fitted to 364 timed tiles of 35 shapes, 7 % mean error: the achieved fill rate is lower than that of the
+            //  1x1 path; the nine taps of a lane are separate requests that mostly hit in the L1, three requests and lane
+            //  shifts where a tile is one row of 14 pixels)
+            const double rate = std::min(0.59 * MC.copy_bytes_per_clk, chip_share);
+            const bool row_mode = d.stride == 1 && t.tw == 14;
+            const double bytes = (double)t.cch * (576.0 + (row_mode ? 0.28 : 0.66) * 576.0) * r;
             const double groups = (double)t.cch / (4.0 * t.wk);
             const double waves_simd = std::ceil((double)g.waves * r / m.simds_per_cu);
-            double clk = MC.stream_setup_clk + MC.stream_latency_clk + 1455.0 + bytes / rate + groups * 9.0 * 5.0 * waves_simd;
-            if (t.wk > 1) clk += MC.sync_clk;
+            // a wave issues its requests one after the other (about 21 cycles each): fewer groups per wave start sooner
+            double clk = MC.stream_setup_clk + MC.stream_latency_clk + 288.0 + 65.0 * (waves_simd - 1.0) + bytes / rate +
+                         groups * (3.0 + (row_mode ? 3.0 : 9.0)) * 21.4;
+            if (t.wk > 1) clk += 1.6 * MC.sync_clk;
             clk += out_bytes * r / 200.0;
             return clk;
         }
