@@ -65,7 +65,8 @@ typedef struct tdc_conv_desc {
  * (mf*mb*wm) output channels of a th x tw tile of output pixels (th is derived:
  * as many rows as fit in the workgroup's mf*nb*wn pixel lanes); its wm*wn*wk
  * computing wavefronts split output channels, pixels and input channels; input channels
- * are staged through LDS `cch` at a time, double-buffered. */
+ * are staged through LDS `cch` at a time, double-buffered (alg 0-2), or requested from
+ * global memory into registers all at once (alg 3-4). */
 typedef struct tdc_tile {
     int32_t mf;   /* MFMA block edge: 32 (v_mfma_f32_32x32x2_f32) or 16 (16x16x4) */
     int32_t mb;   /* MFMA blocks per wave along output channels (1 or 2)        */
@@ -86,7 +87,17 @@ typedef struct tdc_tile {
                          tiles instead of 36; weights read from global memory into registers; mf = 16, mb = nb = 1.
                      2 = direct 3x3 / dilation 1 convolution with the weights read from global memory straight
                          into registers (the LDS holds input only, so a pass can take more input channels);
-                         mb = nb = 1, an even number of channel groups per wave and pass */
+                         mb = nb = 1, an even number of channel groups per wave and pass.
+                     3 = 1x1 / stride 1 / pad 0 convolution with BOTH operands read from global memory straight into
+                         registers: no LDS stage, one pass; a workgroup owns 16 channels x 16 pixels, its wk (<= 16)
+                         waves split the input channels in runs of 16; cch = 16 * wk * {1, 2, 4, 8} >= C
+                         (eight runs per wave: wk <= 8); mf = 16, mb = nb = wm = wn = ks = 1, wl = 0,
+                         tw = min(16, pixels).  Carries the input affine, not a fused tail.
+                     4 = the same for 3x3 / dilation 1 convolutions (any stride): 16 channels x a 16-pixel tile of
+                         width tw per workgroup, the input channels in groups of four; cch = 4 * wk * {1, 2, 4} >= C.
+                         With stride 1 and tw = 14 the three taps of a filter row are lane shifts of one request.
+                     The model offers 3 and 4 where launch and latency dominate (few channels or few pixels); the
+                     staged paths keep the layers whose operands are worth sharing through the LDS. */
 } tdc_tile;
 
 typedef struct tdc_tile_info {
