@@ -205,6 +205,11 @@ def model_set_constants(values):
     check(lib().tdc_model_set_constants(arr, len(values)))
 
 
+def get_autotune() -> int:
+    """The current setting of the measured tile selection (0 = off)."""
+    return int(lib().tdc_get_autotune())
+
+
 def set_autotune(classes: int):
     """Measured tile selection for every plan created from now on without a forced tile: time the model's
     favourite of each of the `classes` most promising tile classes on the device and keep the fastest

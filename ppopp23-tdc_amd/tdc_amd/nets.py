@@ -290,6 +290,46 @@ def densenet121_params(seed=121, num_classes=1000, growth=32, bn_size=4, ranks=(
     return p
 
 
+def _dense_layer(net, src, dst, fused, s1, t1, w1, t2, first, core, last):
+    if fused:
+        # norm1 + relu, conv1, norm2 + relu and the first Tucker factor in one kernel; core + last in another
+        y = net.conv_tail(src, w1, first, bias=t2, relu=True, in_affine=(s1, t1, True))
+        return net.conv_tail(y, core, last, pad=1, dst=dst)
+    # norm1 + relu on the concatenation, conv1, norm2 + relu: one kernel; then the Tucker convolution
+    y = net.affine_conv(src, s1, t1, w1, t2, relu=True)
+    return net.tkconv(y, first, core, last, pad=1, dst=dst)
+
+
+_DENSE_LAYER_FUSES = {}
+
+
+def _dense_layer_fuses(batch, c, h, w, d1, layer):
+    """Whether a dense layer runs faster with its bottleneck convolution and first Tucker factor fused into one kernel
+    (and core + last into another) or as bottleneck + Tucker convolution: the model's answer, checked, when the measured
+    tile selection is switched on, against a measurement (both variants of the layer are built as a network of their
+    own and timed; remembered per shape)."""
+    first = layer[4]
+    if _lib.model_select_with_tail(d1, first.shape[0]) is None:
+        return False
+    model_fuses = _lib.fused_tail_pays(d1, first.shape[0])
+    if _lib.get_autotune() <= 0:
+        return model_fuses
+    key = (batch, c, h, w, tuple(layer[2].shape), tuple(first.shape), tuple(layer[5].shape), tuple(layer[6].shape))
+    if key not in _DENSE_LAYER_FUSES:
+        x = torch.randn(batch, c, h, w, device="cuda")
+        t = []
+        for fused in (True, False):
+            m = Net(batch, c, h, w)
+            m.finalize(_dense_layer(m, 0, -1, fused, *layer))
+            m.forward(x)
+            m.time_ms(iters=10)
+            t.append(min(m.time_ms(iters=30) for _ in range(3)))
+            m.close()
+        # (a layer timed alone sees warmer caches than inside the network: the model's answer is only overruled by 5 %)
+        _DENSE_LAYER_FUSES[key] = (t[0] < 1.05 * t[1]) if model_fuses else (t[0] < 0.95 * t[1])
+    return _DENSE_LAYER_FUSES[key]
+
+
 def build_tucker_densenet121(params, batch=1, H=224, W=224, growth=32):
     """Finalized Net for the logits [batch, num_classes, 1, 1].  The concatenation of a dense block is one
     buffer; every layer's Tucker convolution writes its 32 new channels straight into its slice."""
@@ -311,14 +351,11 @@ def build_tucker_densenet121(params, batch=1, H=224, W=224, growth=32):
             first, core, last = (p[pre + ".conv2.first_kernel"], p[pre + ".conv2.core_kernel"],
                                  p[pre + ".conv2.last_kernel"])
             d1 = _lib.conv_desc(batch, c, w1.shape[0], h, w, 1, 1, 1, 0, 1, True, True)
-            if _lib.fused_tail_pays(d1, first.shape[0]):
-                # norm1 + relu, conv1, norm2 + relu and the first Tucker factor in one kernel; core + last in another
-                y = net.conv_tail(net.view(cat, 0, c), w1, first, bias=t2, relu=True, in_affine=(s1, t1, True))
-                net.conv_tail(y, core, last, pad=1, dst=net.view(cat, c, growth))
+            layer = (s1, t1, w1, t2, first, core, last)
+            if _dense_layer_fuses(batch, c, h, w, d1, layer):
+                _dense_layer(net, net.view(cat, 0, c), net.view(cat, c, growth), True, *layer)
             else:
-                # norm1 + relu on the concatenation, conv1, norm2 + relu: one kernel; then the Tucker convolution
-                y = net.affine_conv(net.view(cat, 0, c), s1, t1, w1, t2, relu=True)
-                net.tkconv(y, first, core, last, pad=1, dst=net.view(cat, c, growth))
+                _dense_layer(net, net.view(cat, 0, c), net.view(cat, c, growth), False, *layer)
             c += growth
         if b < len(DENSENET121_BLOCKS):
             pre = f"features.transition{b}"
