@@ -1232,8 +1232,12 @@ __global__ void __launch_bounds__(1024) tdc_conv3x3_stream_kernel(const ConvKPar
     const __amdgpu_buffer_rsrc_t w_rsrc =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.wpk), (short)0, (int)p.wpk_bytes, 0x00020000);
 
+    // wave = (channel block of the workgroup) * WK + (slice of the input channels)
+    const int wmi = fdiv(wave, p.fd_wk);
+    const int wki = wave - wmi * p.WK;
+    const int mblk = by * p.WM + wmi;   // this wave's block of 16 output channels
     // The weights depend on nothing but the channel block and the wave: request them before any pixel arithmetic.
-    const int a_soff = (by * (p.CCH >> 2) + wave * CG) * 2304;            // nine taps x 64 lanes x 4 bytes per group
+    const int a_soff = (mblk * (p.CCH >> 2) + wki * CG) * 2304;            // nine taps x 64 lanes x 4 bytes per group
     f4_t a0[CG], a1[CG];
     float a8[CG], b[CG][9];
 #pragma unroll
@@ -1252,7 +1256,7 @@ __global__ void __launch_bounds__(1024) tdc_conv3x3_stream_kernel(const ConvKPar
     const int iy0 = oy * p.stride - p.pad, ix0 = ox * p.stride - p.pad;
     const unsigned rowb = (unsigned)p.W * 4u;
     const unsigned chan_bytes = (unsigned)(p.H * p.W) * 4u;
-    const unsigned base = (unsigned)(wave * (4 * CG) + k) * chan_bytes;   // this lane's first channel
+    const unsigned base = (unsigned)(wki * (4 * CG) + k) * chan_bytes;   // this lane's first channel
     if constexpr (ROW) {
         // lane n of a quarter: input column (tile's first column - pad + n) of the three input rows
         const int iyr = tile_y - p.pad, ixr = tile_x * 14 - p.pad + n;
@@ -1322,21 +1326,77 @@ __global__ void __launch_bounds__(1024) tdc_conv3x3_stream_kernel(const ConvKPar
         __builtin_amdgcn_sched_barrier(0);   // group by group, as the data arrives
     }
     f4_t acc = acc0 + acc1;
+    // lane l holds rows 4*(l/16) .. +3 (output channels) of column l%16 (pixel); the slices of a channel block are
+    // added by its first wave, in slice order
     if (p.WK > 1) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) lds[(wave * 4 + i) * 64 + lane] = acc[i];
         __syncthreads();
-        if (wave != 0) return;
-        acc = (f4_t){0.0f, 0.0f, 0.0f, 0.0f};
-        for (int w = 0; w < p.WK; ++w)
+        if (wki == 0) {
+            acc = (f4_t){0.0f, 0.0f, 0.0f, 0.0f};
+            for (int w = 0; w < p.WK; ++w)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) acc[i] += lds[(w * 4 + i) * 64 + lane];
+                for (int i = 0; i < 4; ++i) acc[i] += lds[((wave + w) * 4 + i) * 64 + lane];
+        }
     }
-    if (!live) return;
     const int pp = oy * p.Wo + ox;
+    if (p.tail_w) {
+        // Fused 1x1 tail, out2 = W2 * act(conv + bias): the workgroup owns every output channel of the convolution
+        // (the host guarantees it).  The finished 16-pixel columns are parked in LDS as f[channel][pixel] — the B operand
+        // of a second small GEMM whose A operand, the tail's packed weights, comes from global memory — and its
+        // 16x16 output blocks are dealt to all waves.
+        float *f = lds + p.tail_f_off;
+        const int LD = p.tail_ld;
+        if (wki == 0) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int ml = wmi * 16 + 4 * k + i;
+                const int ch = by * 16 * p.WM + ml;
+                float val = acc[i];
+                if (p.bias && ch < p.N) val += p.bias[ch];
+                if (p.relu) val = fmaxf(val, 0.0f);
+                f[ml * LD + n] = val;
+            }
+        }
+        __syncthreads();
+        const int nwaves = p.WM * p.WK;
+        for (int blk = wave; blk < p.tail_mblk; blk += nwaves) {
+            const float *wa = p.tail_w + (size_t)blk * p.tail_ng * 64 + lane;
+            const float *fb = f + k * LD + n;
+            f4_t acc2 = {0.0f, 0.0f, 0.0f, 0.0f};
+            for (int g0 = 0; g0 < p.tail_ng; g0 += 4) {
+                float ta[4], tb[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const int g = min(g0 + u, p.tail_ng - 1);
+                    ta[u] = wa[g * 64];
+                    tb[u] = fb[g * 4 * LD];
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u)
+                    if (g0 + u < p.tail_ng) acc2 = __builtin_amdgcn_mfma_f32_16x16x4f32(ta[u], tb[u], acc2, 0, 0, 0);
+            }
+            if (live) {
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const int n2 = blk * 16 + 4 * k + v;
+                    if (n2 < p.tail_N) {
+                        float val = acc2[v];
+                        if (p.tail_bias) val += p.tail_bias[n2];
+                        const long long o = (long long)n2 * p.P + pp;
+                        if (resid) val += resid[o];
+                        if (p.tail_relu) val = fmaxf(val, 0.0f);
+                        out[o] = val;
+                    }
+                }
+            }
+        }
+        return;
+    }
+    if (wki != 0 || !live) return;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        const int ch = by * 16 + 4 * k + i;
+        const int ch = mblk * 16 + 4 * k + i;
         if (ch >= p.N) continue;
         float val = acc[i];
         if (p.bias) val += p.bias[ch];
@@ -1361,7 +1421,8 @@ static kernel_fn pick_stream(int nq) {
 const void *conv_kernel_for(const tdc_tile &t, int KH, int KW, int dilation, int stride, bool extras) {
     kernel_fn fn = nullptr;
     if (t.alg == 4) {
-        if (extras || KH != 3 || KW != 3 || dilation != 1 || t.mf != 16 || t.mb != 1 || t.nb != 1 || t.wm != 1 || t.wn != 1 || t.wk < 1 || t.wk > 16)
+        // (`extras` can only mean a fused tail here, which the one kernel carries)
+        if (KH != 3 || KW != 3 || dilation != 1 || t.mf != 16 || t.mb != 1 || t.nb != 1 || t.wm < 1 || t.wn != 1 || t.wk < 1 || t.wm * t.wk > 16)
             return nullptr;
         const int groups = t.cch % (4 * t.wk) == 0 ? t.cch / (4 * t.wk) : 0;
         const bool row = stride == 1 && t.tw == 14;

@@ -137,9 +137,9 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
         // 3x3 convolution streamed from global memory: 16 channels x 16 pixels per workgroup, the input channels
         // split over wk waves in groups of four, everything in one pass
         if (d.KH != 3 || d.KW != 3 || d.dilation != 1) return fail("tile.alg = 4 needs a 3x3 / dilation 1 convolution");
-        if (t.mf != 16 || t.mb != 1 || t.nb != 1 || t.wm != 1 || t.wn != 1) return fail("tile.alg = 4 needs mf = 16 and one block per workgroup");
+        if (t.mf != 16 || t.mb != 1 || t.nb != 1 || t.wn != 1) return fail("tile.alg = 4 needs mf = 16 and one pixel block per workgroup");
+        if (t.wm * t.wk > 16) return fail("tile.alg = 4: at most 16 waves (wm channel blocks x wk channel slices)");
         if (t.ks != 1 || t.wl != 0) return fail("tile.alg = 4 has no split across workgroups and no loader waves");
-        if (tail_N > 0) return fail("tile.alg = 4 cannot carry a fused tail");
         const int groups = (t.cch % (4 * t.wk) == 0) ? t.cch / (4 * t.wk) : 0;
         if (groups != 1 && groups != 2 && groups != 4) return fail("tile.alg = 4 needs cch = 4 * wk * {1, 2, 4}");
         if (t.cch < d.C) return fail("tile.alg = 4 takes all input channels in one pass");
@@ -491,13 +491,20 @@ bool model_evaluate(const tdc_conv_desc &d, const tdc_tile &t, tdc_tile_info &in
             //  shifts where a tile is one row of 14 pixels)
             const double rate = std::min(0.59 * MC.copy_bytes_per_clk, chip_share);
             const bool row_mode = d.stride == 1 && t.tw == 14;
-            const double bytes = (double)t.cch * (576.0 + (row_mode ? 0.28 : 0.66) * 576.0) * r;
+            const double bytes = (double)t.cch * t.wm * (576.0 + (row_mode ? 0.28 : 0.66) * 576.0) * r;
             const double groups = (double)t.cch / (4.0 * t.wk);
             const double waves_simd = std::ceil((double)g.waves * r / m.simds_per_cu);
             // a wave issues its requests one after the other (about 21 cycles each): fewer groups per wave start sooner
             double clk = MC.stream_setup_clk + MC.stream_latency_clk + 288.0 + 65.0 * (waves_simd - 1.0) + bytes / rate +
                          groups * (3.0 + (row_mode ? 3.0 : 9.0)) * 21.4;
             if (t.wk > 1) clk += 1.6 * MC.sync_clk;
+            if (tail_N > 0) {
+                // park the columns, a barrier, the first touch of the tail's weights, its blocks dealt over the waves
+                const double blocks = std::ceil((double)ceil_div(tail_N, 16) / g.waves);
+                clk += MC.sync_clk + MC.stream_latency_clk + blocks * (g.tail_ng * 40.0 + 64.0) +
+                       (double)tail_N * d.N * 4.0 * r / rate + (double)tail_N * 64.0 * r / 200.0;
+                return clk;
+            }
             clk += out_bytes * r / 200.0;
             return clk;
         }
@@ -597,7 +604,7 @@ std::vector<tdc_tile> model_enumerate(const tdc_conv_desc &d, int tail_N) {
         }
     }
     // streamed 3x3 candidates: 1, 2 or 4 groups of four channels per wave, a few shapes of the 16-pixel tile
-    if (d.KH == 3 && d.KW == 3 && d.dilation == 1 && tail_N == 0 && !std::getenv("TDC_EXPERIMENT_NO_STREAMED_3X3")) {
+    if (d.KH == 3 && d.KW == 3 && d.dilation == 1 && !std::getenv("TDC_EXPERIMENT_NO_STREAMED_3X3")) {
         const int groups = ceil_div(d.C, 4);
         std::vector<int> tws;
         for (int tw : {16, 14, 8, 7, 4, std::min(16, Wo)}) {
@@ -607,14 +614,16 @@ std::vector<tdc_tile> model_enumerate(const tdc_conv_desc &d, int tail_N) {
             if (util < 0.6 && tw != std::min(16, Wo)) continue;
             tws.push_back(tw);
         }
+        // (a fused tail needs every output channel in the workgroup: one wave per block of 16 and channel slice)
+        const int wm = tail_N > 0 ? ceil_div(d.N, 16) : 1;
         for (int per_wave : {4, 2, 1}) {
             if (per_wave > groups) continue;
             const int wk = ceil_div(groups, per_wave);
-            if (wk > 16) continue;
+            if (wm * wk > 16) continue;
             for (int tw : tws) {
-                tdc_tile t{16, 1, 1, 1, 1, wk, 4 * per_wave * wk, tw, 1, 0, 4};
+                tdc_tile t{16, 1, 1, wm, 1, wk, 4 * per_wave * wk, tw, 1, 0, 4};
                 Geometry g;
-                if (make_geometry(d, t, g, nullptr, 0)) out.push_back(t);
+                if (make_geometry(d, t, g, nullptr, tail_N)) out.push_back(t);
             }
         }
     }

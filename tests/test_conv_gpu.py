@@ -501,6 +501,42 @@ def test_fused_1x1_tail(shape):
     assert ran >= 10
 
 
+@pytest.mark.parametrize("shape", [(1, 24, 16, 40, 9, 9, 1), (2, 40, 10, 33, 14, 14, 1), (1, 32, 32, 64, 28, 28, 1), (1, 64, 64, 128, 13, 11, 2),
+                                   (1, 16, 128, 64, 7, 7, 1), (1, 13, 37, 5, 6, 5, 1)])
+def test_fused_tail_on_streamed_3x3(shape):
+    """The same fusion behind the streamed 3x3 kernel (tile.alg = 4 with one wave per block of 16 output channels and
+    channel slice): relu(W_tail * relu(conv(x) + b1) + b2 + residual), every admissible split of the waves and a few
+    tile widths, and whatever the model picks when a tail is asked for."""
+    B, C, N, N2, H, W, stride = shape
+    x, w = case(9700 + C + N, B, C, N, H, W, 3)
+    g = seeded(9701 + N2)
+    b1 = torch.randn(N, generator=g) * 0.5
+    w2 = torch.randn(N2, N, 1, 1, generator=g) / math.sqrt(N)
+    b2 = torch.randn(N2, generator=g)
+    want_mid = ref.conv2d_c(x.numpy(), w.numpy(), b1.numpy(), stride=stride, pad=1, relu=True)
+    resid = torch.randn(B, N2, want_mid.shape[2], want_mid.shape[3], generator=g)
+    want = ref.conv2d_c(want_mid, w2.numpy(), b2.numpy(), resid.numpy(), relu=True)
+    Wo = want.shape[3]
+    wm, groups = -(-N // 16), -(-C // 4)
+    tiles = []
+    for per_wave in (4, 2, 1):
+        wk = -(-groups // per_wave)
+        if per_wave <= groups and wm * wk <= 16:
+            for tw in sorted({min(16, Wo), min(14, Wo), min(7, Wo), min(4, Wo)}):
+                tiles.append(tdc_amd.Tile(16, 1, 1, wm, 1, wk, 4 * per_wave * wk, tw, 1, 0, 4))
+    assert tiles
+    xd, rd = x.cuda(), resid.cuda()
+    for t in tiles + [None]:
+        announce("streamed tail", shape, t)
+        plan = tdc_amd.Conv2dPlan(B, C, N, H, W, 3, 3, stride, 1, 1, True, True, tile=t, tail=(N2, True, True))
+        plan.set_weights(w, b1).set_tail_weights(w2, b2)
+        out = torch.full((B, N2, plan.Ho, plan.Wo), float("nan"), device="cuda")
+        plan.forward(xd, rd, out=out)
+        torch.cuda.synchronize()
+        plan.close()
+        assert_close(out.cpu().numpy(), want, f"streamed fused tail {shape} {t}")
+
+
 def test_fused_tail_needs_one_channel_tile():
     with pytest.raises(tdc_amd.TdcError):   # 40 output channels cannot sit in a 16-channel tile
         tdc_amd.Conv2dPlan(1, 8, 40, 9, 9, 3, 3, 1, 1, tile=tdc_amd.Tile(16, 1, 1, 1, 1, 1, 8, 8), tail=(8, False, False))
