@@ -56,10 +56,13 @@ def test_streamed_tiles_only_where_they_apply():
     ok = tdc_amd.model_evaluate(d3, tdc_amd.Tile(16, 1, 1, 1, 1, 4, 64, 14, 1, 0, 4))
     assert (ok.grid_x, ok.grid_y, ok.th, ok.block_threads) == (14, 4, 1, 256)
     assert tdc_amd.model_evaluate(conv3(64, 64, 14, stride=2), tdc_amd.Tile(16, 1, 1, 1, 1, 4, 64, 7, 1, 0, 4)).th == 2
+    wide = tdc_amd.model_evaluate(d3, tdc_amd.Tile(16, 1, 1, 2, 1, 4, 64, 14, 1, 0, 4))   # two blocks of 16 channels per workgroup
+    assert (wide.grid_x, wide.grid_y, wide.block_threads) == (14, 2, 512)
     for d, t in [(d3, tdc_amd.Tile(16, 1, 1, 1, 1, 2, 64, 14, 1, 0, 4)),       # 8 groups per wave
                  (d3, tdc_amd.Tile(16, 1, 1, 1, 1, 4, 32, 14, 1, 0, 4)),       # not all channels in one pass
                  (d3, tdc_amd.Tile(16, 1, 1, 1, 1, 4, 64, 14, 1, 2, 4)),       # loader waves
-                 (d3, tdc_amd.Tile(16, 1, 1, 2, 1, 4, 64, 14, 1, 0, 4)),
+                 (d3, tdc_amd.Tile(16, 1, 1, 8, 1, 4, 64, 14, 1, 0, 4)),       # 32 waves
+                 (d3, tdc_amd.Tile(16, 1, 2, 1, 1, 4, 64, 14, 1, 0, 4)),       # one pixel block per wave
                  (tdc_amd.conv_desc(1, 64, 64, 14, 14, 3, 3, 1, 2, 2), tdc_amd.Tile(16, 1, 1, 1, 1, 4, 64, 14, 1, 0, 4)),  # dilation 2
                  (d1, tdc_amd.Tile(16, 1, 1, 1, 1, 4, 256, 16, 1, 0, 4))]:
         with pytest.raises(tdc_amd.TdcError):
