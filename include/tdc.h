@@ -90,14 +90,15 @@ typedef struct tdc_tile {
                          mb = nb = 1, an even number of channel groups per wave and pass.
                      3 = 1x1 / stride 1 / pad 0 convolution with BOTH operands read from global memory straight into
                          registers: no LDS stage, one pass; a workgroup owns 16 channels x 16 pixels, its wk (<= 16)
-                         waves split the input channels in runs of 16; cch = 16 * wk * {1, 2, 4, 8} >= C
-                         (eight runs per wave: wk <= 8); mf = 16, mb = nb = wm = wn = ks = 1, wl = 0,
+                         waves split the input channels in runs of 16; cch = 16 * wk * {1, 2, 4, 8}
+                         (eight runs per wave: wk <= 8) with ks * cch >= C and ceil(C / cch) = ks: ks > 1 deals slices
+                         of cch channels to ks workgroups; mf = 16, mb = nb = wm = wn = 1, wl = 0,
                          tw = min(16, pixels).  Carries the input affine, not a fused tail.
                      4 = the same for 3x3 / dilation 1 convolutions (any stride): 16 * wm channels x a 16-pixel tile
                          of width tw per workgroup (one wave per block of 16 channels and channel slice, wm * wk <= 16),
-                         the input channels in groups of four; cch = 4 * wk * {1, 2, 4} >= C.  With stride 1 and
+                         the input channels in groups of four; cch = 4 * wk * {1, 2, 4}, ceil(C / cch) = ks.  With stride 1 and
                          tw = 14 the three taps of a filter row are lane shifts of one request.  Carries a fused 1x1
-                         tail when wm covers every output channel.
+                         tail when wm covers every output channel (and ks = 1).
                      The model offers 3 and 4 where launch and latency dominate (few channels or few pixels); the
                      staged paths keep the layers whose operands are worth sharing through the LDS. */
 } tdc_tile;

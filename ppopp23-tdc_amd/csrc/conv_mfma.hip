@@ -1045,6 +1045,64 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
 }
 
 // ---------------------------------------------------------------------------
+// Streamed kernels whose input channels are split over KS workgroups: the lanes that hold a finished partial block
+// (`holder`: four consecutive channels from `ch0` of pixel `pp`) leave it in the workspace ws[image][slice][N][P]; the
+// workgroup that draws the last ticket of its (image, channel tile, pixel tile) reads all KS partials back and adds
+// them in slice order, so the result does not depend on which workgroup that is.  Same protocol as the staged
+// kernel: every workspace access is a relaxed device-scope atomic (written through, read past the die-local L2).
+// Returns false in the workgroups that are done; every thread of the workgroup must call it.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ bool stream_join_slices(const ConvKParams &p, float *lds, f4_t &acc, bool holder, int ch0,
+                                                   int pp, int img, int slice, int by, int bx) {
+    const long long NP = (long long)p.N * p.P;
+    if (holder) {
+        float *wsz = p.ws + ((long long)img * p.KS + slice) * NP;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (ch0 + i < p.N)
+                __hip_atomic_store(wsz + (long long)(ch0 + i) * p.P + pp, acc[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    unsigned *ticket = p.ctr + ((unsigned)img * p.grid_y + by) * p.grid_x + bx;
+    if (threadIdx.x == 0) {
+        const unsigned d = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        reinterpret_cast<unsigned *>(lds)[0] = d;
+    }
+    __syncthreads();
+    const unsigned drawn = reinterpret_cast<const unsigned *>(lds)[0];
+    if (drawn != (unsigned)p.KS - 1u) return false;
+    if (threadIdx.x == 0) __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
+    if (holder) {
+        const float *ws0 = p.ws + (long long)img * p.KS * NP;
+        float part[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) part[i] = 0.0f;
+        // (these loads go past the L2 and take a microsecond: eight slices are requested at once, then added in order)
+        for (int s0 = 0; s0 < p.KS; s0 += 8) {
+            float v[8][4];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const float *src = ws0 + (long long)min(s0 + u, p.KS - 1) * NP + pp;
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    v[u][i] = __hip_atomic_load(src + (long long)min(ch0 + i, p.N - 1) * p.P, __ATOMIC_RELAXED,
+                                                __HIP_MEMORY_SCOPE_AGENT);
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (s0 + u < p.KS) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) part[i] += v[u][i];
+                }
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[i] = part[i];
+    }
+    return true;
+}
+
+// ---------------------------------------------------------------------------
 // 1x1 convolution with many input channels over few pixels (tile.alg = 3): no LDS stage, no passes, no barrier
 // before the reduction.  One workgroup owns a 16-channel x 16-pixel block of the output; its WK waves split the
 // input channels, NQ runs of 16 channels each.  A wave requests ALL its operands up front, straight into
@@ -1056,7 +1114,8 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
 // re-read its last pixel and are never stored.
 // ---------------------------------------------------------------------------
 // (eight runs per wave: 72 registers of operands, 136 with the affine; that variant is built for at most 8 waves)
-template <int NQ, bool AFF>
+// SPLIT: the instantiation whose input channels are dealt to p.KS workgroups (the plain one pays nothing for it).
+template <int NQ, bool AFF, bool SPLIT>
 __global__ void __launch_bounds__(NQ == 8 ? 512 : 1024) tdc_conv1x1_stream_kernel(const ConvKParams p) {
     extern __shared__ __align__(16) float lds[];
     if constexpr (TDC_TOUCH_KERNARGS) {
@@ -1079,8 +1138,11 @@ __global__ void __launch_bounds__(NQ == 8 ? 512 : 1024) tdc_conv1x1_stream_kerne
     if (logical >= p.n_wg) return;
     const int q1 = fdiv(logical, p.fd_g1);
     const int r1 = logical - q1 * p.fd_g1.d;
-    const int img = fdiv(q1, p.fd_g2);
-    const int r2 = q1 - img * p.fd_g2.d;
+    const int bz = fdiv(q1, p.fd_g2);          // image * KS + slice of the input channels
+    const int r2 = q1 - bz * p.fd_g2.d;
+    const int img = SPLIT ? fdiv(bz, p.fd_ks) : bz;
+    const int slice = SPLIT ? bz - img * p.KS : 0;
+    const int KS = SPLIT ? p.KS : 1;
     const int bx = p.channel_major ? r1 : r2;  // pixel block
     const int by = p.channel_major ? r2 : r1;  // channel block
     const float *__restrict__ in = p.in + (long long)img * p.in_bstride;
@@ -1094,12 +1156,13 @@ __global__ void __launch_bounds__(NQ == 8 ? 512 : 1024) tdc_conv1x1_stream_kerne
     const int k = lane >> 4, n = lane & 15;
     const int px = bx * 16 + n;
     const int pxr = min(px, p.P - 1);
-    const int c0 = wave * (16 * NQ) + 4 * k;   // this lane's first channel
+    const int cl = wave * (16 * NQ) + 4 * k;   // this lane's first channel inside the workgroup's slice
+    const int c0 = slice * p.CCH + cl;         // ... and in the image
     const unsigned HW4 = (unsigned)p.W * 4u;   // bytes between channels (the image is one row of H*W pixels)
 
     f4_t a[NQ], sc[NQ], sh[NQ];
     float b[NQ][4];
-    const int a_soff = (by * (p.CCH >> 4) + wave * NQ) * 1024;
+    const int a_soff = ((by * KS + slice) * (p.CCH >> 4) + wave * NQ) * 1024;
     const unsigned b_voff = (unsigned)c0 * HW4 + (unsigned)pxr * 4u;
 #pragma unroll
     for (int q = 0; q < NQ; ++q) {
@@ -1109,9 +1172,9 @@ __global__ void __launch_bounds__(NQ == 8 ? 512 : 1024) tdc_conv1x1_stream_kerne
             b[q][s4] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(in_rsrc, (int)(b_voff + (unsigned)(16 * q + s4) * HW4), 0, 0));
         if constexpr (AFF) {
             const __amdgpu_buffer_rsrc_t aff_rsrc =
-                __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.in_aff), (short)0, p.CCH * 8, 0x00020000);
-            sc[q] = __builtin_bit_cast(f4_t, __builtin_amdgcn_raw_buffer_load_b128(aff_rsrc, (c0 + 16 * q) * 4, 0, 0));
-            sh[q] = __builtin_bit_cast(f4_t, __builtin_amdgcn_raw_buffer_load_b128(aff_rsrc, (p.CCH + c0 + 16 * q) * 4, 0, 0));
+                __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.in_aff + slice * 2 * p.CCH), (short)0, p.CCH * 8, 0x00020000);
+            sc[q] = __builtin_bit_cast(f4_t, __builtin_amdgcn_raw_buffer_load_b128(aff_rsrc, (cl + 16 * q) * 4, 0, 0));
+            sh[q] = __builtin_bit_cast(f4_t, __builtin_amdgcn_raw_buffer_load_b128(aff_rsrc, (p.CCH + cl + 16 * q) * 4, 0, 0));
         }
         __builtin_amdgcn_sched_barrier(0);   // requests in the order the MFMAs consume them
     }
@@ -1139,13 +1202,18 @@ __global__ void __launch_bounds__(NQ == 8 ? 512 : 1024) tdc_conv1x1_stream_kerne
 #pragma unroll
         for (int i = 0; i < 4; ++i) lds[(wave * 4 + i) * 64 + lane] = acc[i];
         __syncthreads();
-        if (wave != 0) return;
-        acc = (f4_t){0.0f, 0.0f, 0.0f, 0.0f};
-        for (int w = 0; w < p.WK; ++w)
+        if (wave == 0) {
+            acc = (f4_t){0.0f, 0.0f, 0.0f, 0.0f};
+            for (int w = 0; w < p.WK; ++w)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) acc[i] += lds[(w * 4 + i) * 64 + lane];
+                for (int i = 0; i < 4; ++i) acc[i] += lds[(w * 4 + i) * 64 + lane];
+        }
     }
-    if (px >= p.P) return;
+    if constexpr (SPLIT) {
+        // the input channels are split over KS workgroups: whoever finishes last adds the partial blocks in slice order
+        if (!stream_join_slices(p, lds, acc, wave == 0 && px < p.P, by * 16 + 4 * k, px, img, slice, by, bx)) return;
+    }
+    if (wave != 0 || px >= p.P) return;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int ch = by * 16 + 4 * k + i;
@@ -1197,7 +1265,7 @@ static int taps_mode(int KH, int KW, int dil) {
 // ROW (stride 1 and a tile of one row of 14 pixels): the 16 lanes of a quarter load the 16 consecutive input pixels
 // that the row of outputs touches, once per filter row, and the three taps of a row are lane shifts of that value
 // (three requests per group of channels instead of nine).
-template <int CG, bool ROW>
+template <int CG, bool ROW, bool SPLIT>
 __global__ void __launch_bounds__(1024) tdc_conv3x3_stream_kernel(const ConvKParams p) {
     extern __shared__ __align__(16) float lds[];
     if constexpr (TDC_TOUCH_KERNARGS) {
@@ -1218,8 +1286,11 @@ __global__ void __launch_bounds__(1024) tdc_conv3x3_stream_kernel(const ConvKPar
     if (logical >= p.n_wg) return;
     const int q1 = fdiv(logical, p.fd_g1);
     const int r1 = logical - q1 * p.fd_g1.d;
-    const int img = fdiv(q1, p.fd_g2);
-    const int r2 = q1 - img * p.fd_g2.d;
+    const int bz = fdiv(q1, p.fd_g2);          // image * KS + slice of the input channels
+    const int r2 = q1 - bz * p.fd_g2.d;
+    const int img = SPLIT ? fdiv(bz, p.fd_ks) : bz;
+    const int slice = SPLIT ? bz - img * p.KS : 0;
+    const int KS = SPLIT ? p.KS : 1;
     const int bx = p.channel_major ? r1 : r2;  // pixel tile
     const int by = p.channel_major ? r2 : r1;  // channel block
     const int tile_y = fdiv(bx, p.fd_ntx);
@@ -1237,7 +1308,8 @@ __global__ void __launch_bounds__(1024) tdc_conv3x3_stream_kernel(const ConvKPar
     const int wki = wave - wmi * p.WK;
     const int mblk = by * p.WM + wmi;   // this wave's block of 16 output channels
     // The weights depend on nothing but the channel block and the wave: request them before any pixel arithmetic.
-    const int a_soff = (mblk * (p.CCH >> 2) + wki * CG) * 2304;            // nine taps x 64 lanes x 4 bytes per group
+    // packed as [channel tile][slice][block of the workgroup][group]: nine taps x 64 lanes x 4 bytes per group
+    const int a_soff = ((((by * KS + slice) * p.WM + wmi) * (p.CCH >> 2)) + wki * CG) * 2304;
     f4_t a0[CG], a1[CG];
     float a8[CG], b[CG][9];
 #pragma unroll
@@ -1256,7 +1328,7 @@ __global__ void __launch_bounds__(1024) tdc_conv3x3_stream_kernel(const ConvKPar
     const int iy0 = oy * p.stride - p.pad, ix0 = ox * p.stride - p.pad;
     const unsigned rowb = (unsigned)p.W * 4u;
     const unsigned chan_bytes = (unsigned)(p.H * p.W) * 4u;
-    const unsigned base = (unsigned)(wki * (4 * CG) + k) * chan_bytes;   // this lane's first channel
+    const unsigned base = (unsigned)(slice * p.CCH + wki * (4 * CG) + k) * chan_bytes;   // this lane's first channel
     if constexpr (ROW) {
         // lane n of a quarter: input column (tile's first column - pad + n) of the three input rows
         const int iyr = tile_y - p.pad, ixr = tile_x * 14 - p.pad + n;
@@ -1393,6 +1465,9 @@ __global__ void __launch_bounds__(1024) tdc_conv3x3_stream_kernel(const ConvKPar
         }
         return;
     }
+    if constexpr (SPLIT) {
+        if (!stream_join_slices(p, lds, acc, wki == 0 && live, mblk * 16 + 4 * k, pp, img, slice, by, bx)) return;
+    }
     if (wki != 0 || !live) return;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -1407,13 +1482,23 @@ __global__ void __launch_bounds__(1024) tdc_conv3x3_stream_kernel(const ConvKPar
     }
 }
 
-template <bool AFF>
+template <bool AFF, bool SPLIT>
 static kernel_fn pick_stream(int nq) {
     switch (nq) {
-        case 1: return tdc_conv1x1_stream_kernel<1, AFF>;
-        case 2: return tdc_conv1x1_stream_kernel<2, AFF>;
-        case 4: return tdc_conv1x1_stream_kernel<4, AFF>;
-        case 8: return tdc_conv1x1_stream_kernel<8, AFF>;
+        case 1: return tdc_conv1x1_stream_kernel<1, AFF, SPLIT>;
+        case 2: return tdc_conv1x1_stream_kernel<2, AFF, SPLIT>;
+        case 4: return tdc_conv1x1_stream_kernel<4, AFF, SPLIT>;
+        case 8: return tdc_conv1x1_stream_kernel<8, AFF, SPLIT>;
+        default: return nullptr;
+    }
+}
+
+template <bool ROW, bool SPLIT>
+static kernel_fn pick_stream3(int groups) {
+    switch (groups) {
+        case 1: return tdc_conv3x3_stream_kernel<1, ROW, SPLIT>;
+        case 2: return tdc_conv3x3_stream_kernel<2, ROW, SPLIT>;
+        case 4: return tdc_conv3x3_stream_kernel<4, ROW, SPLIT>;
         default: return nullptr;
     }
 }
@@ -1426,12 +1511,10 @@ const void *conv_kernel_for(const tdc_tile &t, int KH, int KW, int dilation, int
             return nullptr;
         const int groups = t.cch % (4 * t.wk) == 0 ? t.cch / (4 * t.wk) : 0;
         const bool row = stride == 1 && t.tw == 14;
-        switch (groups) {
-            case 1: return reinterpret_cast<const void *>(row ? static_cast<kernel_fn>(tdc_conv3x3_stream_kernel<1, true>) : static_cast<kernel_fn>(tdc_conv3x3_stream_kernel<1, false>));
-            case 2: return reinterpret_cast<const void *>(row ? static_cast<kernel_fn>(tdc_conv3x3_stream_kernel<2, true>) : static_cast<kernel_fn>(tdc_conv3x3_stream_kernel<2, false>));
-            case 4: return reinterpret_cast<const void *>(row ? static_cast<kernel_fn>(tdc_conv3x3_stream_kernel<4, true>) : static_cast<kernel_fn>(tdc_conv3x3_stream_kernel<4, false>));
-            default: return nullptr;
-        }
+        const bool split = t.ks > 1;
+        kernel_fn f = row ? (split ? pick_stream3<true, true>(groups) : pick_stream3<true, false>(groups))
+                          : (split ? pick_stream3<false, true>(groups) : pick_stream3<false, false>(groups));
+        return reinterpret_cast<const void *>(f);
     }
     if (t.alg == 3) {
         // (`extras` here can only mean the input affine: the host refuses a fused tail for this path)
@@ -1439,7 +1522,8 @@ const void *conv_kernel_for(const tdc_tile &t, int KH, int KW, int dilation, int
         if (t.cch % (16 * t.wk) != 0) return nullptr;
         const int nq = t.cch / (16 * t.wk);
         if (t.wk > (nq == 8 ? 8 : 16)) return nullptr;
-        return reinterpret_cast<const void *>(extras ? pick_stream<true>(nq) : pick_stream<false>(nq));
+        if (t.ks > 1) return reinterpret_cast<const void *>(extras ? pick_stream<true, true>(nq) : pick_stream<false, true>(nq));
+        return reinterpret_cast<const void *>(extras ? pick_stream<true, false>(nq) : pick_stream<false, false>(nq));
     }
     if (t.alg == 1) {
         if (extras || KH != 3 || KW != 3 || dilation != 1 || t.mf != 16 || t.mb != 1 || t.nb != 1) return nullptr;

@@ -44,6 +44,36 @@ __global__ void __launch_bounds__(256) pool2d_kernel(const float *__restrict__ i
     out[b * out_bs + (long long)c * Ho * Wo + pix] = acc;
 }
 
+// The same for the window sizes the networks use (3x3 max pool after the stem, 2x2 average pools in DenseNet's transitions),
+// without branches: every load of the window is issued at once.  An index outside the image is clamped into it; for a max pool
+// the clamped element lies inside the same window (pad < K), so the duplicate changes nothing, and the average variant is only
+// launched when every window lies inside the image.  Same visiting order, so the results equal the general kernel's bit for bit.
+template <int K, int MODE>
+__global__ void __launch_bounds__(256) pool2d_fixed_kernel(const float *__restrict__ in, long long in_bs,
+                                                           float *__restrict__ out, long long out_bs, int H, int W, int Ho,
+                                                           int Wo, int stride, int pad) {
+    const int pix = blockIdx.x * blockDim.x + threadIdx.x;
+    if (pix >= Ho * Wo) return;
+    const int c = blockIdx.y, b = blockIdx.z;
+    const int oy = pix / Wo, ox = pix - oy * Wo;
+    const float *src = in + b * in_bs + (long long)c * H * W;
+    const int iy0 = oy * stride - pad, ix0 = ox * stride - pad;
+    float v[K][K];
+#pragma unroll
+    for (int r = 0; r < K; ++r) {
+        const int iy = min(max(iy0 + r, 0), H - 1);
+#pragma unroll
+        for (int s = 0; s < K; ++s) v[r][s] = src[iy * W + min(max(ix0 + s, 0), W - 1)];
+    }
+    float acc = MODE == 0 ? -FLT_MAX : 0.0f;
+#pragma unroll
+    for (int r = 0; r < K; ++r)
+#pragma unroll
+        for (int s = 0; s < K; ++s) acc = MODE == 0 ? fmaxf(acc, v[r][s]) : acc + v[r][s];
+    if (MODE == 1) acc *= 1.0f / (float)(K * K);
+    out[b * out_bs + (long long)c * Ho * Wo + pix] = acc;
+}
+
 // Global average pool: one wave per plane, lanes stride over the H*W pixels, shuffle reduction.
 __global__ void __launch_bounds__(256) global_avgpool_kernel(const float *__restrict__ in, long long in_bs,
                                                              float *__restrict__ out, long long out_bs, int B, int C,
@@ -95,8 +125,17 @@ static unsigned blocks_for(long long total) { return (unsigned)((total + 255) / 
 int launch_pool2d(const float *in, long long in_bs, float *out, long long out_bs, int B, int C, int H, int W, int Ho,
                   int Wo, int k, int stride, int pad, int mode, void *stream) {
     if (C > 65535 || B > 65535) return (int)hipErrorInvalidValue;
-    hipLaunchKernelGGL(pool2d_kernel, dim3(blocks_for((long long)Ho * Wo), C, B), dim3(256), 0, (hipStream_t)stream, in,
-                       in_bs, out, out_bs, C, H, W, Ho, Wo, k, stride, pad, mode);
+    const dim3 grid(blocks_for((long long)Ho * Wo), C, B);
+    const bool inside = (long long)(Ho - 1) * stride - pad + k <= H && (long long)(Wo - 1) * stride - pad + k <= W;
+    if (mode == 0 && k == 3 && pad < 3 && H >= 1 && W >= 1)
+        hipLaunchKernelGGL((pool2d_fixed_kernel<3, 0>), grid, dim3(256), 0, (hipStream_t)stream, in, in_bs, out, out_bs, H, W,
+                           Ho, Wo, stride, pad);
+    else if (mode == 1 && k == 2 && pad == 0 && inside)
+        hipLaunchKernelGGL((pool2d_fixed_kernel<2, 1>), grid, dim3(256), 0, (hipStream_t)stream, in, in_bs, out, out_bs, H, W,
+                           Ho, Wo, stride, pad);
+    else
+        hipLaunchKernelGGL(pool2d_kernel, grid, dim3(256), 0, (hipStream_t)stream, in, in_bs, out, out_bs, C, H, W, Ho, Wo, k,
+                           stride, pad, mode);
     return (int)hipGetLastError();
 }
 

@@ -139,10 +139,10 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
         if (d.KH != 3 || d.KW != 3 || d.dilation != 1) return fail("tile.alg = 4 needs a 3x3 / dilation 1 convolution");
         if (t.mf != 16 || t.mb != 1 || t.nb != 1 || t.wn != 1) return fail("tile.alg = 4 needs mf = 16 and one pixel block per workgroup");
         if (t.wm * t.wk > 16) return fail("tile.alg = 4: at most 16 waves (wm channel blocks x wk channel slices)");
-        if (t.ks != 1 || t.wl != 0) return fail("tile.alg = 4 has no split across workgroups and no loader waves");
+        if (t.wl != 0) return fail("tile.alg = 4 has no loader waves");
         const int groups = (t.cch % (4 * t.wk) == 0) ? t.cch / (4 * t.wk) : 0;
         if (groups != 1 && groups != 2 && groups != 4) return fail("tile.alg = 4 needs cch = 4 * wk * {1, 2, 4}");
-        if (t.cch < d.C) return fail("tile.alg = 4 takes all input channels in one pass");
+        if (ceil_div(d.C, t.cch) != t.ks) return fail("tile.alg = 4 takes its input channels in one pass: ks slices of cch channels must cover them exactly");
         if ((long long)t.cch * d.H * d.W * 4 >= (1LL << 31)) return fail("image too large for tile.alg = 4");
     }
     g.wino = t.alg == 1;
@@ -151,12 +151,12 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
         // over wk waves in runs of 16, everything in one pass
         if (!flat) return fail("tile.alg = 3 needs a 1x1 / stride 1 / pad 0 convolution");
         if (t.mf != 16 || t.mb != 1 || t.nb != 1 || t.wm != 1 || t.wn != 1) return fail("tile.alg = 3 needs mf = 16 and one block per workgroup");
-        if (t.ks != 1 || t.wl != 0) return fail("tile.alg = 3 has no split across workgroups and no loader waves");
+        if (t.wl != 0) return fail("tile.alg = 3 has no loader waves");
         if (tail_N > 0) return fail("tile.alg = 3 cannot carry a fused tail");
         const int runs = (t.cch % (16 * t.wk) == 0) ? t.cch / (16 * t.wk) : 0;
         if (runs != 1 && runs != 2 && runs != 4 && runs != 8) return fail("tile.alg = 3 needs cch = 16 * wk * {1, 2, 4, 8}");
         if (runs == 8 && t.wk > 8) return fail("tile.alg = 3 with eight runs per wave is built for at most 8 waves");
-        if (t.cch < d.C) return fail("tile.alg = 3 takes all input channels in one pass");
+        if (ceil_div(d.C, t.cch) != t.ks) return fail("tile.alg = 3 takes its input channels in one pass: ks slices of cch channels must cover them exactly");
         if (t.tw != std::min(16, g.Wo)) return fail("tile.alg = 3 needs tw = min(16, pixels)");
         if ((long long)t.cch * g.We * 4 >= (1LL << 31)) return fail("image too large for tile.alg = 3");
     }
@@ -252,6 +252,7 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
         g.tail_f_off = t.wk > 1 ? t.wk * g.MT * g.PT : 0;
         lds = std::max(lds, ((long long)g.tail_f_off + (long long)g.MT * g.tail_ld) * 4);
     }
+    if (t.alg >= 3 && t.ks > 1) lds = std::max<long long>(lds, 16);   // the drawn ticket is passed through LDS
     if (lds > machine().lds_bytes_per_cu) return fail("tile needs more than 160 KiB of LDS");
     g.lds_bytes = (int)lds;
     if (const char *e = std::getenv("TDC_EXPERIMENT_MIN_LDS")) g.lds_bytes = std::max(g.lds_bytes, std::atoi(e));
@@ -297,8 +298,8 @@ void pack_weights(const tdc_conv_desc &d, const tdc_tile &t, const Geometry &g, 
     }
     if (t.alg == 3) {
         // per (channel block, run of 16 input channels): [lane][s], lane (n = l % 16, k = l / 16) holding
-        // w[block*16 + n][16*run + 4*k + s]
-        const int runs = t.cch / 16;
+        // w[block*16 + n][16*run + 4*k + s]; the runs of all slices of a split across workgroups follow each other
+        const int runs = g.nchunks * (t.cch / 16);
         for (int by = 0; by < g.grid_y; ++by)
             for (int r = 0; r < runs; ++r)
                 for (int l = 0; l < 64; ++l)
@@ -505,6 +506,7 @@ bool model_evaluate(const tdc_conv_desc &d, const tdc_tile &t, tdc_tile_info &in
                        (double)tail_N * d.N * 4.0 * r / rate + (double)tail_N * 64.0 * r / 200.0;
                 return clk;
             }
+            if (t.ks > 1) clk += MC.ksplit_clk + 1000.0 * (t.ks - 2) + (double)t.ks * 1024.0 * r / rate;   // (timed: each slice past the second adds 0.4 us)
             clk += out_bytes * r / 200.0;
             return clk;
         }
@@ -522,6 +524,7 @@ bool model_evaluate(const tdc_conv_desc &d, const tdc_tile &t, tdc_tile_info &in
             double clk = MC.stream_setup_clk + MC.stream_latency_clk + 20.0 * (waves_simd - 1.0) + bytes / (0.87 * rate) +
                          runs * 4.0 * 0.5 * mfma_clk * waves_simd;
             if (t.wk > 1) clk += 1.5 * MC.sync_clk;
+            if (t.ks > 1) clk += MC.ksplit_clk + 1000.0 * (t.ks - 2) + (double)t.ks * 1024.0 * r / rate;   // (timed: each slice past the second adds 0.4 us)
             clk += out_bytes * r / 64.0;
             return clk;
         }
@@ -593,19 +596,23 @@ std::vector<tdc_tile> model_enumerate(const tdc_conv_desc &d, int tail_N) {
     static const int wns[] = {1, 2, 4};
     // streamed 1x1 candidates: the input channels in runs of 16, 1, 2, 4 or 8 runs per wave
     if (flat && tail_N == 0 && !std::getenv("TDC_EXPERIMENT_NO_STREAMED_1X1")) {
-        const int runs = ceil_div(d.C, 16);
-        for (int per_wave : {8, 4, 2, 1}) {
-            if (per_wave > runs) continue;   // (more than half of such a wave's channels would be padding)
-            const int wk = ceil_div(runs, per_wave);
-            if (wk > 16) continue;
-            tdc_tile t{16, 1, 1, 1, 1, wk, 16 * per_wave * wk, std::min(16, Wo), 1, 0, 3};
-            Geometry g;
-            if (make_geometry(d, t, g, nullptr, 0)) out.push_back(t);
+        // (a split of the input channels over ks workgroups only where the layer leaves most of the chip idle)
+        for (int ks : {1, 2, 4, 8}) {
+            const int runs = ceil_div(ceil_div(d.C, ks), 16);
+            for (int per_wave : {8, 4, 2, 1}) {
+                if (per_wave > runs) continue;   // (more than half of such a wave's channels would be padding)
+                const int wk = ceil_div(runs, per_wave);
+                if (wk > 16) continue;
+                tdc_tile t{16, 1, 1, 1, 1, wk, 16 * per_wave * wk, std::min(16, Wo), ks, 0, 3};
+                Geometry g;
+                if (!make_geometry(d, t, g, nullptr, 0)) continue;
+                if (ks > 1 && (long long)g.grid_x * g.grid_y * g.grid_z > 2LL * machine().cus) continue;
+                out.push_back(t);
+            }
         }
     }
     // streamed 3x3 candidates: 1, 2 or 4 groups of four channels per wave, a few shapes of the 16-pixel tile
     if (d.KH == 3 && d.KW == 3 && d.dilation == 1 && !std::getenv("TDC_EXPERIMENT_NO_STREAMED_3X3")) {
-        const int groups = ceil_div(d.C, 4);
         std::vector<int> tws;
         for (int tw : {16, 14, 8, 7, 4, std::min(16, Wo)}) {
             if (tw > std::min(16, Wo) || std::find(tws.begin(), tws.end(), tw) != tws.end()) continue;
@@ -616,14 +623,20 @@ std::vector<tdc_tile> model_enumerate(const tdc_conv_desc &d, int tail_N) {
         }
         // (a fused tail needs every output channel in the workgroup: one wave per block of 16 and channel slice)
         const int wm = tail_N > 0 ? ceil_div(d.N, 16) : 1;
-        for (int per_wave : {4, 2, 1}) {
-            if (per_wave > groups) continue;
-            const int wk = ceil_div(groups, per_wave);
-            if (wm * wk > 16) continue;
-            for (int tw : tws) {
-                tdc_tile t{16, 1, 1, wm, 1, wk, 4 * per_wave * wk, tw, 1, 0, 4};
-                Geometry g;
-                if (make_geometry(d, t, g, nullptr, tail_N)) out.push_back(t);
+        for (int ks : {1, 2, 4, 8}) {
+            if (ks > 1 && tail_N > 0) break;
+            const int groups_slice = ceil_div(ceil_div(d.C, ks), 4);
+            for (int per_wave : {4, 2, 1}) {
+                if (per_wave > groups_slice) continue;
+                const int wk = ceil_div(groups_slice, per_wave);
+                if (wm * wk > 16) continue;
+                for (int tw : tws) {
+                    tdc_tile t{16, 1, 1, wm, 1, wk, 4 * per_wave * wk, tw, ks, 0, 4};
+                    Geometry g;
+                    if (!make_geometry(d, t, g, nullptr, tail_N)) continue;
+                    if (ks > 1 && (long long)g.grid_x * g.grid_y * g.grid_z > 2LL * machine().cus) continue;
+                    out.push_back(t);
+                }
             }
         }
     }

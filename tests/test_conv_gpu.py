@@ -417,6 +417,37 @@ def test_split_across_workgroups(tile):
     assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2])
 
 
+@pytest.mark.parametrize("shape,K,pad", [((1, 256, 256, 7, 7), 3, 1), ((2, 130, 40, 5, 6), 3, 1), ((1, 2048, 256, 7, 7), 1, 0),
+                                         ((2, 300, 24, 3, 5), 1, 0)])
+def test_streamed_tiles_split_across_workgroups(shape, K, pad):
+    """Streamed kernels with the input channels dealt to several workgroups (tile.alg = 3 / 4 with tile.ks > 1): the
+    enumeration offers such tiles for layers with few workgroups; every one matches the oracle with the whole epilogue,
+    gives the same bits on every launch (the partial blocks are added in slice order by whichever workgroup comes
+    last), and leaves the ticket counters at zero for the next launch."""
+    B, C, N, H, W = shape
+    x, w = case(6100 + C + N, B, C, N, H, W, K)
+    g = seeded(6101)
+    bias = torch.randn(N, generator=g)
+    resid = torch.randn(B, N, H, W, generator=g)
+    want = ref.conv2d_c(x.numpy(), w.numpy(), bias.numpy(), resid.numpy(), pad=pad, relu=True)
+    tiles = [t for t in tdc_amd.model_enumerate(tdc_amd.conv_desc(B, C, N, H, W, K, K, 1, pad)) if t.alg >= 3 and t.ks > 1]
+    assert tiles and {t.ks for t in tiles} >= {2, 4}
+    xd, rd = x.cuda(), resid.cuda()
+    for t in tiles:
+        announce("streamed split", shape, K, t)
+        plan = tdc_amd.Conv2dPlan(B, C, N, H, W, K, K, 1, pad, 1, True, True, tile=t).set_weights(w, bias)
+        assert plan.info.grid_z == B * t.ks
+        outs = []
+        for rep in range(3):
+            out = torch.full((B, N, H, W), float("nan"), device="cuda")
+            plan.forward(xd, rd, out=out)
+            torch.cuda.synchronize()
+            outs.append(out.cpu().numpy())
+        plan.close()
+        assert_close(outs[0], want, f"streamed split {shape} {t}")
+        assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2])
+
+
 @pytest.mark.parametrize("order", ["0", "1"])
 def test_both_logical_workgroup_orders(order, monkeypatch):
     """The launch is one-dimensional and decoded in the kernel; both decode orders (channel tile fastest / pixel
