@@ -1265,8 +1265,11 @@ static int taps_mode(int KH, int KW, int dil) {
 // ROW (stride 1 and a tile of one row of 14 pixels): the 16 lanes of a quarter load the 16 consecutive input pixels
 // that the row of outputs touches, once per filter row, and the three taps of a row are lane shifts of that value
 // (three requests per group of channels instead of nine).
-template <int CG, bool ROW, bool SPLIT>
+// MODE: 0 = plain, 1 = input channels dealt to p.KS workgroups, 2 = with the fused 1x1 tail.  Separate instantiations:
+// code a launch never runs still costs it (0.13 us per launch measured for the split's code inside the plain kernel).
+template <int CG, bool ROW, int MODE>
 __global__ void __launch_bounds__(1024) tdc_conv3x3_stream_kernel(const ConvKParams p) {
+    constexpr bool SPLIT = MODE == 1, TAIL = MODE == 2;
     extern __shared__ __align__(16) float lds[];
     if constexpr (TDC_TOUCH_KERNARGS) {
         const auto kargs = __builtin_amdgcn_kernarg_segment_ptr();
@@ -1412,7 +1415,7 @@ __global__ void __launch_bounds__(1024) tdc_conv3x3_stream_kernel(const ConvKPar
         }
     }
     const int pp = oy * p.Wo + ox;
-    if (p.tail_w) {
+    if constexpr (TAIL) {
         // Fused 1x1 tail, out2 = W2 * act(conv + bias): the workgroup owns every output channel of the convolution
         // (the host guarantees it).  The finished 16-pixel columns are parked in LDS as f[channel][pixel] — the B operand
         // of a second small GEMM whose A operand, the tail's packed weights, comes from global memory — and its
@@ -1493,12 +1496,12 @@ static kernel_fn pick_stream(int nq) {
     }
 }
 
-template <bool ROW, bool SPLIT>
+template <bool ROW, int MODE>
 static kernel_fn pick_stream3(int groups) {
     switch (groups) {
-        case 1: return tdc_conv3x3_stream_kernel<1, ROW, SPLIT>;
-        case 2: return tdc_conv3x3_stream_kernel<2, ROW, SPLIT>;
-        case 4: return tdc_conv3x3_stream_kernel<4, ROW, SPLIT>;
+        case 1: return tdc_conv3x3_stream_kernel<1, ROW, MODE>;
+        case 2: return tdc_conv3x3_stream_kernel<2, ROW, MODE>;
+        case 4: return tdc_conv3x3_stream_kernel<4, ROW, MODE>;
         default: return nullptr;
     }
 }
@@ -1511,9 +1514,11 @@ const void *conv_kernel_for(const tdc_tile &t, int KH, int KW, int dilation, int
             return nullptr;
         const int groups = t.cch % (4 * t.wk) == 0 ? t.cch / (4 * t.wk) : 0;
         const bool row = stride == 1 && t.tw == 14;
-        const bool split = t.ks > 1;
-        kernel_fn f = row ? (split ? pick_stream3<true, true>(groups) : pick_stream3<true, false>(groups))
-                          : (split ? pick_stream3<false, true>(groups) : pick_stream3<false, false>(groups));
+        if (extras && t.ks > 1) return nullptr;
+        const int mode = extras ? 2 : t.ks > 1 ? 1 : 0;
+        kernel_fn f = nullptr;
+        if (row) f = mode == 2 ? pick_stream3<true, 2>(groups) : mode == 1 ? pick_stream3<true, 1>(groups) : pick_stream3<true, 0>(groups);
+        else f = mode == 2 ? pick_stream3<false, 2>(groups) : mode == 1 ? pick_stream3<false, 1>(groups) : pick_stream3<false, 0>(groups);
         return reinterpret_cast<const void *>(f);
     }
     if (t.alg == 3) {
