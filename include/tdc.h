@@ -88,7 +88,7 @@ typedef struct tdc_tile {
                      2 = direct 3x3 / dilation 1 convolution with the weights read from global memory straight
                          into registers (the LDS holds input only, so a pass can take more input channels);
                          mb = nb = 1, an even number of channel groups per wave and pass.
-                     3 = 1x1 / stride 1 / pad 0 convolution with BOTH operands read from global memory straight into
+                     3 = 1x1 / pad 0 convolution (any stride; ks = 1 when the stride is above 1) with BOTH operands read from global memory straight into
                          registers: no LDS stage, one pass; a workgroup owns 16 channels x 16 pixels, its wk (<= 16)
                          waves split the input channels in runs of 16; cch = 16 * wk * {1, 2, 4, 8}
                          (eight runs per wave: wk <= 8) with ks * cch >= C and ceil(C / cch) = ks: ks > 1 deals slices

@@ -1114,9 +1114,11 @@ __device__ __forceinline__ bool stream_join_slices(const ConvKParams &p, float *
 // re-read its last pixel and are never stored.
 // ---------------------------------------------------------------------------
 // (eight runs per wave: 72 registers of operands, 136 with the affine; that variant is built for at most 8 waves)
-// SPLIT: the instantiation whose input channels are dealt to p.KS workgroups (the plain one pays nothing for it).
-template <int NQ, bool AFF, bool SPLIT>
+// MODE 1: the instantiation whose input channels are dealt to p.KS workgroups.  MODE 2: stride > 1 (ResNet's downsampling
+// shortcuts): output pixel (oy, ox) reads input pixel (oy * stride, ox * stride).  The plain one pays for neither.
+template <int NQ, bool AFF, int MODE>
 __global__ void __launch_bounds__(NQ == 8 ? 512 : 1024) tdc_conv1x1_stream_kernel(const ConvKParams p) {
+    constexpr bool SPLIT = MODE == 1, STRIDED = MODE == 2;
     extern __shared__ __align__(16) float lds[];
     if constexpr (TDC_TOUCH_KERNARGS) {
         static_assert(sizeof(ConvKParams) <= 8 * 64, "touch more lines");
@@ -1158,12 +1160,19 @@ __global__ void __launch_bounds__(NQ == 8 ? 512 : 1024) tdc_conv1x1_stream_kerne
     const int pxr = min(px, p.P - 1);
     const int cl = wave * (16 * NQ) + 4 * k;   // this lane's first channel inside the workgroup's slice
     const int c0 = slice * p.CCH + cl;         // ... and in the image
-    const unsigned HW4 = (unsigned)p.W * 4u;   // bytes between channels (the image is one row of H*W pixels)
+    // bytes between channels (with stride 1 the host presents the image as one row of H*W pixels)
+    const unsigned HW4 = STRIDED ? (unsigned)(p.H * p.W) * 4u : (unsigned)p.W * 4u;
+    unsigned pix4 = (unsigned)pxr * 4u;        // this lane's input pixel, in bytes from the start of a channel
+    if constexpr (STRIDED) {
+        const int oy = fdiv(pxr, p.fd_wtw);    // (fd_wtw holds the output row length here)
+        const int ox = pxr - oy * p.Wo;
+        pix4 = (unsigned)((oy * p.W + ox) * p.stride) * 4u;
+    }
 
     f4_t a[NQ], sc[NQ], sh[NQ];
     float b[NQ][4];
     const int a_soff = ((by * KS + slice) * (p.CCH >> 4) + wave * NQ) * 1024;
-    const unsigned b_voff = (unsigned)c0 * HW4 + (unsigned)pxr * 4u;
+    const unsigned b_voff = (unsigned)c0 * HW4 + pix4;
 #pragma unroll
     for (int q = 0; q < NQ; ++q) {
         a[q] = __builtin_bit_cast(f4_t, __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, lane * 16, a_soff + q * 1024, 0));
@@ -1485,13 +1494,13 @@ __global__ void __launch_bounds__(1024) tdc_conv3x3_stream_kernel(const ConvKPar
     }
 }
 
-template <bool AFF, bool SPLIT>
+template <bool AFF, int MODE>
 static kernel_fn pick_stream(int nq) {
     switch (nq) {
-        case 1: return tdc_conv1x1_stream_kernel<1, AFF, SPLIT>;
-        case 2: return tdc_conv1x1_stream_kernel<2, AFF, SPLIT>;
-        case 4: return tdc_conv1x1_stream_kernel<4, AFF, SPLIT>;
-        case 8: return tdc_conv1x1_stream_kernel<8, AFF, SPLIT>;
+        case 1: return tdc_conv1x1_stream_kernel<1, AFF, MODE>;
+        case 2: return tdc_conv1x1_stream_kernel<2, AFF, MODE>;
+        case 4: return tdc_conv1x1_stream_kernel<4, AFF, MODE>;
+        case 8: return tdc_conv1x1_stream_kernel<8, AFF, MODE>;
         default: return nullptr;
     }
 }
@@ -1527,8 +1536,10 @@ const void *conv_kernel_for(const tdc_tile &t, int KH, int KW, int dilation, int
         if (t.cch % (16 * t.wk) != 0) return nullptr;
         const int nq = t.cch / (16 * t.wk);
         if (t.wk > (nq == 8 ? 8 : 16)) return nullptr;
-        if (t.ks > 1) return reinterpret_cast<const void *>(extras ? pick_stream<true, true>(nq) : pick_stream<false, true>(nq));
-        return reinterpret_cast<const void *>(extras ? pick_stream<true, false>(nq) : pick_stream<false, false>(nq));
+        if (stride > 1 && t.ks > 1) return nullptr;
+        if (stride > 1) return reinterpret_cast<const void *>(extras ? pick_stream<true, 2>(nq) : pick_stream<false, 2>(nq));
+        if (t.ks > 1) return reinterpret_cast<const void *>(extras ? pick_stream<true, 1>(nq) : pick_stream<false, 1>(nq));
+        return reinterpret_cast<const void *>(extras ? pick_stream<true, 0>(nq) : pick_stream<false, 0>(nq));
     }
     if (t.alg == 1) {
         if (extras || KH != 3 || KW != 3 || dilation != 1 || t.mf != 16 || t.mb != 1 || t.nb != 1) return nullptr;

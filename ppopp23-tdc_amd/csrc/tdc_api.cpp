@@ -481,7 +481,7 @@ int tdc_conv_forward_strided(tdc_conv_plan *plan, const float *d_in, int64_t in_
     kp.fd_tw = make_fastdiv(g.TW);
     kp.fd_ntx = make_fastdiv(g.ntx);
     kp.fd_pt = make_fastdiv(g.PT);
-    kp.fd_wtw = make_fastdiv(g.wino ? g.TWt : 1);
+    kp.fd_wtw = make_fastdiv(g.wino ? g.TWt : (plan->tile.alg == 3 && d.stride > 1) ? g.Wo : 1);
     kp.fd_wk = make_fastdiv(plan->tile.wk);
     kp.fd_wn = make_fastdiv(plan->tile.wn);
     kp.fd_ks = make_fastdiv(g.ks);

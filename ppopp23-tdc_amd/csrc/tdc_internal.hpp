@@ -133,7 +133,7 @@ struct ConvKParams {
     FastDiv fd_npx;            // 16-pixel blocks per tile
     FastDiv fd_csv, fd_rsv;      // LDS channel slot / row, in copy elements
     FastDiv fd_tw, fd_ntx, fd_pt;
-    FastDiv fd_wtw;            // Winograd: 2x2 tiles per row of the workgroup tile
+    FastDiv fd_wtw;            // Winograd: 2x2 tiles per row of the workgroup tile; streamed 1x1 with stride > 1: output row length
     FastDiv fd_wk, fd_wn, fd_ks;
     unsigned wpk_bytes;
     unsigned in_image_bytes;   // C*H*W*4: reads at or past it return zero

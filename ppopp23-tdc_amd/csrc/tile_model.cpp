@@ -149,7 +149,8 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
     if (t.alg == 3) {
         // 1x1 convolution streamed from global memory: a 16x16 output block per workgroup, the input channels split
         // over wk waves in runs of 16, everything in one pass
-        if (!flat) return fail("tile.alg = 3 needs a 1x1 / stride 1 / pad 0 convolution");
+        if (d.KH != 1 || d.KW != 1 || d.pad != 0) return fail("tile.alg = 3 needs a 1x1 / pad 0 convolution");
+        if (!flat && t.ks != 1) return fail("tile.alg = 3 with stride > 1 has no split across workgroups");
         if (t.mf != 16 || t.mb != 1 || t.nb != 1 || t.wm != 1 || t.wn != 1) return fail("tile.alg = 3 needs mf = 16 and one block per workgroup");
         if (t.wl != 0) return fail("tile.alg = 3 has no loader waves");
         if (tail_N > 0) return fail("tile.alg = 3 cannot carry a fused tail");
@@ -157,7 +158,7 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
         if (runs != 1 && runs != 2 && runs != 4 && runs != 8) return fail("tile.alg = 3 needs cch = 16 * wk * {1, 2, 4, 8}");
         if (runs == 8 && t.wk > 8) return fail("tile.alg = 3 with eight runs per wave is built for at most 8 waves");
         if (ceil_div(d.C, t.cch) != t.ks) return fail("tile.alg = 3 takes its input channels in one pass: ks slices of cch channels must cover them exactly");
-        if (t.tw != std::min(16, g.Wo)) return fail("tile.alg = 3 needs tw = min(16, pixels)");
+        if (t.tw != std::min(16, g.P)) return fail("tile.alg = 3 needs tw = min(16, pixels)");
         if ((long long)t.cch * g.We * 4 >= (1LL << 31)) return fail("image too large for tile.alg = 3");
     }
     if (t.alg == 2) {
@@ -183,12 +184,18 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
         g.PT = 4 * lanes;   // pixels the workgroup's lanes stand for
     } else {
         g.PT = t.mf * t.nb * t.wn;
-        if (t.tw < 1 || t.tw > g.PT || t.tw > g.Wo) return fail("tile.tw must be in [1, min(Wo, pixel lanes)]");
+        // (the streamed 1x1 kernel walks the output in runs of 16 consecutive pixels, whatever the image's rows are)
+        const bool runs = t.alg == 3 && !flat;
+        if (t.tw < 1 || t.tw > g.PT || (!runs && t.tw > g.Wo)) return fail("tile.tw must be in [1, min(Wo, pixel lanes)]");
         g.TW = t.tw;
-        g.TH = std::min(g.PT / t.tw, g.Ho);
+        g.TH = runs ? 1 : std::min(g.PT / t.tw, g.Ho);
     }
     g.ntx = ceil_div(g.Wo, g.TW);
     g.nty = ceil_div(g.Ho, g.TH);
+    if (t.alg == 3 && !flat) {
+        g.ntx = ceil_div(g.P, 16);
+        g.nty = 1;
+    }
     // (the kernel divides the tile index by ntx with a 32-bit multiply-high)
     if ((long long)g.ntx * g.nty > 65535 * 16) return fail("grid too large");
     if ((long long)g.ntx * g.nty * g.ntx >= (1LL << 32)) return fail("grid too large");
@@ -595,15 +602,16 @@ std::vector<tdc_tile> model_enumerate(const tdc_conv_desc &d, int tail_N) {
     static const int wms[] = {1, 2, 4};
     static const int wns[] = {1, 2, 4};
     // streamed 1x1 candidates: the input channels in runs of 16, 1, 2, 4 or 8 runs per wave
-    if (flat && tail_N == 0 && !std::getenv("TDC_EXPERIMENT_NO_STREAMED_1X1")) {
+    if (d.KH == 1 && d.KW == 1 && d.pad == 0 && tail_N == 0 && !std::getenv("TDC_EXPERIMENT_NO_STREAMED_1X1")) {
         // (a split of the input channels over ks workgroups only where the layer leaves most of the chip idle)
         for (int ks : {1, 2, 4, 8}) {
+            if (ks > 1 && !flat) break;
             const int runs = ceil_div(ceil_div(d.C, ks), 16);
             for (int per_wave : {8, 4, 2, 1}) {
                 if (per_wave > runs) continue;   // (more than half of such a wave's channels would be padding)
                 const int wk = ceil_div(runs, per_wave);
                 if (wk > 16) continue;
-                tdc_tile t{16, 1, 1, 1, 1, wk, 16 * per_wave * wk, std::min(16, Wo), ks, 0, 3};
+                tdc_tile t{16, 1, 1, 1, 1, wk, 16 * per_wave * wk, std::min(16, P), ks, 0, 3};
                 Geometry g;
                 if (!make_geometry(d, t, g, nullptr, 0)) continue;
                 if (ks > 1 && (long long)g.grid_x * g.grid_y * g.grid_z > 2LL * machine().cus) continue;

@@ -149,6 +149,35 @@ def test_every_streamed_1x1_tile(shape):
         assert_close(out.cpu().numpy(), want_aff, f"input affine {shape} {t}")
 
 
+@pytest.mark.parametrize("shape,stride", [((1, 64, 128, 56, 56), 2), ((2, 100, 40, 9, 11), 2), ((1, 256, 512, 14, 14), 2),
+                                          ((3, 19, 5, 7, 5), 3), ((1, 128, 256, 28, 28), 2), ((1, 33, 17, 1, 9), 2)])
+def test_streamed_1x1_with_stride(shape, stride):
+    """The streamed 1x1 kernel on stride > 1 (ResNet's downsampling shortcuts): output pixel (oy, ox) reads input pixel
+    (oy * stride, ox * stride); every launchable tile, odd image sizes, batches, with bias + ReLU, and with the input
+    affine in front."""
+    B, C, N, H, W = shape
+    x, w = case(2400 + C + N + H, B, C, N, H, W, 1)
+    g = seeded(2401)
+    bias = torch.randn(N, generator=g)
+    scale = torch.rand(C, generator=g) * 2 - 0.5
+    shift = torch.randn(C, generator=g) * 0.3
+    want = ref.conv2d_c(x.numpy(), w.numpy(), bias.numpy(), stride=stride, relu=True)
+    xt = (x * scale.view(1, C, 1, 1) + shift.view(1, C, 1, 1)).clamp_min(0)
+    want_aff = ref.conv2d_c(xt.numpy(), w.numpy(), bias.numpy(), stride=stride, relu=True)
+    tiles = [t for t in tdc_amd.model_enumerate(tdc_amd.conv_desc(B, C, N, H, W, 1, 1, stride, 0)) if t.alg == 3]
+    assert tiles
+    for t in tiles:
+        announce("streamed 1x1 stride", shape, stride, t)
+        assert_close(run_conv(x, w, bias, stride=stride, relu=True, tile=t), want, f"{shape} s{stride} {t}")
+        plan = tdc_amd.Conv2dPlan(B, C, N, H, W, 1, 1, stride, 0, 1, True, True, tile=t).set_weights(w, bias)
+        plan.set_input_affine(scale, shift, relu=True)
+        out = torch.full((B, N, plan.Ho, plan.Wo), float("nan"), device="cuda")
+        plan.forward(x.cuda(), out=out)
+        torch.cuda.synchronize()
+        plan.close()
+        assert_close(out.cpu().numpy(), want_aff, f"input affine {shape} s{stride} {t}")
+
+
 @pytest.mark.parametrize("shape,stride,pad", [((1, 16, 16, 7, 7), 1, 1), ((2, 13, 20, 9, 11), 1, 1), ((1, 40, 24, 13, 13), 2, 1),
                                               ((1, 16, 16, 12, 12), 1, 2), ((1, 128, 48, 7, 7), 1, 1), ((1, 64, 32, 28, 28), 1, 1),
                                               ((3, 5, 3, 4, 3), 1, 0), ((1, 250, 17, 5, 5), 2, 1)])

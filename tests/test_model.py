@@ -41,14 +41,19 @@ def test_streamed_tiles_only_where_they_apply():
     d1 = tdc_amd.conv_desc(1, 256, 64, 14, 14, 1, 1, 1, 0)
     ok = tdc_amd.model_evaluate(d1, tdc_amd.Tile(16, 1, 1, 1, 1, 4, 256, 16, 1, 0, 3))
     assert (ok.grid_x, ok.grid_y, ok.block_threads, ok.lds_bytes, ok.nchunks) == (13, 4, 256, 4096, 1)
+    split = tdc_amd.model_evaluate(d1, tdc_amd.Tile(16, 1, 1, 1, 1, 4, 128, 16, 2, 0, 3))   # two workgroups, 128 channels each
+    assert (split.grid_x, split.grid_y, split.grid_z, split.nchunks) == (13, 4, 2, 2)
+    # stride 2: runs of 16 consecutive output pixels (7 x 7 = 49 of them), whatever the rows of the image are
+    s2 = tdc_amd.model_evaluate(tdc_amd.conv_desc(1, 256, 64, 14, 14, 1, 1, 2, 0), tdc_amd.Tile(16, 1, 1, 1, 1, 4, 256, 16, 1, 0, 3))
+    assert (s2.grid_x, s2.grid_y) == (4, 4)
     for d, t in [(d1, tdc_amd.Tile(16, 1, 1, 1, 1, 1, 256, 16, 1, 0, 3)),      # 16 runs per wave
                  (d1, tdc_amd.Tile(16, 1, 1, 1, 1, 4, 128, 16, 1, 0, 3)),      # not all channels in one pass
-                 (d1, tdc_amd.Tile(16, 1, 1, 1, 1, 4, 256, 16, 2, 0, 3)),      # split across workgroups
+                 (d1, tdc_amd.Tile(16, 1, 1, 1, 1, 4, 256, 16, 2, 0, 3)),      # two slices of which one is empty
                  (d1, tdc_amd.Tile(16, 1, 1, 1, 2, 4, 256, 16, 1, 0, 3)),      # more than one block
                  (d1, tdc_amd.Tile(32, 1, 1, 1, 1, 4, 256, 16, 1, 0, 3)),
                  (d1, tdc_amd.Tile(16, 1, 1, 1, 1, 4, 256, 8, 1, 0, 3)),       # tw must be 16 (or all pixels)
                  (tdc_amd.conv_desc(1, 2048, 64, 7, 7, 1, 1, 1, 0), tdc_amd.Tile(16, 1, 1, 1, 1, 16, 2048, 16, 1, 0, 3)),  # 8 runs x 16 waves
-                 (tdc_amd.conv_desc(1, 256, 64, 14, 14, 1, 1, 2, 0), tdc_amd.Tile(16, 1, 1, 1, 1, 4, 256, 16, 1, 0, 3)),   # stride 2
+                 (tdc_amd.conv_desc(1, 256, 64, 14, 14, 1, 1, 2, 0), tdc_amd.Tile(16, 1, 1, 1, 1, 4, 128, 16, 2, 0, 3)),   # stride 2 and a split across workgroups
                  (conv3(64, 64, 14), tdc_amd.Tile(16, 1, 1, 1, 1, 4, 64, 14, 1, 0, 3))]:
         with pytest.raises(tdc_amd.TdcError):
             tdc_amd.model_evaluate(d, t)
