@@ -148,6 +148,14 @@ int tdc_conv_plan_set_tail_weights(tdc_conv_plan *plan, const float *w_tail, con
  * the norm -> relu -> conv order of the reference's DenseNet layers (inference/densenet_inet_tt.py:36-69), where the
  * BatchNorm sits in front of the convolution and cannot be folded into its weights.  Host arrays of C floats. */
 int tdc_conv_plan_set_input_affine(tdc_conv_plan *plan, const float *scale, const float *shift, int32_t relu);
+
+/* Fuse a 1x1 convolution IN FRONT of a plan that already carries a fused tail and runs the streamed 3x3 kernel
+   (tile.alg = 4, stride 1): out = tail(act(conv3x3(W_head * x))).  With the tail this is a whole TKConv
+   (inference/TKConv.py:90-95: the three F.conv2d calls) in one launch; the first factor is recomputed per
+   workgroup on its (TH + 2) x (TW + 2) window and never reaches memory.  The head has no bias (as the reference's
+   first factor), so the core's zero padding is the head applied to zero.  w_head is host [C][head_C] (C = the plan's
+   input channels); from then on the plan's input has head_C channels.  TDC_ERR_UNSUPPORTED for other plans. */
+int tdc_conv_plan_set_head(tdc_conv_plan *plan, int32_t head_C, const float *w_head);
 int tdc_conv_plan_query(const tdc_conv_plan *plan, tdc_tile_info *info_out);
 /* d_residual may be NULL.  Output need not be pre-zeroed.  Asynchronous. */
 int tdc_conv_forward(tdc_conv_plan *plan, const float *d_in, const float *d_residual,

@@ -1274,11 +1274,13 @@ static int taps_mode(int KH, int KW, int dil) {
 // ROW (stride 1 and a tile of one row of 14 pixels): the 16 lanes of a quarter load the 16 consecutive input pixels
 // that the row of outputs touches, once per filter row, and the three taps of a row are lane shifts of that value
 // (three requests per group of channels instead of nine).
-// MODE: 0 = plain, 1 = input channels dealt to p.KS workgroups, 2 = with the fused 1x1 tail.  Separate instantiations:
+// MODE: 0 = plain, 1 = input channels dealt to p.KS workgroups, 2 = with the fused 1x1 tail, 3 = with a fused 1x1 head in
+// front as well (a whole Tucker convolution in one launch: the workgroup first computes the first factor on its window of
+// (TH + 2) x (TW + 2) pixels into LDS, which the core loop then reads instead of global memory).  Separate instantiations:
 // code a launch never runs still costs it (0.13 us per launch measured for the split's code inside the plain kernel).
 template <int CG, bool ROW, int MODE>
 __global__ void __launch_bounds__(1024) tdc_conv3x3_stream_kernel(const ConvKParams p) {
-    constexpr bool SPLIT = MODE == 1, TAIL = MODE == 2;
+    constexpr bool SPLIT = MODE == 1, TAIL = MODE == 2 || MODE == 3, HEAD = MODE == 3;
     extern __shared__ __align__(16) float lds[];
     if constexpr (TDC_TOUCH_KERNARGS) {
         const auto kargs = __builtin_amdgcn_kernarg_segment_ptr();
@@ -1341,6 +1343,60 @@ __global__ void __launch_bounds__(1024) tdc_conv3x3_stream_kernel(const ConvKPar
     const unsigned rowb = (unsigned)p.W * 4u;
     const unsigned chan_bytes = (unsigned)(p.H * p.W) * 4u;
     const unsigned base = (unsigned)(slice * p.CCH + wki * (4 * CG) + k) * chan_bytes;   // this lane's first channel
+    if constexpr (HEAD) {
+        // First factor on the window: 16 x 16 blocks (channels x window pixels) dealt to the waves, both operands
+        // streamed from global memory four runs of 16 input channels at a time; pixels outside the image read zero,
+        // which is the core's zero padding (the factor has no bias).
+        float *F = lds + p.head_f_off;
+        const __amdgpu_buffer_rsrc_t hw_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<float *>(p.head_w), (short)0, p.head_mblk * p.head_runs * 1024, 0x00020000);
+        const int nwaves = p.WM * p.WK;
+        const int nblk = p.head_mblk * p.head_npb;
+        for (int blk = wave; blk < nblk; blk += nwaves) {
+            const int cb = fdiv(blk, p.fd_hnpb);
+            const int pb = blk - cb * p.head_npb;
+            const int wq = pb * 16 + n;
+            const int wy = fdiv(wq, p.fd_hww);
+            const int wx = wq - wy * p.head_ww;
+            const int iy = tile_y * p.TH - p.pad + wy, ix = tile_x * p.TW - p.pad + wx;
+            const bool ok = wq < p.head_wq && (unsigned)iy < (unsigned)p.H && (unsigned)ix < (unsigned)p.W;
+            const unsigned pix = ok ? (unsigned)(iy * p.W + ix) * 4u + (unsigned)(4 * k) * chan_bytes : (unsigned)OOB_OFFSET;
+            f4_t h0 = (f4_t){0.0f, 0.0f, 0.0f, 0.0f}, h1 = (f4_t){0.0f, 0.0f, 0.0f, 0.0f};
+            // (four runs per round trip: eight at once measured slower, the workgroup is bound by its compute unit's fill rate)
+            for (int q0 = 0; q0 < p.head_runs; q0 += 4) {
+                f4_t ha[4];
+                float hb[4][4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    ha[u] = __builtin_bit_cast(f4_t, __builtin_amdgcn_raw_buffer_load_b128(
+                                                         hw_rsrc, lane * 16, (cb * p.head_runs + q0 + u) * 1024, 0));
+#pragma unroll
+                    for (int s4 = 0; s4 < 4; ++s4)
+                        hb[u][s4] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                            in_rsrc, (int)(pix + (unsigned)(16 * (q0 + u) + s4) * chan_bytes), 0, 0));
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u)
+#pragma unroll
+                    for (int s4 = 0; s4 < 4; ++s4) {
+                        if (s4 & 1) h1 = __builtin_amdgcn_mfma_f32_16x16x4f32(ha[u][s4], hb[u][s4], h1, 0, 0, 0);
+                        else h0 = __builtin_amdgcn_mfma_f32_16x16x4f32(ha[u][s4], hb[u][s4], h0, 0, 0, 0);
+                    }
+            }
+            const f4_t h = h0 + h1;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) F[(cb * 16 + 4 * k + i) * p.head_ld + wq] = h[i];
+        }
+        __syncthreads();
+        // the core's pixel operand comes from that window: output pixel (jy, jx), tap (r, c) = window pixel (jy + r, jx + c)
+        const float *Fk = F + (wki * (4 * CG) + k) * p.head_ld;
+        const int wmax = p.head_npb * 16 - 1;
+#pragma unroll
+        for (int g = 0; g < CG; ++g)
+#pragma unroll
+            for (int t = 0; t < 9; ++t)
+                b[g][t] = Fk[4 * g * p.head_ld + min((jy + t / 3) * p.head_ww + jx + t % 3, wmax)];
+    } else
     if constexpr (ROW) {
         // lane n of a quarter: input column (tile's first column - pad + n) of the three input rows
         const int iyr = tile_y - p.pad, ixr = tile_x * 14 - p.pad + n;
@@ -1513,6 +1569,12 @@ static kernel_fn pick_stream3(int groups) {
         case 4: return tdc_conv3x3_stream_kernel<4, ROW, MODE>;
         default: return nullptr;
     }
+}
+
+// The streamed 3x3 kernel with a fused 1x1 head and tail (a whole Tucker convolution), for a tile.alg = 4 tile.
+const void *conv_kernel_with_head(const tdc_tile &t) {
+    if (t.alg != 4 || t.ks != 1 || t.cch % (4 * t.wk) != 0) return nullptr;
+    return reinterpret_cast<const void *>(pick_stream3<false, 3>(t.cch / (4 * t.wk)));
 }
 
 const void *conv_kernel_for(const tdc_tile &t, int KH, int KW, int dilation, int stride, bool extras) {

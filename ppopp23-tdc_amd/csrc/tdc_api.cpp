@@ -55,6 +55,9 @@ struct tdc_conv_plan {
     int tail_N = 0;               // fused 1x1 tail (0 = none): outputs, epilogue flags, packed weights
     int tail_has_bias = 0, tail_relu = 0;
     float *d_tail_w = nullptr, *d_tail_bias = nullptr;
+    int head_C = 0;               // fused 1x1 head (0 = none): its input channels, packed weights, LDS layout
+    float *d_head_w = nullptr;
+    int head_runs = 0, head_mblk = 0, head_npb = 0, head_ww = 0, head_wq = 0, head_ld = 0, head_f_off = 0;
     bool have_tail_weights = false;
     int in_relu = 0;
     bool have_weights = false;
@@ -68,6 +71,8 @@ static void free_plan_buffers(tdc_conv_plan *p) {
     if (p->d_in_aff) (void)hipFree(p->d_in_aff);
     if (p->d_tail_w) (void)hipFree(p->d_tail_w);
     if (p->d_tail_bias) (void)hipFree(p->d_tail_bias);
+    if (p->d_head_w) (void)hipFree(p->d_head_w);
+    p->d_head_w = nullptr;
     p->d_in_aff = p->d_tail_w = p->d_tail_bias = nullptr;
     p->d_wpk = p->d_bias = p->d_ws = nullptr;
     p->d_ctr = nullptr;
@@ -79,6 +84,7 @@ struct tdc_tkconv {
     tdc_conv_plan *core = nullptr;
     tdc_conv_plan *last = nullptr;
     tdc_conv_plan *core_last = nullptr;   // core convolution with the last factor fused behind it, when that is faster
+    tdc_conv_plan *whole = nullptr;       // first factor + core + last factor in one launch, when that is faster still
     float *d_f1 = nullptr;  // [batch, R1, H, W]
     float *d_f2 = nullptr;  // [batch, R2, Ho, Wo]
     size_t f1_floats = 0, f2_floats = 0;
@@ -418,6 +424,49 @@ int tdc_conv_plan_set_input_affine(tdc_conv_plan *plan, const float *scale, cons
     return TDC_OK;
 }
 
+int tdc_conv_plan_set_head(tdc_conv_plan *plan, int32_t head_C, const float *w_head) {
+    if (!plan || !w_head) return fail(TDC_ERR_INVALID, "null argument");
+    if (head_C < 1) return fail(TDC_ERR_INVALID, "head_C must be >= 1");
+    const tdc_conv_desc &d = plan->desc;
+    const tdc_tile &t = plan->tile;
+    Geometry &g = plan->geo;
+    if (t.alg != 4 || plan->tail_N <= 0 || d.KH != 3 || d.KW != 3 || d.stride != 1 || d.dilation != 1)
+        return fail(TDC_ERR_UNSUPPORTED, "a fused head needs a streamed 3x3 / stride 1 plan (tile.alg = 4) with a fused tail");
+    if (plan->d_in_aff) return fail(TDC_ERR_UNSUPPORTED, "a fused head cannot be combined with an input affine");
+    if ((long long)head_C * d.H * d.W * 4 >= (1LL << 31)) return fail(TDC_ERR_UNSUPPORTED, "image too large for a fused head");
+    const void *kernel = conv_kernel_with_head(t);
+    if (!kernel) return fail(TDC_ERR_UNSUPPORTED, "no kernel instantiated for this tile");
+    const int runs = ((head_C + 15) / 16 + 3) / 4 * 4;   // the kernel requests four runs at a time
+    const int mblk = (t.cch + 15) / 16;                   // every input channel row of the core, padding included
+    const int ww = g.TW + 2, wq = (g.TH + 2) * ww, npb = (wq + 15) / 16;
+    int ld = npb * 16;
+    if (ld % 32 == 0) ld += 16;                           // the four channel quarters of a K-step in different banks
+    const int f_off = g.tail_f_off + g.MT * g.tail_ld;
+    const long long lds = ((long long)f_off + (long long)mblk * 16 * ld) * 4;
+    if (lds > machine().lds_bytes_per_cu) return fail(TDC_ERR_UNSUPPORTED, "the window of the fused head does not fit the LDS");
+    // [16-row block][run][lane][4]: lane l (row l % 16, quarter l / 16) holds w_head[block*16 + l%16][16*run + 4*(l/16) + e]
+    std::vector<float> packed((size_t)mblk * runs * 256, 0.0f);
+    for (int cb = 0; cb < mblk; ++cb)
+        for (int r = 0; r < runs; ++r)
+            for (int l = 0; l < 64; ++l)
+                for (int e = 0; e < 4; ++e) {
+                    const int n = cb * 16 + l % 16, c = 16 * r + 4 * (l / 16) + e;
+                    if (n < d.C && c < head_C) packed[(((size_t)cb * runs + r) * 64 + l) * 4 + e] = w_head[(size_t)n * head_C + c];
+                }
+    if (plan->d_head_w) (void)hipFree(plan->d_head_w);
+    plan->d_head_w = nullptr;
+    hipError_t e = hipMalloc((void **)&plan->d_head_w, packed.size() * sizeof(float));
+    if (e == hipSuccess) e = hipMemcpy(plan->d_head_w, packed.data(), packed.size() * sizeof(float), hipMemcpyHostToDevice);
+    if (e != hipSuccess) return hip_fail("fused head upload", e);
+    g.lds_bytes = std::max(g.lds_bytes, (int)lds);
+    plan->info.lds_bytes = g.lds_bytes;
+    plan->kernel = kernel;
+    if (int he = prepare_conv_kernel(plan->kernel, g)) return hip_fail("hipFuncSetAttribute(MaxDynamicSharedMemorySize)", he);
+    plan->head_C = head_C; plan->head_runs = runs; plan->head_mblk = mblk; plan->head_npb = npb;
+    plan->head_ww = ww; plan->head_wq = wq; plan->head_ld = ld; plan->head_f_off = f_off;
+    return TDC_OK;
+}
+
 int tdc_conv_plan_query(const tdc_conv_plan *plan, tdc_tile_info *info_out) {
     if (!plan || !info_out) return fail(TDC_ERR_INVALID, "null argument");
     *info_out = plan->info;
@@ -438,7 +487,7 @@ int tdc_conv_forward_strided(tdc_conv_plan *plan, const float *d_in, int64_t in_
         return fail(TDC_ERR_STATE, "tdc_conv_forward before tdc_conv_plan_set_tail_weights");
     const tdc_conv_desc &d = plan->desc;
     const Geometry &g = plan->geo;
-    const long long in_image = (long long)d.C * d.H * d.W;
+    const long long in_image = (long long)(plan->head_C > 0 ? plan->head_C : d.C) * d.H * d.W;
     const long long out_image = (long long)(plan->tail_N > 0 ? plan->tail_N : d.N) * g.P;
     if ((in_batch_stride && in_batch_stride < in_image) || (out_batch_stride && out_batch_stride < out_image) ||
         (residual_batch_stride && residual_batch_stride < out_image))
@@ -455,6 +504,11 @@ int tdc_conv_forward_strided(tdc_conv_plan *plan, const float *d_in, int64_t in_
     kp.tail_bias = plan->d_tail_bias;
     kp.tail_N = plan->tail_N; kp.tail_mblk = (plan->tail_N + 15) / 16; kp.tail_ng = g.tail_ng; kp.tail_relu = plan->tail_relu;
     kp.tail_ld = g.tail_ld; kp.tail_f_off = g.tail_f_off;
+    kp.head_w = plan->d_head_w;
+    kp.head_C = plan->head_C; kp.head_runs = plan->head_runs; kp.head_mblk = plan->head_mblk; kp.head_npb = plan->head_npb;
+    kp.head_ww = plan->head_ww; kp.head_wq = plan->head_wq; kp.head_ld = plan->head_ld; kp.head_f_off = plan->head_f_off;
+    kp.fd_hww = make_fastdiv(std::max(plan->head_ww, 1));
+    kp.fd_hnpb = make_fastdiv(std::max(plan->head_npb, 1));
     kp.fd_npx = make_fastdiv(g.PT / 16);
     kp.in_relu = plan->in_relu;
     kp.ctr = plan->d_ctr;
@@ -676,6 +730,69 @@ static int tkconv_measure_fusion(tdc_tkconv *op) {
     return TDC_OK;
 }
 
+// One launch for the whole operator, or the first factor on its own in front of core + last?  Timed as dependent
+// chains on the operator's own intermediates (synthetic weights); remembered per problem.
+static std::map<std::array<int, 13>, bool> g_whole_pays;
+
+static int tkconv_measure_whole(tdc_tkconv *op) {
+    const tdc_tkconv_desc &d = op->desc;
+    const std::array<int, 13> key{d.batch, d.C, d.R1, d.R2, d.N, d.H, d.W, d.K, d.stride, d.pad, d.dilation, d.has_bias, d.relu};
+    bool known = false, pays = false;
+    {
+        std::lock_guard<std::mutex> lock(g_tune_mutex);
+        auto hit = g_whole_pays.find(key);
+        if (hit != g_whole_pays.end()) {
+            known = true;
+            pays = hit->second;
+        }
+    }
+    if (!known) {
+        const size_t in_floats = (size_t)d.batch * d.C * d.H * d.W;
+        const size_t out_floats = (size_t)d.batch * d.N * (op->f2_floats / ((size_t)d.batch * d.R2));
+        float *d_in = nullptr, *d_out = nullptr;
+        hipError_t e = hipMalloc((void **)&d_in, in_floats * sizeof(float));
+        if (e == hipSuccess) e = hipMalloc((void **)&d_out, out_floats * sizeof(float));
+        if (e == hipSuccess) e = hipMemset(d_in, 0x3c, in_floats * sizeof(float));
+        if (e != hipSuccess) {
+            if (d_in) (void)hipFree(d_in);
+            if (d_out) (void)hipFree(d_out);
+            return hip_fail("hipMalloc(fusion timing)", e);
+        }
+        int st = synthetic_weights(op->first, true);
+        if (st == TDC_OK) st = synthetic_weights(op->core_last, true);
+        if (st == TDC_OK) st = synthetic_weights(op->whole, true);
+        tdc_conv_plan *two[2] = {op->first, op->core_last};
+        const float *ins[2] = {d_in, op->d_f1};
+        float *outs[2] = {op->d_f1, d_out};
+        tdc_conv_plan *one[1] = {op->whole};
+        double us_two = 1e30, us_one = 1e30;
+        for (int rep = 0; rep < 4 && st == TDC_OK; ++rep) {   // the first repetition warms up
+            float ms = 0.0f;
+            st = time_plans(two, ins, outs, 2, 10, 2, 1, &ms);
+            if (st == TDC_OK && rep > 0) us_two = std::min(us_two, (double)ms * 1e3 / 20);
+            if (st == TDC_OK) st = time_plans(one, ins, outs + 1, 1, 10, 2, 1, &ms);
+            if (st == TDC_OK && rep > 0) us_one = std::min(us_one, (double)ms * 1e3 / 20);
+        }
+        (void)hipFree(d_in);
+        (void)hipFree(d_out);
+        synthetic_weights(op->first, false);
+        synthetic_weights(op->core_last, false);
+        synthetic_weights(op->whole, false);
+        if (st != TDC_OK) return st;
+        pays = us_one < 0.97 * us_two;
+        if (log_tuning())
+            std::fprintf(stderr, "tdc tune: tkconv C%d R%d,%d N%d %dx%d K%d s%d: one launch %.2f us, first + core+last %.2f us\n",
+                         d.C, d.R1, d.R2, d.N, d.H, d.W, d.K, d.stride, us_one, us_two);
+        std::lock_guard<std::mutex> lock(g_tune_mutex);
+        g_whole_pays[key] = pays;
+    }
+    if (!pays) {
+        tdc_conv_plan_destroy(op->whole);
+        op->whole = nullptr;
+    }
+    return TDC_OK;
+}
+
 int tdc_tkconv_create(const tdc_tkconv_desc *desc, tdc_tkconv **op_out) {
     if (!desc || !op_out) return fail(TDC_ERR_INVALID, "null argument");
     *op_out = nullptr;
@@ -699,6 +816,7 @@ int tdc_tkconv_create(const tdc_tkconv_desc *desc, tdc_tkconv **op_out) {
         tdc_conv_plan_destroy(op->core);
         tdc_conv_plan_destroy(op->last);
         tdc_conv_plan_destroy(op->core_last);
+        tdc_conv_plan_destroy(op->whole);
         if (op->d_f1) (void)hipFree(op->d_f1);
         if (op->d_f2) (void)hipFree(op->d_f2);
     };
@@ -725,6 +843,25 @@ int tdc_tkconv_create(const tdc_tkconv_desc *desc, tdc_tkconv **op_out) {
             if (st != TDC_OK) { cleanup(); return st; }
             if (measure && (st = tkconv_measure_fusion(op.get())) != TDC_OK) { cleanup(); return st; }
         }
+        // The first factor too, recomputed per workgroup on its window (streamed 3x3 kernel, stride 1).  Every
+        // workgroup then pulls the whole first factor through its compute unit, so this only pays while that factor is
+        // small: without measurement, up to 16 KiB of its weights and 64 input channels.
+        if (op->core_last && op->core_last->tile.alg == 4 && desc->K == 3 && desc->stride == 1 && desc->dilation == 1 &&
+            !std::getenv("TDC_EXPERIMENT_NO_FUSED_HEAD") &&
+            (measure ? (long long)desc->C * desc->R1 <= 32768 : ((long long)desc->C * desc->R1 <= 4096 && desc->C <= 64))) {
+            st = tdc_conv_plan_create_with_tail(&d2, desc->N, desc->has_bias, desc->relu, &op->core_last->tile, &op->whole);
+            if (st == TDC_OK) {
+                const std::vector<float> zeros((size_t)desc->R1 * desc->C, 0.0f);
+                st = tdc_conv_plan_set_head(op->whole, desc->C, zeros.data());
+                if (st == TDC_ERR_UNSUPPORTED) {
+                    tdc_conv_plan_destroy(op->whole);
+                    op->whole = nullptr;
+                    st = TDC_OK;
+                }
+            }
+            if (st != TDC_OK) { cleanup(); return st; }
+            if (op->whole && measure && (st = tkconv_measure_whole(op.get())) != TDC_OK) { cleanup(); return st; }
+        }
     }
     *op_out = op.release();
     return TDC_OK;
@@ -741,6 +878,11 @@ int tdc_tkconv_set_weights(tdc_tkconv *op, const float *first, const float *core
         if ((st = tdc_conv_plan_set_weights(op->core_last, core, nullptr)) != TDC_OK) return st;
         if ((st = tdc_conv_plan_set_tail_weights(op->core_last, last, bias)) != TDC_OK) return st;
     }
+    if (op->whole) {
+        if ((st = tdc_conv_plan_set_weights(op->whole, core, nullptr)) != TDC_OK) return st;
+        if ((st = tdc_conv_plan_set_tail_weights(op->whole, last, bias)) != TDC_OK) return st;
+        if ((st = tdc_conv_plan_set_head(op->whole, op->desc.C, first)) != TDC_OK) return st;
+    }
     return TDC_OK;
 }
 
@@ -752,7 +894,7 @@ static int tkconv_forward_unfused(tdc_tkconv *op, const float *d_in, int64_t in_
     return tdc_conv_forward_strided(op->last, op->d_f2, 0, d_residual, residual_batch_stride, d_out, out_batch_stride, stream);
 }
 
-int tdc_tkconv_num_kernels(const tdc_tkconv *op) { return op ? (op->core_last ? 2 : 3) : 0; }
+int tdc_tkconv_num_kernels(const tdc_tkconv *op) { return op ? (op->whole ? 1 : op->core_last ? 2 : 3) : 0; }
 
 int tdc_tkconv_forward(tdc_tkconv *op, const float *d_in, const float *d_residual, float *d_out, void *stream) {
     return tdc_tkconv_forward_strided(op, d_in, 0, d_residual, 0, d_out, 0, stream);
@@ -764,6 +906,9 @@ int tdc_tkconv_forward_strided(tdc_tkconv *op, const float *d_in, int64_t in_bat
     if (!op->core_last)
         return tkconv_forward_unfused(op, d_in, in_batch_stride, d_residual, residual_batch_stride, d_out, out_batch_stride,
                                       stream);
+    if (op->whole)
+        return tdc_conv_forward_strided(op->whole, d_in, in_batch_stride, d_residual, residual_batch_stride, d_out,
+                                        out_batch_stride, stream);
     int st;
     if ((st = tdc_conv_forward_strided(op->first, d_in, in_batch_stride, nullptr, 0, op->d_f1, 0, stream)) != TDC_OK) return st;
     return tdc_conv_forward_strided(op->core_last, op->d_f1, 0, d_residual, residual_batch_stride, d_out, out_batch_stride,
@@ -807,6 +952,7 @@ void tdc_tkconv_destroy(tdc_tkconv *op) {
     tdc_conv_plan_destroy(op->core);
     tdc_conv_plan_destroy(op->last);
     tdc_conv_plan_destroy(op->core_last);
+    tdc_conv_plan_destroy(op->whole);
     if (op->d_f1) (void)hipFree(op->d_f1);
     if (op->d_f2) (void)hipFree(op->d_f2);
     delete op;

@@ -109,6 +109,7 @@ struct ConvKParams {
     const float *in_aff;       // optional per-input-channel affine in front of a 1x1 convolution: [pass][scale(CCH) | shift(CCH)]
     const float *tail_w;       // fused 1x1 tail: packed weights [16-row block][K-step][64 lanes], or null
     const float *tail_bias;
+    const float *head_w;       // fused 1x1 head (first factor in front of a streamed 3x3 core): packed [16-row block][run of 16 channels][lane][4]
     float *out;
     float *ws;                 // partial tiles of a split across workgroups: [image][slice][N][P]
     unsigned *ctr;             // one ticket counter per (image, channel tile, pixel tile), zero between launches
@@ -130,6 +131,11 @@ struct ConvKParams {
     int in_relu;               // ReLU after the input affine
     int tail_N, tail_mblk, tail_ng, tail_relu;   // tail outputs, their 16-row blocks, K-steps (ceil(N/4)), ReLU after it
     int tail_ld, tail_f_off;   // row stride and offset (floats) of the parked tile in LDS
+    int head_C, head_runs;     // fused head: its input channels, runs of 16 of them (rounded up to a multiple of 4)
+    int head_mblk, head_npb;   // ... 16-row blocks of its output (the core's input channels), 16-pixel blocks of the window
+    int head_ww, head_wq;      // ... window width (TW + 2) and pixels ((TH + 2) * (TW + 2))
+    int head_ld, head_f_off;   // ... row stride and offset (floats) of its output in LDS
+    FastDiv fd_hww, fd_hnpb;
     FastDiv fd_npx;            // 16-pixel blocks per tile
     FastDiv fd_csv, fd_rsv;      // LDS channel slot / row, in copy elements
     FastDiv fd_tw, fd_ntx, fd_pt;
@@ -145,6 +151,7 @@ struct ConvKParams {
 // The instantiated kernel for a tile and filter size (nullptr if none).
 // `extras`: the instantiation that also carries the input affine and the fused 1x1 tail.
 const void *conv_kernel_for(const tdc_tile &t, int KH, int KW, int dilation, int stride, bool extras);
+const void *conv_kernel_with_head(const tdc_tile &t);
 // One-time per-plan attribute setup (dynamic LDS above 64 KiB).  hipError_t as int.
 int prepare_conv_kernel(const void *fn, const Geometry &g);
 // Enqueue the kernel.  Returns a hipError_t as int.

@@ -18,7 +18,7 @@ TDC_OK, TDC_ERR_INVALID, TDC_ERR_UNSUPPORTED, TDC_ERR_HIP, TDC_ERR_NOMEM, TDC_ER
 EXPORTS = (
     "tdc_last_error_string", "tdc_version", "tdc_load_bin", "tdc_save_bin",
     "tdc_conv_plan_create", "tdc_conv_plan_create_with_tail", "tdc_conv_plan_set_tail_weights",
-    "tdc_conv_plan_set_weights", "tdc_conv_plan_set_input_affine", "tdc_conv_plan_query",
+    "tdc_conv_plan_set_weights", "tdc_conv_plan_set_input_affine", "tdc_conv_plan_set_head", "tdc_conv_plan_query",
     "tdc_conv_forward",
     "tdc_conv_forward_strided", "tdc_tkconv_forward_strided",
     "tdc_conv_time", "tdc_conv_time_many", "tdc_conv_plan_destroy",

@@ -77,6 +77,16 @@ class Conv2dPlan:
                                                    c_void_p(b.data_ptr()) if b is not None else None))
         return self
 
+    def set_head(self, weight):
+        """Fuse a 1x1 convolution [C, head_C] (or [C, head_C, 1, 1]) in front of a streamed 3x3 plan with a fused tail:
+        with the tail, a whole TKConv in one launch.  The plan's input then has head_C channels."""
+        w = _host_f32(weight)
+        if w.dim() not in (2, 4) or w.shape[0] != self.desc.C or w.numel() != w.shape[0] * w.shape[1]:
+            raise ValueError("head weight must be [C, head_C]")
+        check(lib().tdc_conv_plan_set_head(self._h, int(w.shape[1]), c_void_p(w.data_ptr())))
+        self.head_C = int(w.shape[1])
+        return self
+
     def set_input_affine(self, scale, shift, relu=True):
         """y = conv(relu?(x * scale[c] + shift[c])) in one kernel (1x1 convolutions without padding only)."""
         sc, sh = _host_f32(scale), _host_f32(shift)
@@ -87,7 +97,7 @@ class Conv2dPlan:
 
     def forward(self, x, residual=None, out=None):
         d = self.desc
-        _dev_check(x, (d.batch, d.C, d.H, d.W), "input")
+        _dev_check(x, (d.batch, getattr(self, "head_C", None) or d.C, d.H, d.W), "input")
         oshape = (d.batch, self.tail[0] if self.tail else d.N, self.Ho, self.Wo)
         if out is None:
             out = torch.empty(oshape, device=x.device, dtype=torch.float32)
@@ -193,6 +203,11 @@ class TKConvOp:
             out = torch.empty((d.batch, d.R2, self.Ho, self.Wo), device=x.device, dtype=torch.float32)
         check(lib().tdc_tkconv_core_forward(self._h, c_void_p(x.data_ptr()), c_void_p(out.data_ptr()), _stream_ptr()))
         return out
+
+    @property
+    def num_kernels(self):
+        """Launches per forward: 3, 2 (core + last factor fused) or 1 (the first factor fused in front as well)."""
+        return int(lib().tdc_tkconv_num_kernels(self._h))
 
     def query(self, which):
         info = TileInfo()

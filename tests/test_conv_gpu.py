@@ -597,6 +597,61 @@ def test_fused_tail_on_streamed_3x3(shape):
         assert_close(out.cpu().numpy(), want, f"streamed fused tail {shape} {t}")
 
 
+@pytest.mark.parametrize("shape", [(1, 40, 24, 16, 40, 9, 9), (2, 100, 40, 10, 33, 14, 14), (1, 128, 64, 16, 32, 14, 14),
+                                   (1, 128, 64, 16, 32, 7, 7), (1, 64, 32, 32, 64, 28, 28), (1, 300, 64, 64, 70, 13, 11),
+                                   (3, 5, 3, 4, 6, 4, 3), (1, 128, 64, 64, 128, 56, 56)])
+def test_fused_head_and_tail_on_streamed_3x3(shape):
+    """A whole Tucker convolution in one launch: 1x1 head (no bias) -> 3x3 core (pad 1, + bias, ReLU) -> 1x1 tail
+    (+ bias, + residual, ReLU) on the streamed 3x3 kernel.  The head is recomputed on every tile's window, where pixels
+    outside the image must read as the core's zero padding; ragged channel counts, every tile shape, batches."""
+    B, C0, C, N, N2, H, W = shape
+    g = seeded(9800 + C0 + N2)
+    x = torch.rand(B, C0, H, W, generator=g) * 2 - 1
+    w0 = torch.randn(C, C0, 1, 1, generator=g) / math.sqrt(C0)
+    w = torch.randn(N, C, 3, 3, generator=g) * math.sqrt(2.0 / (9 * C))
+    b1 = torch.randn(N, generator=g) * 0.5
+    w2 = torch.randn(N2, N, 1, 1, generator=g) / math.sqrt(N)
+    b2 = torch.randn(N2, generator=g)
+    resid = torch.randn(B, N2, H, W, generator=g)
+    f1 = ref.conv2d_c(x.numpy(), w0.numpy())
+    mid = ref.conv2d_c(f1, w.numpy(), b1.numpy(), pad=1, relu=True)
+    want = ref.conv2d_c(mid, w2.numpy(), b2.numpy(), resid.numpy(), relu=True)
+    wm, groups = -(-N // 16), -(-C // 4)
+    tiles = []
+    for per_wave in (4, 2, 1):
+        wk = -(-groups // per_wave)
+        if per_wave <= groups and wm * wk <= 16:
+            for tw in sorted({min(16, W), min(14, W), min(7, W), min(4, W)}):
+                tiles.append(tdc_amd.Tile(16, 1, 1, wm, 1, wk, 4 * per_wave * wk, tw, 1, 0, 4))
+    assert tiles
+    xd, rd = x.cuda(), resid.cuda()
+    for t in tiles:
+        announce("streamed head + tail", shape, t)
+        plan = tdc_amd.Conv2dPlan(B, C, N, H, W, 3, 3, 1, 1, 1, True, True, tile=t, tail=(N2, True, True))
+        plan.set_weights(w, b1).set_tail_weights(w2, b2).set_head(w0)
+        outs = []
+        for rep in range(2):
+            out = torch.full((B, N2, H, W), float("nan"), device="cuda")
+            plan.forward(xd, rd, out=out)
+            torch.cuda.synchronize()
+            outs.append(out.cpu().numpy())
+        plan.close()
+        assert_close(outs[0], want, f"streamed fused head + tail {shape} {t}")
+        assert np.array_equal(outs[0], outs[1])
+
+
+def test_fused_head_is_refused_where_it_does_not_apply():
+    plan = tdc_amd.Conv2dPlan(1, 8, 16, 9, 9, 3, 3, 1, 1, tile=tdc_amd.Tile(16, 1, 1, 1, 1, 2, 8, 9, 1, 0, 4)).set_weights(torch.randn(16, 8, 3, 3))
+    with pytest.raises(tdc_amd.TdcError) as e:   # no fused tail
+        plan.set_head(torch.randn(8, 20))
+    assert e.value.status == tdc_amd._lib.TDC_ERR_UNSUPPORTED
+    plan.close()
+    plan = tdc_amd.Conv2dPlan(1, 8, 16, 9, 9, 3, 3, 2, 1, tile=tdc_amd.Tile(16, 1, 1, 1, 1, 2, 8, 5, 1, 0, 4), tail=(8, False, False))
+    with pytest.raises(tdc_amd.TdcError):        # stride 2
+        plan.set_head(torch.randn(8, 20))
+    plan.close()
+
+
 def test_fused_tail_needs_one_channel_tile():
     with pytest.raises(tdc_amd.TdcError):   # 40 output channels cannot sit in a 16-channel tile
         tdc_amd.Conv2dPlan(1, 8, 40, 9, 9, 3, 3, 1, 1, tile=tdc_amd.Tile(16, 1, 1, 1, 1, 1, 8, 8), tail=(8, False, False))

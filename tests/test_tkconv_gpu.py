@@ -57,6 +57,38 @@ def test_block_against_c_oracle_small():
         op.close()
 
 
+@pytest.mark.parametrize("shape", [(1, 32, 16, 16, 32, 14, 14), (2, 64, 32, 32, 64, 28, 28), (1, 64, 32, 32, 64, 56, 56), (3, 20, 6, 10, 14, 9, 11)])
+@pytest.mark.parametrize("measured", [False, True])
+def test_whole_operator_in_one_launch(shape, measured):
+    """Small first factors are fused in front of core + last factor (one launch per TKConv): same answer as the
+    oracle's three convolutions with bias, residual and ReLU on the last one, whether the choice is the model's or
+    measured, and the feature maps of forward_features still come from the three separate plans."""
+    B, C, R1, R2, N, H, W = shape
+    g = seeded(880 + C + H)
+    x = torch.rand(B, C, H, W, generator=g) * 2 - 1
+    first = torch.randn(R1, C, 1, 1, generator=g) / C ** 0.5
+    core = torch.randn(R2, R1, 3, 3, generator=g) * (2.0 / (9 * R1)) ** 0.5
+    last = torch.randn(N, R2, 1, 1, generator=g) / R2 ** 0.5
+    bias = torch.randn(N, generator=g)
+    resid = torch.randn(B, N, H, W, generator=g)
+    want, f1, f2 = ref.tkconv_c(x.numpy(), first.numpy(), core.numpy(), last.numpy(), bias.numpy(), 1, 1, 1)
+    want = np.maximum(want + resid.numpy(), 0.0)
+    prev = tdc_amd.set_autotune(4 if measured else 0)
+    try:
+        op = tdc_amd.TKConvOp(B, C, R1, R2, N, H, W, 3, 1, 1, 1, bias=True, relu=True).set_weights(first, core, last, bias)
+    finally:
+        tdc_amd.set_autotune(prev)
+    announce("whole TKConv", shape, "measured" if measured else "model", "kernels", op.num_kernels)
+    if not measured:
+        assert op.num_kernels == 1
+    got = op.forward(x.cuda(), resid.cuda()).cpu().numpy()
+    assert_close(got, want, f"one-launch TKConv {shape}")
+    _, feats = op.forward_features(x.cuda())
+    assert_close(feats[0].cpu().numpy(), f1, "first feature")
+    assert_close(feats[1].cpu().numpy(), f2, "core feature")
+    op.close()
+
+
 def test_module_forward_matches_reference_forward():
     """TKConv2dC.forward(x) == F.conv2d(F.conv2d(F.conv2d(x, first), core, None, stride, padding, dilation), last, bias)."""
     torch.manual_seed(5)
