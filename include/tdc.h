@@ -211,8 +211,10 @@ int tdc_tkconv_forward_features(tdc_tkconv *op, const float *d_in, float *d_feat
                                 float *d_feat_core, float *d_out, void *stream);
 /* Only the KxK core conv: d_in is [batch,R1,H,W], d_out [batch,R2,Ho,Wo]. */
 int tdc_tkconv_core_forward(tdc_tkconv *op, const float *d_in, float *d_out, void *stream);
-/* Launches per forward: 3, or 2 when the last factor is fused behind the core convolution (done automatically
- * when the tile model predicts it faster; TDC_EXPERIMENT_NO_FUSED_TAIL in the environment turns it off). */
+/* Launches per forward: 3; 2 when the last factor is fused behind the core convolution (done automatically
+ * when the tile model predicts it faster; TDC_EXPERIMENT_NO_FUSED_TAIL in the environment turns it off); 1 when the
+ * first factor is fused in front as well (small first factors on 3x3 / stride 1 cores, see tdc_conv_plan_set_head;
+ * TDC_EXPERIMENT_NO_FUSED_HEAD turns it off). */
 int tdc_tkconv_num_kernels(const tdc_tkconv *op);
 /* which: 0 = first 1x1, 1 = core, 2 = last 1x1 */
 int tdc_tkconv_query(const tdc_tkconv *op, int which, tdc_tile_info *info_out);
