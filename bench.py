@@ -305,11 +305,13 @@ def main():
                 sys.exit("bench.py: Tucker block parity check failed (max err %g)" % berr)
             bnet.time_ms(iters=20)
             us = min(bnet.time_ms(iters=200) for _ in range(3)) * 1e3
+            us_stream = min(bnet.time_ms(iters=200, graph=False) for _ in range(3)) * 1e3   # the same launches, not from a graph
             flops = 2.0 * hw * hw * (C * R1 + 9 * R1 * R2 + R2 * N)
             nbytes = 4.0 * (hw * hw * (C + N) + C * R1 + 9 * R1 * R2 + R2 * N)
             roof = max(nbytes / 8e6, flops / 157.3e6)
             blocks.append({"C": C, "R1": R1, "R2": R2, "N": N, "H": hw, "us": round(us, 3), "roof_us": round(roof, 3),
-                           "frac": round(roof / us, 4), "kernels": bnet.num_kernels})
+                           "frac": round(roof / min(us, us_stream), 4), "kernels": bnet.num_kernels,
+                           "us_stream_launches": round(us_stream, 3)})   # us: one graph replay per block (a replay costs ~5 us by itself)
             bnet.close()
         out["tucker_blocks_b1"] = blocks
 
