@@ -157,6 +157,22 @@ int tdc_conv_plan_set_input_affine(tdc_conv_plan *plan, const float *scale, cons
    input channels); from then on the plan's input has head_C channels.  TDC_ERR_UNSUPPORTED for other plans. */
 int tdc_conv_plan_set_head(tdc_conv_plan *plan, int32_t head_C, const float *w_head);
 int tdc_conv_plan_query(const tdc_conv_plan *plan, tdc_tile_info *info_out);
+/* Occupancy probe: what the COMPILED kernel of this plan uses and how many of its workgroups the runtime places on one
+ * compute unit (hipFuncGetAttributes, hipOccupancyMaxActiveBlocksPerMultiprocessor), next to what the analytic model
+ * assumed for the same tile.  The counterpart of the reference's per-candidate occupancy measurement
+ * (2080Ti-evaluation/Gen-occupancy/template.cu:277-284: cudaOccupancyMaxActiveBlocksPerMultiprocessor for every
+ * (TH, TW, TC) kernel).  Needs the device; launches nothing. */
+typedef struct tdc_kernel_occupancy {
+    int32_t kernel_vgprs;            /* registers per lane of the compiled kernel (arch + acc)          */
+    int32_t kernel_static_lds_bytes;
+    int32_t kernel_max_threads;      /* its launch bound                                                 */
+    int32_t runtime_wg_per_cu;       /* resident workgroups per CU for this plan's block size and LDS    */
+    int32_t block_threads;
+    int32_t dynamic_lds_bytes;
+    int32_t model_vgprs;             /* tdc_tile_info.vgpr_estimate of the plan                          */
+    int32_t model_wg_per_cu;         /* tdc_tile_info.wg_per_cu of the plan                              */
+} tdc_kernel_occupancy;
+int tdc_conv_plan_occupancy(const tdc_conv_plan *plan, tdc_kernel_occupancy *out);
 /* d_residual may be NULL.  Output need not be pre-zeroed.  Asynchronous. */
 int tdc_conv_forward(tdc_conv_plan *plan, const float *d_in, const float *d_residual,
                      float *d_out, void *stream);
@@ -301,6 +317,14 @@ int tdc_model_select(const tdc_conv_desc *desc, tdc_tile_info *info_out);
  * desc->N channels in one workgroup only); fails if there is none.  Compare pred_us with the sum of the two
  * separate convolutions to decide whether the fusion pays. */
 int tdc_model_select_with_tail(const tdc_conv_desc *desc, int32_t tail_N, tdc_tile_info *info_out);
+/* Which compiled kernel serves `tile` for this convolution (`extras` != 0: the instantiation that also carries the
+ * input affine / fused 1x1 tail), by the name the compiler's resource report and the profiler print, e.g.
+ * "tdc_conv_mfma_kernel<16, 1, 1, 9, 16, false>", and the registers per lane the model's occupancy term assumes for
+ * it (the compiled count rounded up to the allocation granule of 8) and the waves of it that fit one SIMD (vector
+ * and scalar register limits, at most 8).  Host only; any output pointer may be NULL.  With tdc_conv_plan_occupancy
+ * this replaces the reference's occupancy probe (2080Ti-evaluation/Gen-occupancy/template.cu:277-284). */
+int tdc_model_kernel_info(const tdc_conv_desc *desc, const tdc_tile *tile, int32_t extras, char *name_out, int32_t cap,
+                          int32_t *vgprs_out, int32_t *waves_per_simd_out);
 /* Calibration constants of the latency model (launch floor, copy latency and rate, barrier cost, ...;
  * the counterpart of num_sm / num_threads / a,b,c / ratio in the reference's model.py:265-266,278).
  * get: writes up to `cap` values, *count_out = how many there are.  set: all of them, all > 0;

@@ -47,6 +47,8 @@
 //   * bias, residual add and ReLU are fused into the store.
 #include <hip/hip_runtime.h>
 
+#include <mutex>
+
 #include "tdc_internal.hpp"
 
 #ifndef TDC_TOUCH_KERNARGS
@@ -102,7 +104,7 @@ struct Mfma<16> {
 // every lane holds all 16 positions of its tile) into the 2x2 outputs.
 // TAPS_3x3G: the direct 3x3 loop with its weights read from global memory straight into registers (like the
 // Winograd path) instead of being staged in LDS: the LDS then holds input only and a pass can take all input channels.
-enum : int { TAPS_GENERIC = 0, TAPS_1x1 = 1, TAPS_3x3 = 9, TAPS_3x3G = 10, TAPS_WINO = 16 };
+// (the TAPS_* values themselves are declared next to KernelId)
 
 constexpr int OOB_OFFSET = 0x7ffffff0;  // beyond any buffer: the load returns zero
 
@@ -1237,34 +1239,6 @@ __global__ void __launch_bounds__(NQ == 8 ? 512 : 1024) tdc_conv1x1_stream_kerne
 }
 
 // ---------------------------------------------------------------------------
-// Instantiation table.  A 2x2 block grid of MFMAs per wave is built for at
-// most 8 waves per workgroup (256 registers per lane); everything else for 16.
-// ---------------------------------------------------------------------------
-typedef void (*kernel_fn)(const ConvKParams);
-
-template <int MF, int TAPS, bool EXT>
-static kernel_fn pick_mbnb(int mb, int nb) {
-    if (mb == 1 && nb == 1) return tdc_conv_mfma_kernel<MF, 1, 1, TAPS, 16, EXT>;
-    if (mb == 1 && nb == 2) return tdc_conv_mfma_kernel<MF, 1, 2, TAPS, 16, EXT>;
-    if (mb == 2 && nb == 1) return tdc_conv_mfma_kernel<MF, 2, 1, TAPS, 16, EXT>;
-    if (mb == 2 && nb == 2) return tdc_conv_mfma_kernel<MF, 2, 2, TAPS, 8, EXT>;
-    return nullptr;
-}
-
-template <int TAPS, bool EXT>
-static kernel_fn pick_mf(int mf, int mb, int nb) {
-    if (mf == 32) return pick_mbnb<32, TAPS, EXT>(mb, nb);
-    if (mf == 16) return pick_mbnb<16, TAPS, EXT>(mb, nb);
-    return nullptr;
-}
-
-static int taps_mode(int KH, int KW, int dil) {
-    if (KH == 3 && KW == 3 && dil == 1) return TAPS_3x3;
-    if (KH == 1 && KW == 1) return TAPS_1x1;
-    return TAPS_GENERIC;
-}
-
-// ---------------------------------------------------------------------------
 // 3x3 convolution streamed the same way (tile.alg = 4): one workgroup owns 16 output channels of a TH x TW tile of 16
 // pixels, its WK waves split the input channels, CG groups of four channels each.  Per group a lane requests its nine
 // input values (one per tap, four channels across the lane quarters) and its nine weights (packed as for
@@ -1550,6 +1524,29 @@ __global__ void __launch_bounds__(1024) tdc_conv3x3_stream_kernel(const ConvKPar
     }
 }
 
+// ---------------------------------------------------------------------------
+// Instantiation table: KernelId (worked out on the host from tile and filter, see kernel_id_for) -> function.
+// A 2x2 block grid of MFMAs per wave is built for at most 8 waves per workgroup (256 registers per lane), the
+// Winograd loop for 12, everything else for 16.
+// ---------------------------------------------------------------------------
+typedef void (*kernel_fn)(const ConvKParams);
+
+template <int MF, int TAPS, bool EXT>
+static kernel_fn pick_mbnb(int mb, int nb) {
+    if (mb == 1 && nb == 1) return tdc_conv_mfma_kernel<MF, 1, 1, TAPS, 16, EXT>;
+    if (mb == 1 && nb == 2) return tdc_conv_mfma_kernel<MF, 1, 2, TAPS, 16, EXT>;
+    if (mb == 2 && nb == 1) return tdc_conv_mfma_kernel<MF, 2, 1, TAPS, 16, EXT>;
+    if (mb == 2 && nb == 2) return tdc_conv_mfma_kernel<MF, 2, 2, TAPS, 8, EXT>;
+    return nullptr;
+}
+
+template <int TAPS, bool EXT>
+static kernel_fn pick_mf(int mf, int mb, int nb) {
+    if (mf == 32) return pick_mbnb<32, TAPS, EXT>(mb, nb);
+    if (mf == 16) return pick_mbnb<16, TAPS, EXT>(mb, nb);
+    return nullptr;
+}
+
 template <bool AFF, int MODE>
 static kernel_fn pick_stream(int nq) {
     switch (nq) {
@@ -1571,54 +1568,50 @@ static kernel_fn pick_stream3(int groups) {
     }
 }
 
-// The streamed 3x3 kernel with a fused 1x1 head and tail (a whole Tucker convolution), for a tile.alg = 4 tile.
-const void *conv_kernel_with_head(const tdc_tile &t) {
-    if (t.alg != 4 || t.ks != 1 || t.cch % (4 * t.wk) != 0) return nullptr;
-    return reinterpret_cast<const void *>(pick_stream3<false, 3>(t.cch / (4 * t.wk)));
-}
-
-const void *conv_kernel_for(const tdc_tile &t, int KH, int KW, int dilation, int stride, bool extras) {
+const void *kernel_function(const KernelId &k) {
     kernel_fn fn = nullptr;
-    if (t.alg == 4) {
-        // (`extras` can only mean a fused tail here, which the one kernel carries)
-        if (KH != 3 || KW != 3 || dilation != 1 || t.mf != 16 || t.mb != 1 || t.nb != 1 || t.wm < 1 || t.wn != 1 || t.wk < 1 || t.wm * t.wk > 16)
-            return nullptr;
-        const int groups = t.cch % (4 * t.wk) == 0 ? t.cch / (4 * t.wk) : 0;
-        const bool row = stride == 1 && t.tw == 14;
-        if (extras && t.ks > 1) return nullptr;
-        const int mode = extras ? 2 : t.ks > 1 ? 1 : 0;
-        kernel_fn f = nullptr;
-        if (row) f = mode == 2 ? pick_stream3<true, 2>(groups) : mode == 1 ? pick_stream3<true, 1>(groups) : pick_stream3<true, 0>(groups);
-        else f = mode == 2 ? pick_stream3<false, 2>(groups) : mode == 1 ? pick_stream3<false, 1>(groups) : pick_stream3<false, 0>(groups);
-        return reinterpret_cast<const void *>(f);
-    }
-    if (t.alg == 3) {
-        // (`extras` here can only mean the input affine: the host refuses a fused tail for this path)
-        if (KH != 1 || KW != 1 || t.mf != 16 || t.mb != 1 || t.nb != 1 || t.wm != 1 || t.wn != 1 || t.wk < 1) return nullptr;
-        if (t.cch % (16 * t.wk) != 0) return nullptr;
-        const int nq = t.cch / (16 * t.wk);
-        if (t.wk > (nq == 8 ? 8 : 16)) return nullptr;
-        if (stride > 1 && t.ks > 1) return nullptr;
-        if (stride > 1) return reinterpret_cast<const void *>(extras ? pick_stream<true, 2>(nq) : pick_stream<false, 2>(nq));
-        if (t.ks > 1) return reinterpret_cast<const void *>(extras ? pick_stream<true, 1>(nq) : pick_stream<false, 1>(nq));
-        return reinterpret_cast<const void *>(extras ? pick_stream<true, 0>(nq) : pick_stream<false, 0>(nq));
-    }
-    if (t.alg == 1) {
-        if (extras || KH != 3 || KW != 3 || dilation != 1 || t.mf != 16 || t.mb != 1 || t.nb != 1) return nullptr;
-        return reinterpret_cast<const void *>(static_cast<kernel_fn>(tdc_conv_mfma_kernel<16, 1, 1, TAPS_WINO, 12, false>));
-    }
-    if (t.alg == 2) {
-        if (extras || KH != 3 || KW != 3 || dilation != 1 || t.mb != 1 || t.nb != 1) return nullptr;
-        if (t.mf == 16) return reinterpret_cast<const void *>(static_cast<kernel_fn>(tdc_conv_mfma_kernel<16, 1, 1, TAPS_3x3G, 16, false>));
-        if (t.mf == 32) return reinterpret_cast<const void *>(static_cast<kernel_fn>(tdc_conv_mfma_kernel<32, 1, 1, TAPS_3x3G, 16, false>));
-        return nullptr;
-    }
-    switch (taps_mode(KH, KW, dilation)) {
-        case TAPS_3x3: fn = extras ? pick_mf<TAPS_3x3, true>(t.mf, t.mb, t.nb) : pick_mf<TAPS_3x3, false>(t.mf, t.mb, t.nb); break;
-        case TAPS_1x1: fn = extras ? pick_mf<TAPS_1x1, true>(t.mf, t.mb, t.nb) : pick_mf<TAPS_1x1, false>(t.mf, t.mb, t.nb); break;
-        default: fn = extras ? pick_mf<TAPS_GENERIC, true>(t.mf, t.mb, t.nb) : pick_mf<TAPS_GENERIC, false>(t.mf, t.mb, t.nb); break;
+    if (k.family == KernelId::STAGED) {
+        const bool ext = k.p[5] != 0;
+        switch (k.p[3]) {
+            case TAPS_WINO:
+                if (k.p[0] == 16 && k.p[1] == 1 && k.p[2] == 1 && !ext) fn = tdc_conv_mfma_kernel<16, 1, 1, TAPS_WINO, 12, false>;
+                break;
+            case TAPS_3x3G:
+                if (k.p[1] == 1 && k.p[2] == 1 && !ext)
+                    fn = k.p[0] == 16 ? static_cast<kernel_fn>(tdc_conv_mfma_kernel<16, 1, 1, TAPS_3x3G, 16, false>)
+                       : k.p[0] == 32 ? static_cast<kernel_fn>(tdc_conv_mfma_kernel<32, 1, 1, TAPS_3x3G, 16, false>) : nullptr;
+                break;
+            case TAPS_3x3: fn = ext ? pick_mf<TAPS_3x3, true>(k.p[0], k.p[1], k.p[2]) : pick_mf<TAPS_3x3, false>(k.p[0], k.p[1], k.p[2]); break;
+            case TAPS_1x1: fn = ext ? pick_mf<TAPS_1x1, true>(k.p[0], k.p[1], k.p[2]) : pick_mf<TAPS_1x1, false>(k.p[0], k.p[1], k.p[2]); break;
+            case TAPS_GENERIC: fn = ext ? pick_mf<TAPS_GENERIC, true>(k.p[0], k.p[1], k.p[2]) : pick_mf<TAPS_GENERIC, false>(k.p[0], k.p[1], k.p[2]); break;
+            default: break;
+        }
+    } else if (k.family == KernelId::STREAM_1x1) {
+        const int nq = k.p[0], mode = k.p[2];
+        if (k.p[1]) fn = mode == 2 ? pick_stream<true, 2>(nq) : mode == 1 ? pick_stream<true, 1>(nq) : mode == 0 ? pick_stream<true, 0>(nq) : nullptr;
+        else fn = mode == 2 ? pick_stream<false, 2>(nq) : mode == 1 ? pick_stream<false, 1>(nq) : mode == 0 ? pick_stream<false, 0>(nq) : nullptr;
+    } else if (k.family == KernelId::STREAM_3x3) {
+        const int cg = k.p[0], mode = k.p[2];
+        if (k.p[1]) fn = mode == 2 ? pick_stream3<true, 2>(cg) : mode == 1 ? pick_stream3<true, 1>(cg) : mode == 0 ? pick_stream3<true, 0>(cg) : nullptr;
+        else fn = mode == 3 ? pick_stream3<false, 3>(cg) : mode == 2 ? pick_stream3<false, 2>(cg) : mode == 1 ? pick_stream3<false, 1>(cg)
+                : mode == 0 ? pick_stream3<false, 0>(cg) : nullptr;
     }
     return reinterpret_cast<const void *>(fn);
+}
+
+int kernel_resources(const void *fn, int block_threads, int dynamic_lds_bytes, int *vgprs, int *static_lds, int *max_threads,
+                     int *max_wg_per_cu) {
+    hipFuncAttributes attr{};
+    hipError_t e = hipFuncGetAttributes(&attr, fn);
+    if (e != hipSuccess) return (int)e;
+    int blocks = 0;
+    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, fn, block_threads, (size_t)dynamic_lds_bytes);
+    if (e != hipSuccess) return (int)e;
+    *vgprs = attr.numRegs;
+    *static_lds = (int)attr.sharedSizeBytes;
+    *max_threads = attr.maxThreadsPerBlock;
+    *max_wg_per_cu = blocks;
+    return 0;
 }
 
 int prepare_conv_kernel(const void *fn, const Geometry &g) {

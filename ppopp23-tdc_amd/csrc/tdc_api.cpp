@@ -134,6 +134,21 @@ int tdc_model_select_with_tail(const tdc_conv_desc *desc, int32_t tail_N, tdc_ti
     return TDC_OK;
 }
 
+int tdc_model_kernel_info(const tdc_conv_desc *desc, const tdc_tile *tile, int32_t extras, char *name_out, int32_t cap,
+                          int32_t *vgprs_out, int32_t *waves_per_simd_out) {
+    if (!desc || !tile || (cap > 0 && !name_out)) return fail(TDC_ERR_INVALID, "null argument");
+    const KernelId k = kernel_id_for(*tile, desc->KH, desc->KW, desc->dilation, desc->stride, extras != 0);
+    if (k.family == KernelId::NONE) return fail(TDC_ERR_UNSUPPORTED, "no kernel instantiated for this tile");
+    const std::string name = kernel_name(k);
+    if (cap > 0) {
+        std::strncpy(name_out, name.c_str(), (size_t)cap - 1);
+        name_out[cap - 1] = '\0';
+    }
+    if (vgprs_out) *vgprs_out = kernel_vgprs(k);
+    if (waves_per_simd_out) *waves_per_simd_out = kernel_waves_per_simd(k);
+    return TDC_OK;
+}
+
 int tdc_load_bin(const char *path, float *dst, uint64_t count) {
     if (!path || (!dst && count)) return fail(TDC_ERR_INVALID, "null argument");
     FILE *f = std::fopen(path, "rb");
@@ -467,6 +482,23 @@ int tdc_conv_plan_set_head(tdc_conv_plan *plan, int32_t head_C, const float *w_h
     return TDC_OK;
 }
 
+int tdc_conv_plan_occupancy(const tdc_conv_plan *plan, tdc_kernel_occupancy *out) {
+    if (!plan || !out) return fail(TDC_ERR_INVALID, "null argument");
+    std::memset(out, 0, sizeof(*out));
+    int vgprs = 0, static_lds = 0, max_threads = 0, wg = 0;
+    if (int he = kernel_resources(plan->kernel, plan->geo.threads, plan->geo.lds_bytes, &vgprs, &static_lds, &max_threads, &wg))
+        return hip_fail("hipFuncGetAttributes / hipOccupancyMaxActiveBlocksPerMultiprocessor", he);
+    out->kernel_vgprs = vgprs;
+    out->kernel_static_lds_bytes = static_lds;
+    out->kernel_max_threads = max_threads;
+    out->runtime_wg_per_cu = wg;
+    out->block_threads = plan->geo.threads;
+    out->dynamic_lds_bytes = plan->geo.lds_bytes;
+    out->model_vgprs = plan->info.vgpr_estimate;
+    out->model_wg_per_cu = plan->info.wg_per_cu;
+    return TDC_OK;
+}
+
 int tdc_conv_plan_query(const tdc_conv_plan *plan, tdc_tile_info *info_out) {
     if (!plan || !info_out) return fail(TDC_ERR_INVALID, "null argument");
     *info_out = plan->info;
@@ -477,8 +509,22 @@ int tdc_conv_forward(tdc_conv_plan *plan, const float *d_in, const float *d_resi
     return tdc_conv_forward_strided(plan, d_in, 0, d_residual, 0, d_out, 0, stream);
 }
 
+// The launch behind every forward entry point.  `ws` / `ctr`: where a plan whose tile splits the input channels over
+// several workgroups keeps its partial tiles and ticket counters (the plan's own buffers, or the static scratch).
+static int forward_impl(tdc_conv_plan *plan, const float *d_in, int64_t in_batch_stride, const float *d_residual,
+                        int64_t residual_batch_stride, float *d_out, int64_t out_batch_stride, float *ws, unsigned *ctr,
+                        void *stream);
+
 int tdc_conv_forward_strided(tdc_conv_plan *plan, const float *d_in, int64_t in_batch_stride, const float *d_residual,
                              int64_t residual_batch_stride, float *d_out, int64_t out_batch_stride, void *stream) {
+    if (!plan) return fail(TDC_ERR_INVALID, "null argument");
+    return forward_impl(plan, d_in, in_batch_stride, d_residual, residual_batch_stride, d_out, out_batch_stride, plan->d_ws,
+                        plan->d_ctr, stream);
+}
+
+static int forward_impl(tdc_conv_plan *plan, const float *d_in, int64_t in_batch_stride, const float *d_residual,
+                        int64_t residual_batch_stride, float *d_out, int64_t out_batch_stride, float *ws, unsigned *ctr,
+                        void *stream) {
     if (!plan || !d_in || !d_out) return fail(TDC_ERR_INVALID, "null argument");
     if (in_batch_stride < 0 || out_batch_stride < 0 || residual_batch_stride < 0)
         return fail(TDC_ERR_INVALID, "negative batch stride");
@@ -498,7 +544,7 @@ int tdc_conv_forward_strided(tdc_conv_plan *plan, const float *d_in, int64_t in_
     kp.bias = plan->d_bias;
     kp.resid = d_residual;
     kp.out = d_out;
-    kp.ws = plan->d_ws;
+    kp.ws = ws;
     kp.in_aff = plan->d_in_aff;
     kp.tail_w = plan->tail_N > 0 ? plan->d_tail_w : nullptr;
     kp.tail_bias = plan->d_tail_bias;
@@ -511,7 +557,7 @@ int tdc_conv_forward_strided(tdc_conv_plan *plan, const float *d_in, int64_t in_
     kp.fd_hnpb = make_fastdiv(std::max(plan->head_npb, 1));
     kp.fd_npx = make_fastdiv(g.PT / 16);
     kp.in_relu = plan->in_relu;
-    kp.ctr = plan->d_ctr;
+    kp.ctr = ctr;
     kp.in_image_bytes = (unsigned)(in_image * 4);
     kp.in_bstride = in_batch_stride ? in_batch_stride : in_image;
     kp.out_bstride = out_batch_stride ? out_batch_stride : out_image;

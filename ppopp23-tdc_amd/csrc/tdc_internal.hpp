@@ -148,14 +148,45 @@ struct ConvKParams {
     long long resid_bstride;   // ... of the residual
 };
 
-// The instantiated kernel for a tile and filter size (nullptr if none).
-// `extras`: the instantiation that also carries the input affine and the fused 1x1 tail.
-const void *conv_kernel_for(const tdc_tile &t, int KH, int KW, int dilation, int stride, bool extras);
-const void *conv_kernel_with_head(const tdc_tile &t);
+// Inner loop of the staged kernel (its TAPS template argument).
+enum : int { TAPS_GENERIC = 0, TAPS_1x1 = 1, TAPS_3x3 = 9, TAPS_3x3G = 10, TAPS_WINO = 16 };
+
+// Which kernel instantiation serves a tile: worked out on the host (no device needed), so that the tile model, the
+// launcher and the occupancy probe all speak of the same function.
+//   STAGED      tdc_conv_mfma_kernel<MF, MB, NB, TAPS, MAXW, EXT>     p = {MF, MB, NB, TAPS, MAXW, EXT}
+//   STREAM_1x1  tdc_conv1x1_stream_kernel<NQ, AFF, MODE>              p = {NQ, AFF, MODE}
+//   STREAM_3x3  tdc_conv3x3_stream_kernel<CG, ROW, MODE>              p = {CG, ROW, MODE}
+struct KernelId {
+    enum Family : int { NONE = 0, STAGED = 1, STREAM_1x1 = 2, STREAM_3x3 = 3 };
+    int family = NONE;
+    int p[6] = {0, 0, 0, 0, 0, 0};
+};
+// `extras`: the instantiation that also carries the input affine and the fused 1x1 tail.  family == NONE: no kernel.
+KernelId kernel_id_for(const tdc_tile &t, int KH, int KW, int dilation, int stride, bool extras);
+KernelId kernel_id_with_head(const tdc_tile &t);   // streamed 3x3 with fused 1x1 head and tail
+// The kernel's name as the compiler's resource report and the profiler print it, e.g.
+// "tdc_conv_mfma_kernel<16, 1, 1, 9, 16, false>".
+std::string kernel_name(const KernelId &k);
+// Registers per lane (arch + acc) of that instantiation as compiled, rounded up to the allocation granule of 8;
+// 0 for an unknown one.  Kept in step with the compiler's report by tests/test_model.py.
+int kernel_vgprs(const KernelId &k);
+// Resident waves of that instantiation per SIMD, as limited by vector and scalar registers (at most 8).
+int kernel_waves_per_simd(const KernelId &k);
+// The function itself (nullptr if not instantiated).
+const void *kernel_function(const KernelId &k);
+inline const void *conv_kernel_for(const tdc_tile &t, int KH, int KW, int dilation, int stride, bool extras) {
+    return kernel_function(kernel_id_for(t, KH, KW, dilation, stride, extras));
+}
+inline const void *conv_kernel_with_head(const tdc_tile &t) { return kernel_function(kernel_id_with_head(t)); }
 // One-time per-plan attribute setup (dynamic LDS above 64 KiB).  hipError_t as int.
 int prepare_conv_kernel(const void *fn, const Geometry &g);
 // Enqueue the kernel.  Returns a hipError_t as int.
 int launch_conv(const void *fn, const Geometry &g, const ConvKParams &kp, void *stream);
+
+// What the compiled kernel really uses: registers per lane, static LDS, its launch bound, and how many workgroups
+// of `block_threads` threads with `dynamic_lds_bytes` of LDS the runtime places on one compute unit.
+int kernel_resources(const void *fn, int block_threads, int dynamic_lds_bytes, int *vgprs, int *static_lds, int *max_threads,
+                     int *max_wg_per_cu);
 
 // Pooling / concatenation kernels of the whole-network graphs (hipError_t as int).
 // Batch strides are in floats; a tensor may be a channel slice of a wider buffer.

@@ -13,6 +13,7 @@
 #include <array>
 #include <map>
 #include <cmath>
+#include <cstdio>
 #include <cstdlib>
 #include <cstring>
 
@@ -410,19 +411,130 @@ double *mc_field(int i) {
     }
 }
 
-// Registers per lane of the instantiated kernels, rounded up to the allocation granule of 8.
-int kernel_vgprs(const tdc_tile &t, int taps_mode) {
-    const int nacc = (t.mf == 32) ? 16 : 4;
-    int regs = nacc * t.mb * t.nb + 6 * (t.mb + t.nb) + 24;
-    if (taps_mode == 9) regs += 6 * t.nb;
-    if (t.alg == 1) regs = 136;   // 64 accumulators, two sets of 16 B and 16 A operands, the raw patch
-    if (t.alg == 2) regs = 104;   // two sets of 18 A and 18 B operands
-    if (t.alg == 3) regs = 40 + 16 * (t.cch / (16 * t.wk));   // per run of 16 channels: 4 A, 4 B, 8 scale/shift
-    if (t.alg == 4) regs = 40 + 18 * (t.cch / (4 * t.wk));    // per group of 4 channels: 9 A, 9 B
-    return round_up(regs, 8);
+}  // namespace
+
+// Waves of this kernel that fit one SIMD: 512 vector registers per lane shared by its waves, at most 8 waves, and
+// 800 scalar registers handed out in blocks of 16 — the staged kernel needs 106 (112 allocated), which leaves room
+// for 7 waves, not 8, so a 1024-thread workgroup of it is alone on its compute unit however few vector registers it
+// uses (the HIP runtime's occupancy query says the same).  The streamed kernels stay under 96 scalar registers.
+int kernel_waves_per_simd(const KernelId &k) {
+    const int regs = kernel_vgprs(k);
+    if (regs <= 0) return 0;
+    const Machine &m = machine();
+    const int by_sgpr = k.family == KernelId::STAGED ? 800 / 112 : 800 / 96;
+    return std::min(std::min(m.max_waves_per_simd, m.vgprs_per_simd_lane / regs), by_sgpr);
 }
 
-}  // namespace
+KernelId kernel_id_with_head(const tdc_tile &t) {
+    KernelId k;
+    if (t.alg != 4 || t.ks != 1 || t.wk < 1 || t.cch % (4 * t.wk) != 0) return k;
+    const int cg = t.cch / (4 * t.wk);
+    if (cg != 1 && cg != 2 && cg != 4) return k;
+    k.family = KernelId::STREAM_3x3;
+    k.p[0] = cg; k.p[1] = 0; k.p[2] = 3;
+    return k;
+}
+
+KernelId kernel_id_for(const tdc_tile &t, int KH, int KW, int dilation, int stride, bool extras) {
+    KernelId k;
+    if (t.alg == 4) {
+        // (`extras` can only mean a fused tail here, which the one kernel carries)
+        if (KH != 3 || KW != 3 || dilation != 1 || t.mf != 16 || t.mb != 1 || t.nb != 1 || t.wm < 1 || t.wn != 1 || t.wk < 1 ||
+            t.wm * t.wk > 16 || t.cch % (4 * t.wk) != 0)
+            return k;
+        const int cg = t.cch / (4 * t.wk);
+        if ((cg != 1 && cg != 2 && cg != 4) || (extras && t.ks > 1)) return k;
+        k.family = KernelId::STREAM_3x3;
+        k.p[0] = cg;
+        k.p[1] = stride == 1 && t.tw == 14;   // one row of 14 pixels: the taps of a filter row are lane shifts
+        k.p[2] = extras ? 2 : t.ks > 1 ? 1 : 0;
+        return k;
+    }
+    if (t.alg == 3) {
+        // (`extras` here can only mean the input affine: the host refuses a fused tail for this path)
+        if (KH != 1 || KW != 1 || t.mf != 16 || t.mb != 1 || t.nb != 1 || t.wm != 1 || t.wn != 1 || t.wk < 1 ||
+            t.cch % (16 * t.wk) != 0)
+            return k;
+        const int nq = t.cch / (16 * t.wk);
+        if ((nq != 1 && nq != 2 && nq != 4 && nq != 8) || t.wk > (nq == 8 ? 8 : 16) || (stride > 1 && t.ks > 1)) return k;
+        k.family = KernelId::STREAM_1x1;
+        k.p[0] = nq; k.p[1] = extras; k.p[2] = stride > 1 ? 2 : t.ks > 1 ? 1 : 0;
+        return k;
+    }
+    if (t.mf != 16 && t.mf != 32) return k;
+    if (t.mb < 1 || t.mb > 2 || t.nb < 1 || t.nb > 2) return k;
+    int taps;
+    if (t.alg == 1) {
+        if (extras || KH != 3 || KW != 3 || dilation != 1 || t.mf != 16 || t.mb != 1 || t.nb != 1) return k;
+        taps = TAPS_WINO;
+    } else if (t.alg == 2) {
+        if (extras || KH != 3 || KW != 3 || dilation != 1 || t.mb != 1 || t.nb != 1) return k;
+        taps = TAPS_3x3G;
+    } else if (t.alg == 0) {
+        taps = (KH == 3 && KW == 3 && dilation == 1) ? TAPS_3x3 : (KH == 1 && KW == 1) ? TAPS_1x1 : TAPS_GENERIC;
+    } else {
+        return k;
+    }
+    k.family = KernelId::STAGED;
+    k.p[0] = t.mf; k.p[1] = t.mb; k.p[2] = t.nb; k.p[3] = taps;
+    k.p[4] = taps == TAPS_WINO ? 12 : (t.mb == 2 && t.nb == 2) ? 8 : 16;   // launch bound in waves
+    k.p[5] = extras;
+    return k;
+}
+
+std::string kernel_name(const KernelId &k) {
+    char buf[96];
+    const char *tf[2] = {"false", "true"};
+    switch (k.family) {
+        case KernelId::STAGED:
+            std::snprintf(buf, sizeof buf, "tdc_conv_mfma_kernel<%d, %d, %d, %d, %d, %s>", k.p[0], k.p[1], k.p[2], k.p[3], k.p[4], tf[k.p[5] != 0]);
+            break;
+        case KernelId::STREAM_1x1:
+            std::snprintf(buf, sizeof buf, "tdc_conv1x1_stream_kernel<%d, %s, %d>", k.p[0], tf[k.p[1] != 0], k.p[2]);
+            break;
+        case KernelId::STREAM_3x3:
+            std::snprintf(buf, sizeof buf, "tdc_conv3x3_stream_kernel<%d, %s, %d>", k.p[0], tf[k.p[1] != 0], k.p[2]);
+            break;
+        default: return "";
+    }
+    return buf;
+}
+
+// Registers per lane of the compiled instantiations (hipcc's kernel-resource-usage report: VGPRs + AGPRs), rounded
+// up to the allocation granule of 8.  The reference measures occupancy per candidate by compiling and probing each
+// (2080Ti-evaluation/Gen-occupancy/template.cu:277-284); here the candidates share a few dozen instantiations, so
+// the table is short, and a test compares it with the report of the build at hand.
+int kernel_vgprs(const KernelId &k) {
+    if (k.family == KernelId::STREAM_1x1) {
+        const int nq = k.p[0], aff = k.p[1], mode = k.p[2];
+        if (aff) return nq == 1 ? (mode == 1 ? 72 : 40) : nq == 2 ? (mode == 1 ? 72 : 48) : nq == 4 ? 80 : 144;
+        if (mode == 1) return nq == 8 ? 96 : 72;
+        return nq == 1 ? 40 : nq == 2 ? 40 : nq == 4 ? 48 : 80;
+    }
+    if (k.family == KernelId::STREAM_3x3) {
+        const int cg = k.p[0], row = k.p[1], mode = k.p[2];
+        if (cg == 4) return 88;
+        if (mode == 1) return 64;
+        if (mode == 3) return cg == 1 ? 56 : 64;
+        if (cg == 1) return row && mode == 0 ? 40 : 48;
+        return row ? 48 : 56;
+    }
+    if (k.family != KernelId::STAGED) return 0;
+    const int mf = k.p[0], mb = k.p[1], nb = k.p[2], taps = k.p[3], ext = k.p[5];
+    if (taps == TAPS_WINO) return 128;
+    if (taps == TAPS_3x3G) return mf == 16 ? 104 : 120;
+    const int blk = (mb - 1) * 2 + (nb - 1);   // 1x1, 1x2, 2x1, 2x2 blocks per wave
+    // [mf 16/32][taps generic/1x1/3x3][blocks][plain/extras]
+    static const int tab[2][3][4][2] = {
+        {{{32, 32}, {48, 48}, {40, 40}, {64, 64}},
+         {{48, 72}, {56, 80}, {64, 80}, {80, 88}},
+         {{64, 64}, {88, 88}, {96, 96}, {120, 120}}},
+        {{{48, 48}, {80, 80}, {64, 64}, {128, 128}},
+         {{56, 80}, {88, 104}, {88, 104}, {128, 144}},
+         {{80, 80}, {112, 112}, {112, 112}, {168, 168}}}};
+    const int ti = taps == TAPS_GENERIC ? 0 : taps == TAPS_1x1 ? 1 : 2;
+    return tab[mf == 32][ti][blk][ext != 0];
+}
 
 bool model_evaluate(const tdc_conv_desc &d, const tdc_tile &t, tdc_tile_info &info, std::string *why, int tail_N) {
     Geometry g;
@@ -437,11 +549,16 @@ bool model_evaluate(const tdc_conv_desc &d, const tdc_tile &t, tdc_tile_info &in
     info.lds_bytes = g.lds_bytes;
     info.nchunks = g.nchunks;
     info.th = g.TH;
-    const int mode = (d.KH == 3 && d.KW == 3 && d.dilation == 1) ? 9 : (d.KH == 1 && d.KW == 1) ? 1 : 0;
-    info.vgpr_estimate = kernel_vgprs(t, mode);
+    // (a fused tail needs the instantiation with the extras; an input affine, which the model does not know of, too)
+    const KernelId kid = kernel_id_for(t, d.KH, d.KW, d.dilation, d.stride, tail_N > 0);
+    info.vgpr_estimate = kernel_vgprs(kid);
+    if (info.vgpr_estimate <= 0) {
+        if (why) *why = "no kernel instantiated for this tile";
+        return false;
+    }
 
     // --- occupancy (replaces cudaOccupancyMaxActiveBlocksPerMultiprocessor) ---
-    const int waves_simd_vgpr = std::min(m.max_waves_per_simd, m.vgprs_per_simd_lane / info.vgpr_estimate);
+    const int waves_simd_vgpr = kernel_waves_per_simd(kid);   // registers per lane, and scalar registers per wave
     const int wg_waves_per_simd = ceil_div(g.waves, m.simds_per_cu);
     const int wg_by_vgpr = waves_simd_vgpr / wg_waves_per_simd;
     const int wg_by_lds = m.lds_bytes_per_cu / std::max(g.lds_bytes, 1);

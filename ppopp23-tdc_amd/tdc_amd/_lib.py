@@ -19,12 +19,12 @@ EXPORTS = (
     "tdc_last_error_string", "tdc_version", "tdc_load_bin", "tdc_save_bin",
     "tdc_conv_plan_create", "tdc_conv_plan_create_with_tail", "tdc_conv_plan_set_tail_weights",
     "tdc_conv_plan_set_weights", "tdc_conv_plan_set_input_affine", "tdc_conv_plan_set_head", "tdc_conv_plan_query",
-    "tdc_conv_forward",
+    "tdc_conv_forward", "tdc_conv_plan_occupancy",
     "tdc_conv_forward_strided", "tdc_tkconv_forward_strided",
     "tdc_conv_time", "tdc_conv_time_many", "tdc_conv_plan_destroy",
     "tdc_tkconv_create", "tdc_tkconv_set_weights", "tdc_tkconv_forward", "tdc_tkconv_forward_features",
     "tdc_tkconv_core_forward", "tdc_tkconv_query", "tdc_tkconv_num_kernels", "tdc_tkconv_destroy",
-    "tdc_model_evaluate", "tdc_model_enumerate", "tdc_model_select", "tdc_model_select_with_tail", "tdc_model_get_constants",
+    "tdc_model_evaluate", "tdc_model_kernel_info", "tdc_model_enumerate", "tdc_model_select", "tdc_model_select_with_tail", "tdc_model_get_constants",
     "tdc_model_set_constants", "tdc_set_autotune", "tdc_get_autotune",
     "tdc_net_create", "tdc_net_tensor", "tdc_net_view", "tdc_net_affine", "tdc_net_affine_conv", "tdc_net_conv", "tdc_net_conv_tail", "tdc_net_set_input_affine", "tdc_net_tkconv", "tdc_net_pool", "tdc_net_global_avgpool", "tdc_net_concat",
     "tdc_net_tensor_shape", "tdc_net_num_kernels", "tdc_net_finalize", "tdc_net_forward", "tdc_net_time",
@@ -68,6 +68,14 @@ class TileInfo(Structure):
         return d
 
 
+class KernelOccupancy(Structure):
+    _fields_ = [(n, c_int32) for n in ("kernel_vgprs", "kernel_static_lds_bytes", "kernel_max_threads", "runtime_wg_per_cu",
+                                       "block_threads", "dynamic_lds_bytes", "model_vgprs", "model_wg_per_cu")]
+
+    def asdict(self):
+        return {n: getattr(self, n) for n, _ in self._fields_}
+
+
 class TKConvDesc(Structure):
     _fields_ = [(n, c_int32) for n in ("batch", "C", "R1", "R2", "N", "H", "W", "K", "stride", "pad", "dilation",
                                        "has_bias", "relu")]
@@ -95,6 +103,7 @@ def lib():
     L.tdc_conv_plan_set_weights.argtypes = [c_void_p, c_void_p, c_void_p]
     L.tdc_conv_plan_query.argtypes = [c_void_p, POINTER(TileInfo)]
     L.tdc_conv_forward.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]
+    L.tdc_conv_plan_occupancy.argtypes = [c_void_p, POINTER(KernelOccupancy)]
     L.tdc_conv_time.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, POINTER(ctypes.c_float)]
     L.tdc_conv_time_many.argtypes = [POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p), c_int32, c_int32, c_int32,
                                      POINTER(ctypes.c_float)]
@@ -111,6 +120,8 @@ def lib():
     L.tdc_model_evaluate.argtypes = [POINTER(ConvDesc), POINTER(Tile), POINTER(TileInfo)]
     L.tdc_model_enumerate.argtypes = [POINTER(ConvDesc), POINTER(Tile), c_int32, POINTER(c_int32)]
     L.tdc_model_select.argtypes = [POINTER(ConvDesc), POINTER(TileInfo)]
+    L.tdc_model_kernel_info.argtypes = [POINTER(ConvDesc), POINTER(Tile), c_int32, c_char_p, c_int32, POINTER(c_int32),
+                                        POINTER(c_int32)]
     L.tdc_model_get_constants.argtypes = [POINTER(c_double), c_int32, POINTER(c_int32)]
     L.tdc_model_set_constants.argtypes = [POINTER(c_double), c_int32]
     i32, i32p, fpv = c_int32, POINTER(c_int32), c_void_p
@@ -164,6 +175,28 @@ def model_evaluate(desc: ConvDesc, tile: Tile) -> TileInfo:
     info = TileInfo()
     check(lib().tdc_model_evaluate(byref(desc), byref(tile), byref(info)))
     return info
+
+
+def model_kernel_info(desc: ConvDesc, tile: Tile, extras: bool = False):
+    """(name of the compiled kernel that serves `tile`, registers per lane the model assumes for it, waves of it per
+    SIMD by the model's register arithmetic)."""
+    buf = ctypes.create_string_buffer(128)
+    regs, waves = c_int32(0), c_int32(0)
+    check(lib().tdc_model_kernel_info(byref(desc), byref(tile), int(extras), buf, 128, byref(regs), byref(waves)))
+    return buf.value.decode(), regs.value, waves.value
+
+
+def kernel_resources():
+    """The compiler's resource report of the built kernels: {name: dict(vgprs, agprs, sgprs, scratch, waves_per_simd,
+    static_lds)} from kernel_resources.txt, which the build writes next to the library."""
+    path = os.path.join(_HERE, "kernel_resources.txt")
+    out = {}
+    for line in open(path):
+        if line.startswith("#") or not line.strip():
+            continue
+        f = [x.strip() for x in line.split("|")]
+        out[f[0]] = dict(zip(("vgprs", "agprs", "sgprs", "scratch", "waves_per_simd", "static_lds"), map(int, f[1:])))
+    return out
 
 
 MODEL_CONSTANT_NAMES = ("launch_us", "setup_clk", "copy_latency_clk", "copy_bytes_per_clk", "l2_bytes_per_clk",

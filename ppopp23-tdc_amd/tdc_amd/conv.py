@@ -112,6 +112,13 @@ class Conv2dPlan:
 
     __call__ = forward
 
+    def occupancy(self):
+        """What the compiled kernel of this plan uses (registers per lane, resident workgroups per compute unit as the
+        HIP runtime computes them) next to the tile model's assumptions: a ``_lib.KernelOccupancy``."""
+        occ = _lib.KernelOccupancy()
+        check(lib().tdc_conv_plan_occupancy(self._h, byref(occ)))
+        return occ
+
     def time_us(self, x, out, residual=None, iters=100, graph=True):
         """Device microseconds per launch: hipEvents around `iters` back-to-back launches issued from C
         (replayed from one HIP graph when `graph`)."""

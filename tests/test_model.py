@@ -158,3 +158,37 @@ def test_stride2_and_stem_shapes_have_tiles():
               tdc_amd.conv_desc(8, 64, 16, 56, 56, 3, 3, 1, 1)):
         i = tdc_amd.model_select(d)
         assert i.grid_x > 0 and i.lds_bytes <= LDS_BYTES
+
+
+def test_model_register_table_matches_the_compiled_kernels():
+    """Occupancy probe, host side: for every kernel instantiation that any candidate tile of a spread of layers maps
+    to, the registers per lane the model's occupancy term assumes equal what hipcc reports for the build at hand
+    (VGPRs + AGPRs, rounded up to the allocation granule of 8), and no kernel spills to scratch.  The reference
+    measures occupancy per candidate by compiling and probing each one
+    (2080Ti-evaluation/Gen-occupancy/template.cu:277-284)."""
+    from tdc_amd import _lib
+    compiled = _lib.kernel_resources()
+    assert len(compiled) >= 90
+    assert all(r["scratch"] == 0 for r in compiled.values()), "a kernel spills registers to scratch memory"
+    seen = {}
+    descs = [conv3(64, 64, 56), conv3(128, 128, 56), conv3(16, 16, 7), conv3(256, 256, 7), conv3(40, 24, 13, stride=2),
+             tdc_amd.conv_desc(1, 256, 64, 56, 56, 1, 1, 1, 0), tdc_amd.conv_desc(1, 2048, 256, 7, 7, 1, 1, 1, 0),
+             tdc_amd.conv_desc(1, 64, 128, 56, 56, 1, 1, 2, 0), tdc_amd.conv_desc(1, 3, 64, 224, 224, 7, 7, 2, 3),
+             tdc_amd.conv_desc(2, 100, 36, 14, 14, 1, 1, 1, 0)]
+    for d in descs:
+        for t in tdc_amd.model_enumerate(d):
+            for extras in (False, True):
+                try:
+                    name, regs, waves = _lib.model_kernel_info(d, t, extras)
+                except tdc_amd.TdcError:
+                    continue   # (no instantiation with extras for this path)
+                seen[name] = (regs, waves)
+                if not extras:
+                    assert tdc_amd.model_evaluate(d, t).vgpr_estimate == regs
+    assert len(seen) >= 60, sorted(seen)
+    for name, (regs, waves) in sorted(seen.items()):
+        assert name in compiled, f"{name}: the model names a kernel the build does not contain"
+        real = compiled[name]["vgprs"] + compiled[name]["agprs"]
+        assert regs == (real + 7) // 8 * 8, f"{name}: model assumes {regs} registers per lane, compiled kernel uses {real}"
+        # the compiler's own waves-per-SIMD figure (vector and scalar register limits) is the model's
+        assert compiled[name]["waves_per_simd"] == waves, f"{name}: {compiled[name]} against the model's {waves} waves per SIMD"
