@@ -49,14 +49,16 @@ DENSENET121_BLOCKS = (6, 12, 24, 16)
 
 
 @torch.no_grad()
-def tucker_densenet121_forward(p, x):
+def tucker_densenet121_forward(p, x, return_features=False):
     """inference/densenet_inet_tt.py: TenDenseLayer.forward (:96-112, norm1 -> conv1 -> norm2 -> conv2 on the
     concatenation of all earlier features), TenDenseBlock.forward (:132-137), TenDenseTransition (:140-158),
     features -> norm5 -> global pool -> classifier.  The norm layers are BatchNorm + ReLU."""
     def bnrelu(t, prefix):
         return F.relu(_bn(t, p, prefix))
 
+    out_feats = {}
     x = bnrelu(F.conv2d(x, p["features.conv0.weight"], None, 2, 3), "features.norm0")
+    out_feats["stem"] = x
     x = F.max_pool2d(x, 3, 2, 1)
     for b, nl in enumerate(DENSENET121_BLOCKS, start=1):
         feats = [x]
@@ -69,9 +71,11 @@ def tucker_densenet121_forward(p, x):
             y = F.conv2d(y, p[pre + ".conv2.last_kernel"], None)
             feats.append(y)
         x = torch.cat(feats, 1)
+        out_feats[f"denseblock{b}"] = x
         if b < len(DENSENET121_BLOCKS):
             pre = f"features.transition{b}"
             x = F.avg_pool2d(F.conv2d(bnrelu(x, pre + ".norm"), p[pre + ".conv.weight"]), 2, 2)
     x = bnrelu(x, "features.norm5")
     x = torch.flatten(F.adaptive_avg_pool2d(x, (1, 1)), 1)
-    return F.linear(x, p["classifier.weight"], p["classifier.bias"])
+    x = F.linear(x, p["classifier.weight"], p["classifier.bias"])
+    return (x, out_feats) if return_features else x

@@ -183,15 +183,19 @@ RESNET18_STAGES = ((64, 1), (128, 2), (256, 2), (512, 2))   # (planes, stride of
 
 def resnet18_params(seed=18, num_classes=1000, rank_ratio=0.5):
     """Random-init Tucker ResNet-18 with the reference's state-dict key names: Kaiming-normal convolutions,
-    non-trivial BatchNorm statistics (so that the folding is exercised), ranks R1 = R2 = planes * rank_ratio."""
+    non-trivial BatchNorm statistics (so that the folding is exercised), ranks R1 = R2 = planes * rank_ratio.
+    The Kaiming gain of 2 is applied once per ReLU, not once per convolution: a Tucker convolution is three linear
+    maps in a row with a single ReLU behind them (first factor and core get gain 1, the last factor gain 2), and the
+    BatchNorm that closes a residual branch is scaled by 0.3, so activations stay of order one through all eight
+    blocks instead of growing by orders of magnitude, and element-wise tolerances mean something."""
     g = torch.Generator().manual_seed(seed)
 
-    def kaiming(*shape):
+    def kaiming(*shape, gain=2.0):
         fan_in = shape[1] * shape[2] * shape[3]
-        return torch.empty(*shape).normal_(0, math.sqrt(2.0 / fan_in), generator=g)
+        return torch.empty(*shape).normal_(0, math.sqrt(gain / fan_in), generator=g)
 
-    def bn(prefix, n, p):
-        p[prefix + ".weight"] = torch.rand(n, generator=g) * 0.5 + 0.75
+    def bn(prefix, n, p, scale=1.0):
+        p[prefix + ".weight"] = (torch.rand(n, generator=g) * 0.5 + 0.75) * scale
         p[prefix + ".bias"] = torch.randn(n, generator=g) * 0.1
         p[prefix + ".running_mean"] = torch.randn(n, generator=g) * 0.1
         p[prefix + ".running_var"] = torch.rand(n, generator=g) * 0.5 + 0.75
@@ -205,10 +209,10 @@ def resnet18_params(seed=18, num_classes=1000, rank_ratio=0.5):
             cin = inplanes if b == 0 else planes
             for k, c in (("conv1", cin), ("conv2", planes)):
                 pre = f"layer{s}.{b}.{k}"
-                p[pre + ".first_kernel"] = kaiming(r, c, 1, 1)
-                p[pre + ".core_kernel"] = kaiming(r, r, 3, 3)
+                p[pre + ".first_kernel"] = kaiming(r, c, 1, 1, gain=1.0)
+                p[pre + ".core_kernel"] = kaiming(r, r, 3, 3, gain=1.0)
                 p[pre + ".last_kernel"] = kaiming(planes, r, 1, 1)
-                bn(f"layer{s}.{b}.bn{k[-1]}", planes, p)
+                bn(f"layer{s}.{b}.bn{k[-1]}", planes, p, scale=0.3 if k == "conv2" else 1.0)
             if b == 0 and (stride != 1 or inplanes != planes):
                 p[f"layer{s}.0.downsample.0.weight"] = kaiming(planes, inplanes, 1, 1)
                 bn(f"layer{s}.0.downsample.1", planes, p)
@@ -223,8 +227,11 @@ def build_tucker_resnet18(params, batch=1, H=224, W=224):
     p = params
     net = Net(batch, 3, H, W)
     s, t = bn_scale_shift(p, "bn1")
+    net.feature_ids = {}    # tensor ids of the stage outputs, by the names oracle/nets_ref.py uses
     x = net.conv(0, fold_dense(p["conv1.weight"], s), t, stride=2, pad=3, relu=True)      # conv1 + bn1 + relu
+    net.feature_ids["stem"] = x
     x = net.pool(x, "max", 3, 2, 1)
+    net.feature_ids["maxpool"] = x
     for st, (planes, stride) in enumerate(RESNET18_STAGES, start=1):
         for b in range(2):
             pre = f"layer{st}.{b}"
@@ -239,6 +246,7 @@ def build_tucker_resnet18(params, batch=1, H=224, W=224):
             s2, t2 = bn_scale_shift(p, pre + ".bn2")
             x = net.tkconv(y, p[pre + ".conv2.first_kernel"], p[pre + ".conv2.core_kernel"],
                            fold_dense(p[pre + ".conv2.last_kernel"], s2), t2, stride=1, pad=1, residual=identity, relu=True)
+            net.feature_ids[pre] = x
     x = net.global_avgpool(x)
     x = net.conv(x, p["fc.weight"].reshape(p["fc.weight"].shape[0], -1, 1, 1), p["fc.bias"])
     return net.finalize(x)
@@ -252,11 +260,14 @@ DENSENET121_BLOCKS = (6, 12, 24, 16)
 
 
 def densenet121_params(seed=121, num_classes=1000, growth=32, bn_size=4, ranks=(64, 16)):
+    """Random-init Tucker DenseNet-121 with the reference's state-dict key names.  As in ``resnet18_params`` the
+    Kaiming gain of 2 goes to the convolutions that read a ReLU's output (conv0, conv1, the first factor, the
+    transitions); core and last factor read a linear map's output and get gain 1, so activations stay of order one."""
     g = torch.Generator().manual_seed(seed)
 
-    def kaiming(*shape):
+    def kaiming(*shape, gain=2.0):
         fan_in = shape[1] * shape[2] * shape[3]
-        return torch.empty(*shape).normal_(0, math.sqrt(2.0 / fan_in), generator=g)
+        return torch.empty(*shape).normal_(0, math.sqrt(gain / fan_in), generator=g)
 
     def bn(prefix, n, p):
         p[prefix + ".weight"] = torch.rand(n, generator=g) * 0.5 + 0.75
@@ -276,8 +287,8 @@ def densenet121_params(seed=121, num_classes=1000, growth=32, bn_size=4, ranks=(
             p[pre + ".conv1.weight"] = kaiming(mid, c, 1, 1)
             bn(pre + ".norm2", mid, p)
             p[pre + ".conv2.first_kernel"] = kaiming(r1, mid, 1, 1)
-            p[pre + ".conv2.core_kernel"] = kaiming(r2, r1, 3, 3)
-            p[pre + ".conv2.last_kernel"] = kaiming(growth, r2, 1, 1)
+            p[pre + ".conv2.core_kernel"] = kaiming(r2, r1, 3, 3, gain=1.0)
+            p[pre + ".conv2.last_kernel"] = kaiming(growth, r2, 1, 1, gain=1.0)
             c += growth
         if b < len(DENSENET121_BLOCKS):
             pre = f"features.transition{b}"
@@ -344,6 +355,7 @@ def build_tucker_densenet121(params, batch=1, H=224, W=224, growth=32):
     h, w = (h + 2 - 3) // 2 + 1, (w + 2 - 3) // 2 + 1
     cat = net.tensor(c + DENSENET121_BLOCKS[0] * growth, h, w)
     net.pool(x, "max", 3, 2, 1, dst=net.view(cat, 0, c))
+    net.feature_ids = {"stem": x}    # tensor ids of the block outputs, by the names oracle/nets_ref.py uses
     for b, nl in enumerate(DENSENET121_BLOCKS, start=1):
         for l in range(1, nl + 1):
             pre = f"features.denseblock{b}.denselayer{l}"
@@ -359,6 +371,7 @@ def build_tucker_densenet121(params, batch=1, H=224, W=224, growth=32):
             else:
                 _dense_layer(net, net.view(cat, 0, c), net.view(cat, c, growth), False, *layer)
             c += growth
+        net.feature_ids[f"denseblock{b}"] = cat
         if b < len(DENSENET121_BLOCKS):
             pre = f"features.transition{b}"
             st, tt = bn_scale_shift(p, pre + ".norm")

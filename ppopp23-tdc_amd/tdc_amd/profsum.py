@@ -7,6 +7,7 @@ geometry (grid, workgroup, LDS) is what tells the layers apart.
     python -m tdc_amd.profsum kernel <dir-with-*_kernel_trace.csv>
     python -m tdc_amd.profsum pmc    <dir-with-*_counter_collection.csv> [--copy-bytes N]
     python -m tdc_amd.profsum timeline <dir-with-*_kernel_trace.csv> --last N
+    python -m tdc_amd.profsum isolated <dir-with-*_kernel_trace.csv> --layers <output of bench.py --isolated-layers>
 
 ``kernel``: count / mean / min / max duration in microseconds per (kernel, grid, workgroup, LDS).
 ``pmc``: mean counter value per (kernel, grid, workgroup); with ``--copy-bytes N`` the FETCH_SIZE /
@@ -14,6 +15,7 @@ WRITE_SIZE readings (KiB) of every kernel are also shown scaled by the reading o
 copy kernel in the same run, which is known to read and write N bytes.
 ``timeline``: the last N dispatches of the trace in launch order (one forward of a network of N kernels):
 start offset, duration, and the idle gap since the previous kernel ended.
+``isolated``: median / p10 kernel duration per benchmark layer from a trace of ``bench.py --isolated-layers``.
 """
 from __future__ import annotations
 
@@ -103,14 +105,53 @@ def timeline(path, last, out=sys.stdout):
         len(rows), (prev_end - t0) * 1e-3, busy, idle))
 
 
+def isolated(path, layers_json, out=sys.stdout):
+    """Kernel-only durations per layer from a trace of ``bench.py --isolated-layers`` (every launch followed by a stream
+    synchronisation, so a kernel's start-to-end time contains no other kernel): the last (layers x launches)
+    convolution dispatches of the trace, in launch order, against the layer list that run printed."""
+    import json
+    info = None
+    for line in open(layers_json):
+        line = line.strip()
+        if line.startswith("{") and "isolated_layers" in line:
+            info = json.loads(line)
+    if info is None:
+        raise SystemExit(f"no --isolated-layers result line in {layers_json}")
+    per = info["launches_per_layer"] - 1          # (the first launch of each layer was its parity check, earlier in the trace)
+    files = sorted(glob.glob(os.path.join(path, "**", "*kernel_trace.csv"), recursive=True))
+    rows = []
+    for f in files:
+        rows += [r for r in csv.DictReader(open(f)) if "tdc_conv" in r["Kernel_Name"]]
+    rows.sort(key=lambda r: int(r["Start_Timestamp"]))
+    need = per * len(info["layers"])
+    if len(rows) < need:
+        raise SystemExit(f"trace holds {len(rows)} convolution dispatches, expected at least {need}")
+    rows = rows[-need:]
+    out.write("# columns: R1 (input channels) R2 (output channels) H=W tile(mf,mb,nb,wm,wn,wk,cch,tw,ks,wl,alg) median_us p10_us"
+              "   | kernel, launches, min_us, max_us\n")
+    for i, (r1, r2, hw, tile) in enumerate(info["layers"]):
+        chunk = rows[i * per:(i + 1) * per]
+        names = {_short(r["Kernel_Name"]) for r in chunk}
+        if len(names) != 1:
+            raise SystemExit(f"layer {i}: the dispatches do not line up with the layer list ({names})")
+        d = sorted((int(r["End_Timestamp"]) - int(r["Start_Timestamp"])) * 1e-3 for r in chunk)
+        out.write("kernel_only_us: %d %d %d %s %.3f %.3f   | %s n=%d min %.3f max %.3f\n" % (
+            r1, r2, hw, ",".join(str(v) for v in tile), d[len(d) // 2], d[len(d) // 10], names.pop(), len(d), d[0], d[-1]))
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser()
-    ap.add_argument("mode", choices=["kernel", "pmc", "timeline"])
+    ap.add_argument("mode", choices=["kernel", "pmc", "timeline", "isolated"])
     ap.add_argument("path")
     ap.add_argument("--copy-bytes", type=int, default=None)
+    ap.add_argument("--layers", default=None, help="isolated: file holding the JSON line bench.py --isolated-layers printed")
     ap.add_argument("--last", type=int, default=64, help="timeline: how many dispatches from the end of the trace")
     a = ap.parse_args(argv)
-    if a.mode == "kernel":
+    if a.mode == "isolated":
+        if not a.layers:
+            raise SystemExit("isolated: --layers <file with the output of bench.py --isolated-layers> is required")
+        isolated(a.path, a.layers)
+    elif a.mode == "kernel":
         kernel_summary(a.path)
     elif a.mode == "timeline":
         timeline(a.path, a.last)

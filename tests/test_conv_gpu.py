@@ -418,63 +418,98 @@ def test_deterministic_bitwise():
     assert np.array_equal(a, b)
 
 
+def _split_rounds(plan, B, C, N, H, W, K, pad, seed, what, reupload_weights=False):
+    """One plan, four launches whose data CHANGES between launches (input x, a new input, x again; optionally new
+    weights for a fourth), each into a NaN-filled output and each checked against the oracle; the first and third
+    must agree bit for bit.  With unchanged data a partial tile left over from the previous launch, or read before
+    its writer had stored it, would still hold the right value and go unseen."""
+    g = seeded(seed)
+    bias = torch.randn(N, generator=g)
+    resid = torch.randn(B, N, plan.Ho, plan.Wo, generator=g)
+    xs = [torch.rand(B, C, H, W, generator=g) * 2 - 1 for _ in range(2)]
+    ws = [torch.empty(N, C, K, K).normal_(0, math.sqrt(2.0 / (C * K * K)), generator=g) for _ in range(2)]
+    plan.set_weights(ws[0], bias)
+    rd = resid.cuda()
+    outs = []
+    rounds = [(0, 0), (1, 0), (0, 0)] + ([(1, 1)] if reupload_weights else [])
+    for xi, wi in rounds:
+        if wi != 0:
+            plan.set_weights(ws[wi], bias)
+        out = torch.full((B, N, plan.Ho, plan.Wo), float("nan"), device="cuda")
+        plan.forward(xs[xi].cuda(), rd, out=out)
+        torch.cuda.synchronize()
+        got = out.cpu().numpy()
+        want = ref.conv2d_c(xs[xi].numpy(), ws[wi].numpy(), bias.numpy(), resid.numpy(), pad=pad, relu=True)
+        assert_close(got, want, f"{what}, launch {len(outs)} (input {xi}, weights {wi})")
+        outs.append(got)
+    assert np.array_equal(outs[0], outs[2]), f"{what}: the same input gave different bits after another launch in between"
+    assert not np.array_equal(outs[0], outs[1])
+
+
 @pytest.mark.parametrize("tile", [tdc_amd.Tile(16, 1, 1, 1, 1, 1, 8, 8, ks=5),      # 5 slices of one pass each
-                                  tdc_amd.Tile(16, 1, 1, 2, 1, 2, 16, 8, ks=2) ,    # 3 passes over 2 slices: 2 + 1
+                                  tdc_amd.Tile(16, 1, 1, 2, 1, 2, 16, 8, ks=2),     # 3 passes over 2 slices: 2 + 1
                                   tdc_amd.Tile(32, 1, 2, 1, 1, 4, 8, 9, ks=3),
+                                  tdc_amd.Tile(16, 1, 1, 1, 1, 1, 4, 8, ks=4),
                                   tdc_amd.Tile(32, 2, 2, 1, 1, 1, 4, 9, ks=10)])
 def test_split_across_workgroups(tile):
-    """Input-channel passes dealt to several workgroups (tile.ks > 1): same answer as the oracle with the whole
-    epilogue, the same bits on every launch, and the ticket counters are back at zero for the next launch."""
+    """Input-channel passes dealt to several workgroups (tile.ks > 1; here 2, 3, 4, 5 and 10 slices at batch 2): the
+    oracle's answer with the whole epilogue on every launch while inputs and weights change between launches, the same
+    bits for the same input, and the ticket counters back at zero for the next launch."""
     announce("ksplit", tile)
     B, C, N, H, W = 2, 40, 37, 9, 9
-    x, w = case(6000, B, C, N, H, W, 3)
-    g = seeded(6001)
-    bias = torch.randn(N, generator=g)
-    resid = torch.randn(B, N, H, W, generator=g)
-    want = ref.conv2d_c(x.numpy(), w.numpy(), bias.numpy(), resid.numpy(), pad=1, relu=True)
-    plan = tdc_amd.Conv2dPlan(B, C, N, H, W, 3, 3, 1, 1, 1, True, True, tile=tile).set_weights(w, bias)
+    plan = tdc_amd.Conv2dPlan(B, C, N, H, W, 3, 3, 1, 1, 1, True, True, tile=tile)
     assert plan.info.grid_z == B * tile.ks
-    xd, rd = x.cuda(), resid.cuda()
-    outs = []
-    for rep in range(3):
-        out = torch.full((B, N, H, W), float("nan"), device="cuda")
-        plan.forward(xd, rd, out=out)
-        torch.cuda.synchronize()
-        outs.append(out.cpu().numpy())
+    _split_rounds(plan, B, C, N, H, W, 3, 1, 6000, f"split-K {tile}", reupload_weights=tile.ks == 5)
     plan.close()
-    assert_close(outs[0], want, f"split-K {tile}")
-    assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2])
 
 
 @pytest.mark.parametrize("shape,K,pad", [((1, 256, 256, 7, 7), 3, 1), ((2, 130, 40, 5, 6), 3, 1), ((1, 2048, 256, 7, 7), 1, 0),
                                          ((2, 300, 24, 3, 5), 1, 0)])
 def test_streamed_tiles_split_across_workgroups(shape, K, pad):
     """Streamed kernels with the input channels dealt to several workgroups (tile.alg = 3 / 4 with tile.ks > 1): the
-    enumeration offers such tiles for layers with few workgroups; every one matches the oracle with the whole epilogue,
-    gives the same bits on every launch (the partial blocks are added in slice order by whichever workgroup comes
-    last), and leaves the ticket counters at zero for the next launch."""
+    enumeration offers such tiles for layers with few workgroups; every one matches the oracle with the whole epilogue
+    on every launch while the input changes between launches (the partial blocks are added in slice order by whichever
+    workgroup comes last), gives the same bits for the same input, and leaves the ticket counters at zero."""
     B, C, N, H, W = shape
-    x, w = case(6100 + C + N, B, C, N, H, W, K)
-    g = seeded(6101)
-    bias = torch.randn(N, generator=g)
-    resid = torch.randn(B, N, H, W, generator=g)
-    want = ref.conv2d_c(x.numpy(), w.numpy(), bias.numpy(), resid.numpy(), pad=pad, relu=True)
     tiles = [t for t in tdc_amd.model_enumerate(tdc_amd.conv_desc(B, C, N, H, W, K, K, 1, pad)) if t.alg >= 3 and t.ks > 1]
     assert tiles and {t.ks for t in tiles} >= {2, 4}
-    xd, rd = x.cuda(), resid.cuda()
-    for t in tiles:
+    for i, t in enumerate(tiles):
         announce("streamed split", shape, K, t)
-        plan = tdc_amd.Conv2dPlan(B, C, N, H, W, K, K, 1, pad, 1, True, True, tile=t).set_weights(w, bias)
+        plan = tdc_amd.Conv2dPlan(B, C, N, H, W, K, K, 1, pad, 1, True, True, tile=t)
         assert plan.info.grid_z == B * t.ks
-        outs = []
-        for rep in range(3):
-            out = torch.full((B, N, H, W), float("nan"), device="cuda")
-            plan.forward(xd, rd, out=out)
-            torch.cuda.synchronize()
-            outs.append(out.cpu().numpy())
+        _split_rounds(plan, B, C, N, H, W, K, pad, 6100 + C + N, f"streamed split {shape} {t}", reupload_weights=i == 0)
         plan.close()
-        assert_close(outs[0], want, f"streamed split {shape} {t}")
-        assert np.array_equal(outs[0], outs[1]) and np.array_equal(outs[0], outs[2])
+
+
+@pytest.mark.parametrize("C,K,pad,alg", [(256, 3, 1, 0), (256, 3, 1, 4), (2048, 1, 0, 0), (2048, 1, 0, 3)])
+def test_split_hand_over_many_launches(C, K, pad, alg):
+    """The hand-over between the workgroups of a split (partials through the workspace, a ticket per tile) over 2000
+    back-to-back launches of one plan on the two layers that rely on it (256 -> 256 @7x7 3x3, 2048 -> 256 @7x7 1x1),
+    staged and streamed kernels.  The input alternates between x and -x: with no bias and no ReLU the two results are
+    exact negations of each other, so a partial tile that is read stale (the previous launch's) or too early flips a
+    sign and cannot hide.  Every launch is compared bit for bit on the device; the test stops at the first mismatch."""
+    N, H, W = 256, 7, 7
+    desc = tdc_amd.conv_desc(1, C, N, H, W, K, K, 1, pad)
+    tiles = [t for t in tdc_amd.model_enumerate(desc) if t.alg == alg and t.ks > 1]
+    assert tiles
+    # the model's favourite among the split tiles of this kernel family
+    tile = min(tiles, key=lambda t: tdc_amd.model_evaluate(desc, t).pred_us)
+    announce("hand-over soak", C, K, tile)
+    x, w = case(6200 + C + alg, 1, C, N, H, W, K)
+    plan = tdc_amd.Conv2dPlan(1, C, N, H, W, K, K, 1, pad, tile=tile).set_weights(w)
+    xp, xn = x.cuda(), (-x).cuda()
+    first = plan.forward(xp)
+    torch.cuda.synchronize()
+    assert_close(first.cpu().numpy(), ref.conv2d_c(x.numpy(), w.numpy(), pad=pad), f"soak reference {tile}")
+    neg = -first
+    out = torch.empty_like(first)
+    for i in range(2000):
+        flip = i & 1
+        out.fill_(float("nan"))
+        plan.forward(xn if flip else xp, out=out)
+        same = torch.equal(out, neg if flip else first)     # (synchronises)
+        assert same, f"launch {i} of {tile}: result differs from the first launch"
+    plan.close()
 
 
 @pytest.mark.parametrize("order", ["0", "1"])
