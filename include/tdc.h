@@ -176,6 +176,18 @@ int tdc_conv_plan_occupancy(const tdc_conv_plan *plan, tdc_kernel_occupancy *out
 /* d_residual may be NULL.  Output need not be pre-zeroed.  Asynchronous. */
 int tdc_conv_forward(tdc_conv_plan *plan, const float *d_in, const float *d_residual,
                      float *d_out, void *stream);
+/* tdc_conv_forward for callers that cannot allocate device memory or hold on to plan-owned scratch: HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  (No counterpart in the reference, whose layer
+ * objects cudaMalloc at will.)  A plan whose tile deals the input channels to several workgroups (tile.ks > 1)
+ * normally keeps their partial tiles and ticket counters in buffers the plan allocated; this entry point places them
+ * in a device array that is part of the library image instead (4 MiB of partial tiles, 64 KiB of counters, one copy
+ * per GPU for the life of the process) and clears the counters with a fill kernel on `stream` before the launch.  It
+ * calls no hipMalloc / hipFree.  TDC_ERR_UNSUPPORTED when batch * ks * N * Ho * Wo * 4 exceeds 4 MiB or the plan has
+ * more than 16384 (image, channel tile, pixel tile) counters.  Results are bit-identical to tdc_conv_forward.
+ * Every call on one GPU shares that GPU's array: calls that can overlap on the device (different streams, or graph
+ * branches) race; serialise them.  Plans with ks = 1 use no scratch and behave exactly like tdc_conv_forward. */
+int tdc_conv_forward_static_ws(tdc_conv_plan *plan, const float *d_in, const float *d_residual,
+                               float *d_out, void *stream);
 /* Same with explicit distances (in floats) between consecutive images of the batch, so that a tensor can be
  * a channel slice of a wider NCHW buffer; 0 = densely packed. */
 int tdc_conv_forward_strided(tdc_conv_plan *plan, const float *d_in, int64_t in_batch_stride,

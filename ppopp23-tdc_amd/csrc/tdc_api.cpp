@@ -522,6 +522,27 @@ int tdc_conv_forward_strided(tdc_conv_plan *plan, const float *d_in, int64_t in_
                         plan->d_ctr, stream);
 }
 
+int tdc_conv_forward_static_ws(tdc_conv_plan *plan, const float *d_in, const float *d_residual, float *d_out, void *stream) {
+    if (!plan) return fail(TDC_ERR_INVALID, "null argument");
+    if (plan->tile.ks <= 1)   // no partial tiles, no counters: nothing to place
+        return forward_impl(plan, d_in, 0, d_residual, 0, d_out, 0, nullptr, nullptr, stream);
+    const size_t ws_bytes = (size_t)plan->geo.grid_z * plan->desc.N * plan->geo.P * sizeof(float);
+    const size_t ctr_bytes = (size_t)plan->desc.batch * plan->geo.grid_y * plan->geo.grid_x * sizeof(unsigned);
+    if (ws_bytes > static_scratch_ws_bytes() || ctr_bytes > static_scratch_ctr_bytes())
+        return fail(TDC_ERR_UNSUPPORTED,
+                    "tdc_conv_forward_static_ws: this plan needs " + std::to_string(ws_bytes) + " bytes of partial tiles and " +
+                        std::to_string(ctr_bytes) + " bytes of counters; the static scratch holds " +
+                        std::to_string(static_scratch_ws_bytes()) + " and " + std::to_string(static_scratch_ctr_bytes()));
+    void *base = nullptr;
+    if (int he = static_scratch_address(&base)) return hip_fail("hipGetSymbolAddress(static scratch)", he);
+    float *ws = reinterpret_cast<float *>(base);
+    unsigned *ctr = reinterpret_cast<unsigned *>(reinterpret_cast<char *>(base) + static_scratch_ws_bytes());
+    // The array keeps whatever the last call (of any plan) left in it: the counters this launch uses must start at
+    // zero.  A fill kernel, not hipMemsetAsync: this call may sit inside a stream capture.
+    if (int he = launch_zero_words(ctr, (int)(ctr_bytes / sizeof(unsigned)), stream)) return hip_fail("counter fill launch", he);
+    return forward_impl(plan, d_in, 0, d_residual, 0, d_out, 0, ws, ctr, stream);
+}
+
 static int forward_impl(tdc_conv_plan *plan, const float *d_in, int64_t in_batch_stride, const float *d_residual,
                         int64_t residual_batch_stride, float *d_out, int64_t out_batch_stride, float *ws, unsigned *ctr,
                         void *stream) {

@@ -183,6 +183,14 @@ int prepare_conv_kernel(const void *fn, const Geometry &g);
 // Enqueue the kernel.  Returns a hipError_t as int.
 int launch_conv(const void *fn, const Geometry &g, const ConvKParams &kp, void *stream);
 
+// Static scratch (a device array that lives from module load to process exit, one copy per GPU) for the partial
+// tiles and ticket counters of a split across workgroups, for callers that cannot allocate.  The address is the
+// CURRENT device's copy (hipGetSymbolAddress, once per device); hipError_t as int.
+size_t static_scratch_ws_bytes();
+size_t static_scratch_ctr_bytes();
+int static_scratch_address(void **ptr_out);
+// dst[0..n) = 0 with a small fill kernel (safe under stream capture, unlike hipMemsetAsync).
+int launch_zero_words(unsigned *dst, int n, void *stream);
 // What the compiled kernel really uses: registers per lane, static LDS, its launch bound, and how many workgroups
 // of `block_threads` threads with `dynamic_lds_bytes` of LDS the runtime places on one compute unit.
 int kernel_resources(const void *fn, int block_threads, int dynamic_lds_bytes, int *vgprs, int *static_lds, int *max_threads,

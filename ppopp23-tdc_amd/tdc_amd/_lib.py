@@ -19,7 +19,7 @@ EXPORTS = (
     "tdc_last_error_string", "tdc_version", "tdc_load_bin", "tdc_save_bin",
     "tdc_conv_plan_create", "tdc_conv_plan_create_with_tail", "tdc_conv_plan_set_tail_weights",
     "tdc_conv_plan_set_weights", "tdc_conv_plan_set_input_affine", "tdc_conv_plan_set_head", "tdc_conv_plan_query",
-    "tdc_conv_forward", "tdc_conv_plan_occupancy",
+    "tdc_conv_forward", "tdc_conv_forward_static_ws", "tdc_conv_plan_occupancy",
     "tdc_conv_forward_strided", "tdc_tkconv_forward_strided",
     "tdc_conv_time", "tdc_conv_time_many", "tdc_conv_plan_destroy",
     "tdc_tkconv_create", "tdc_tkconv_set_weights", "tdc_tkconv_forward", "tdc_tkconv_forward_features",
@@ -103,6 +103,7 @@ def lib():
     L.tdc_conv_plan_set_weights.argtypes = [c_void_p, c_void_p, c_void_p]
     L.tdc_conv_plan_query.argtypes = [c_void_p, POINTER(TileInfo)]
     L.tdc_conv_forward.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]
+    L.tdc_conv_forward_static_ws.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]
     L.tdc_conv_plan_occupancy.argtypes = [c_void_p, POINTER(KernelOccupancy)]
     L.tdc_conv_time.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, POINTER(ctypes.c_float)]
     L.tdc_conv_time_many.argtypes = [POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p), c_int32, c_int32, c_int32,

@@ -112,6 +112,23 @@ class Conv2dPlan:
 
     __call__ = forward
 
+    def forward_static_ws(self, x, residual=None, out=None):
+        """``forward`` through tdc_conv_forward_static_ws: the partial tiles and counters of a split across workgroups
+        live in the library's static device array instead of plan-owned buffers (for callers that cannot allocate)."""
+        d = self.desc
+        _dev_check(x, (d.batch, getattr(self, "head_C", None) or d.C, d.H, d.W), "input")
+        oshape = (d.batch, self.tail[0] if self.tail else d.N, self.Ho, self.Wo)
+        if out is None:
+            out = torch.empty(oshape, device=x.device, dtype=torch.float32)
+        else:
+            _dev_check(out, oshape, "out")
+        rp = None
+        if residual is not None:
+            _dev_check(residual, oshape, "residual")
+            rp = c_void_p(residual.data_ptr())
+        check(lib().tdc_conv_forward_static_ws(self._h, c_void_p(x.data_ptr()), rp, c_void_p(out.data_ptr()), _stream_ptr()))
+        return out
+
     def occupancy(self):
         """What the compiled kernel of this plan uses (registers per lane, resident workgroups per compute unit as the
         HIP runtime computes them) next to the tile model's assumptions: a ``_lib.KernelOccupancy``."""
