@@ -57,14 +57,14 @@ REFERENCE_LAYERS = (
 
 
 def kernel_only_durations():
-    """{(R1, R2, H, tile): (median us, p10 us)} of isolated launches from the committed rocprofv3 kernel-trace summary
+    """{(R1, R2, H): (median us, p10 us, tile)} of isolated launches from the committed rocprofv3 kernel-trace summary
     (lines `kernel_only_us: R1 R2 H tile median p10`)."""
     out = {}
     try:
         for line in open(KERNEL_ONLY_FILE):
             if line.startswith("kernel_only_us:"):
                 f = line.split()
-                out[(int(f[1]), int(f[2]), int(f[3]), tuple(int(v) for v in f[4].split(",")))] = (float(f[5]), float(f[6]))
+                out[(int(f[1]), int(f[2]), int(f[3]))] = (float(f[5]), float(f[6]), [int(v) for v in f[4].split(",")])
     except (OSError, ValueError, IndexError):
         pass
     return out
@@ -240,8 +240,10 @@ def main():
 
     # -- per-layer device time and roofline fraction ------------------------------
     # `us` = launch-to-launch time (median of three runs of 100 graph-replayed launches: what a layer costs inside a
-    # stream of work); `kernel_us` = duration of the kernel alone from the committed rocprofv3 trace of isolated
-    # launches, where one exists for the tile at hand (median, p10).
+    # stream of work); `kernel_us` = begin-to-end duration of the kernel alone from the committed rocprofv3 trace of
+    # isolated launches (every launch followed by a stream synchronisation; median, p10).  An isolated launch starts
+    # on an idle, cold chip and pays its whole dispatch ramp and drain, which back-to-back launches overlap with their
+    # neighbours: it is the LARGER of the two figures for every layer.
     kernel_only = kernel_only_durations()
 
     def layer_row(l):
@@ -251,9 +253,11 @@ def main():
                "roof_us": round(info.roof_us, 4), "frac": round(info.roof_us / us, 4),
                "gflops": round(info.flops / us * 1e-3, 1), "tile": list(info.tile.astuple()),
                "parity_share_of_tolerance": round(l["parity"], 4)}
-        ko = kernel_only.get((l["r1"], l["r2"], l["hw"], tuple(row["tile"])))
+        ko = kernel_only.get((l["r1"], l["r2"], l["hw"]))
         if ko:
             row["kernel_us"] = {"median": ko[0], "p10": ko[1]}
+            if ko[2] != row["tile"]:      # (the measured selection settled on another tile when that trace was taken)
+                row["kernel_us"]["tile"] = ko[2]
         return row
 
     table = []

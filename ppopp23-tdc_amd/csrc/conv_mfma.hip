@@ -55,6 +55,28 @@
 #define TDC_TOUCH_KERNARGS 1
 #endif
 
+// Profiling build only (make STAMPS=1): every wave records s_memrealtime (the 100 MHz constant clock, comparable
+// across compute units and dies) at the boundaries of its phases and leaves the eight values in a plan-owned buffer,
+// [workgroup][wave][8].  The product build compiles none of it.
+#ifndef TDC_STAMPS
+#define TDC_STAMPS 0
+#endif
+#if TDC_STAMPS
+#define TDC_STAMP_DECL unsigned long long tdc_stamp_[8] = {0, 0, 0, 0, 0, 0, 0, 0}
+#define TDC_STAMP(i) tdc_stamp_[i] = __builtin_amdgcn_s_memrealtime()
+#define TDC_STAMP_FLUSH(p, wg, wave, lane)                                                             \
+    do {                                                                                               \
+        if ((p).stamps && (lane) == 0) {                                                               \
+            unsigned long long *dst_ = (p).stamps + ((size_t)(wg) * 16 + (wave)) * 8;                   \
+            for (int i_ = 0; i_ < 8; ++i_) dst_[i_] = tdc_stamp_[i_];                                   \
+        }                                                                                              \
+    } while (0)
+#else
+#define TDC_STAMP_DECL
+#define TDC_STAMP(i)
+#define TDC_STAMP_FLUSH(p, wg, wave, lane)
+#endif
+
 namespace tdc {
 
 typedef float f4_t __attribute__((ext_vector_type(4)));
@@ -110,6 +132,25 @@ constexpr int OOB_OFFSET = 0x7ffffff0;  // beyond any buffer: the load returns z
 
 __device__ __forceinline__ int fdiv(int n, const FastDiv &f) {
     return (int)(__umulhi((unsigned)n, f.m) + ((unsigned)n & f.pass));
+}
+
+// The kernel arguments (about 400 bytes) are read through the scalar cache.  Left alone, the compiler fetches them in
+// several dependent batches, and every batch that touches a cache line for the first time costs a round trip to L2
+// before the first request can go out.  Touch every line of the argument block at once: whatever order the compiler
+// then loads the values in, it hits the scalar cache.
+__device__ __forceinline__ void touch_kernel_arguments() {
+    if constexpr (TDC_TOUCH_KERNARGS) {
+        static_assert(sizeof(ConvKParams) <= 8 * 64, "touch more lines");
+        const auto kargs = __builtin_amdgcn_kernarg_segment_ptr();
+        unsigned t0, t1, t2, t3, t4, t5, t6, t7;
+        asm volatile(
+            "s_load_dword %0, %8, 0x0\n\ts_load_dword %1, %8, 0x40\n\ts_load_dword %2, %8, 0x80\n\t"
+            "s_load_dword %3, %8, 0xc0\n\ts_load_dword %4, %8, 0x100\n\ts_load_dword %5, %8, 0x140\n\t"
+            "s_load_dword %6, %8, 0x180\n\ts_load_dword %7, %8, 0x1c0\n\ts_waitcnt lgkmcnt(0)"
+            : "=&s"(t0), "=&s"(t1), "=&s"(t2), "=&s"(t3), "=&s"(t4), "=&s"(t5), "=&s"(t6), "=&s"(t7)
+            : "s"(kargs)
+            : "memory");
+    }
 }
 
 // Copy planning.  A pass moves the input window of CCH channels and the weight
@@ -202,24 +243,12 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
     using acc_t = typename M::acc_t;
     constexpr int KC = M::KC;
     constexpr int NACC = M::NACC;
+    constexpr bool WINO = TAPS == TAPS_WINO;
     extern __shared__ __align__(16) float lds[];
 
-    // The kernel arguments (about 400 bytes) are read through the scalar cache.  Left alone, the compiler fetches
-    // them in several dependent batches, and every batch that touches a cache line for the first time costs a
-    // round trip to L2 before the first copy can start.  Touch every line of the argument block at once: whatever
-    // order the compiler then loads the values in, it hits the scalar cache.
-    if constexpr (TDC_TOUCH_KERNARGS) {
-        static_assert(sizeof(ConvKParams) <= 8 * 64, "touch more lines");
-        const auto kargs = __builtin_amdgcn_kernarg_segment_ptr();
-        unsigned t0, t1, t2, t3, t4, t5, t6, t7;
-        asm volatile(
-            "s_load_dword %0, %8, 0x0\n\ts_load_dword %1, %8, 0x40\n\ts_load_dword %2, %8, 0x80\n\t"
-            "s_load_dword %3, %8, 0xc0\n\ts_load_dword %4, %8, 0x100\n\ts_load_dword %5, %8, 0x140\n\t"
-            "s_load_dword %6, %8, 0x180\n\ts_load_dword %7, %8, 0x1c0\n\ts_waitcnt lgkmcnt(0)"
-            : "=&s"(t0), "=&s"(t1), "=&s"(t2), "=&s"(t3), "=&s"(t4), "=&s"(t5), "=&s"(t6), "=&s"(t7)
-            : "s"(kargs)
-            : "memory");
-    }
+    touch_kernel_arguments();
+    TDC_STAMP_DECL;
+    TDC_STAMP(0);   // entry
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -239,7 +268,7 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
     const int wn = wave_nk - wm * p.WN;
 
     // pixel lanes of the workgroup (>= TH*TW); a Winograd lane stands for 2x2 pixels
-    const int PT = (TAPS == TAPS_WINO ? 4 : 1) * MF * NB * p.WN;
+    const int PT = (WINO ? 4 : 1) * MF * NB * p.WN;
     const int MT = MF * MB * p.WM;
     // Workgroups are handed to the eight compute dies (XCDs, each with its own L2) round-robin by launch
     // index.  The launch is one-dimensional and the index is re-read as (die, slot), so that each die
@@ -284,7 +313,7 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
 
     // The weight copies of the first pass need no per-lane arithmetic: start them before anything else.
     const int lane16 = lane * 16;
-    if constexpr (TAPS != TAPS_WINO && TAPS != TAPS_3x3G)   // (those paths read their weights from global memory into registers)
+    if constexpr (!WINO && TAPS != TAPS_3x3G)   // (those paths read their weights from global memory into registers)
         issue_weights<EXT>(p, w_rsrc, lds, lane16, (int)(w_byte_base + (unsigned)chunk0 * w_pass_bytes), wave, nwaves, chunk0);
 
     // Offsets of this lane's elements in its wave's first MAXPRE input blocks (pass 0), for the steady dealing
@@ -327,7 +356,7 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
         // Copy issue competes for the SIMD with other waves' MFMA streams and loses by default (measured:
         // ~330 cycles per copy instruction instead of ~115); it is short, so let it go first.
         __builtin_amdgcn_s_setprio(3);
-        if constexpr (TAPS != TAPS_WINO && TAPS != TAPS_3x3G) issue_weights<EXT>(p, w_rsrc, stage, lane16, w_byte0, dw, dn, chunk);
+        if constexpr (!WINO && TAPS != TAPS_3x3G) issue_weights<EXT>(p, w_rsrc, stage, lane16, w_byte0, dw, dn, chunk);
         issue_inputs(p, in_rsrc, stage, pre, true, chunk, iy0, ix0a, dw, dn, lane);
         __builtin_amdgcn_s_setprio(0);
     };
@@ -347,7 +376,7 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
     // exists (lanes past the workgroup tile re-read its last row of tiles and are never stored).
     int wino_off = 0, wino_ty = 0, wino_tx = 0;
     bool wino_live = false;
-    if constexpr (TAPS == TAPS_WINO) {
+    if constexpr (WINO) {
         const int j = wn * 16 + (lane & 15);
         const int tht = p.TH >> 1;
         int ty = fdiv(j, p.fd_wtw);
@@ -357,8 +386,8 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
         wino_ty = ty;
         wino_off = 2 * ty * p.RS + 2 * wino_tx + (ix0 - ix0a) + (lane >> 4) * p.CS;
     }
-    f4_t wacc[TAPS == TAPS_WINO ? 16 : 1];
-    if constexpr (TAPS == TAPS_WINO) {
+    f4_t wacc[WINO ? 16 : 1];
+    if constexpr (WINO) {
 #pragma unroll
         for (int x = 0; x < 16; ++x) wacc[x] = (f4_t){0.0f, 0.0f, 0.0f, 0.0f};
     }
@@ -371,20 +400,23 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
 #pragma unroll
             for (int v = 0; v < NACC; ++v) acc[mb][nb][v] = 0.0f;
 
-    const int taps = (TAPS == TAPS_GENERIC) ? p.KH * p.KW : (TAPS == TAPS_3x3G) ? 9 : TAPS;
+    const int taps = (TAPS == TAPS_GENERIC) ? p.KH * p.KW : (TAPS == TAPS_3x3G) ? 9 : WINO ? 16 : TAPS;
     const int ncg_pass = p.CCH / KC;  // channel groups per pass
     const int ncgw = p.CPW / KC;      // ... of which this wave takes [wk*ncgw, (wk+1)*ncgw)
 
     // Winograd: the A operands come from global memory and do not depend on the staged input, so the first group
     // of every pass is requested before the wait and the barrier of that pass and is in registers when they end.
-    f4_t wu0[TAPS == TAPS_WINO ? 4 : 1];
+    f4_t wu0[WINO ? 4 : 1];
     auto wino_load_a = [&](int chunk, int g, f4_t(&u)[4]) {
+#if defined(TDC_PROBE) && (TDC_PROBE & 1)
+        if (g > 0) return;   // timing probe (wrong results): no weight requests inside the loop
+#endif
         const int soff = (int)(w_byte_base + (unsigned)chunk * w_pass_bytes) + ((wm * ncg_pass + wk * ncgw + g) * 16) * 256;
 #pragma unroll
         for (int q = 0; q < 4; ++q)
             u[q] = __builtin_bit_cast(f4_t, __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, lane16, soff + q * 1024, 0));
     };
-    if constexpr (TAPS == TAPS_WINO) {
+    if constexpr (WINO) {
         if (!loader) wino_load_a(chunk0, 0, wu0);
     }
     // Direct 3x3 with weights from global memory: a group is a PAIR of channel groups (18 K-steps per block, long
@@ -413,11 +445,14 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
         if (!loader) g3_load_a(chunk0, 0, ga0);
     }
 
+    TDC_STAMP(1);   // first copies issued, offsets and operand addresses worked out
     for (int chunk = chunk0; chunk < chunk1; ++chunk) {
         // My copies of this pass have landed; after the barrier everybody's have, and
         // everybody is done reading the stage the next pass is about to overwrite.
         __builtin_amdgcn_s_waitcnt(0);
+        if (chunk == chunk0) TDC_STAMP(2);   // my first copies have landed
         __syncthreads();
+        if (chunk == chunk0) TDC_STAMP(3);   // everybody's have
         if (chunk + 1 < chunk1) issue(chunk + 1);
         if constexpr (EXT && TAPS == TAPS_1x1) {
             // Optional per-input-channel affine (+ReLU) in front of the convolution (an inference BatchNorm that
@@ -480,12 +515,12 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
         for (int mb = 0; mb < MB; ++mb)
             sw[mb] = stage + p.in_stage_floats + (((wm * MB + mb) * ncg_pass + wk * ncgw) * taps) * 64 + lane;
 
-        if constexpr (TAPS == TAPS_WINO) {
+        if constexpr (WINO) {
             // One group = four input channels: 16 raw patch values per lane (8 two-word LDS reads), the 16 A
             // operands (four 128-bit reads), the register transform, 16 MFMAs.  Two register sets ping-pong as
             // in the direct loops: patch and weights of group g+1 are read, and the patch transformed, between the
             // MFMAs of group g.
-            static_assert(TAPS != TAPS_WINO || (MF == 16 && MB == 1 && NB == 1), "Winograd path: one 16x16 block per wave");
+            static_assert(!WINO || (MF == 16 && MB == 1 && NB == 1), "Winograd path: one 16x16 block per wave");
             const float *praw = sin + wino_off;
             // A operands: straight from the packed weights in global memory (L2), 16 bytes per lane and quarter,
             // one group ahead like the patch reads; the scalar operand carries everything but the lane.
@@ -494,12 +529,21 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
             float v0[16], v1[16];
             f4_t u1[4];
             auto load_patch = [&](int g, float(&v)[16]) {
+#if defined(TDC_PROBE) && (TDC_PROBE & 2)
+                if (g > 0) return;   // timing probe (wrong results): no patch reads and no input transform inside the loop
+#endif
                 const float *b = praw + g * gstep;
                 float d[4][4];
 #pragma unroll
                 for (int r = 0; r < 4; ++r)
 #pragma unroll
                     for (int c = 0; c < 4; ++c) d[r][c] = b[r * RS + c];
+#if defined(TDC_PROBE) && (TDC_PROBE & 4)
+                // timing probe (wrong results): the patch is read but not transformed
+#pragma unroll
+                for (int i = 0; i < 16; ++i) v[i] = d[i >> 2][i & 3];
+                return;
+#endif
                 float tr[4][4];   // B^T d: rows
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {
@@ -760,9 +804,10 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
             }
         }
     }
+    TDC_STAMP(4);   // all passes done
     // Epilogue.  `each_output(sink)` walks this thread's share of the workgroup's output tile and
     // hands (channel, pixel offset in the image, accumulated value) to the sink.
-    if constexpr (TAPS == TAPS_WINO) {
+    if constexpr (WINO) {
         // Output transform Y = A^T M A, A^T = [1 1 1 0; 0 1 -1 -1], per accumulator register (= output channel):
         // all 16 positions of a tile sit in the same lane.  The 2x2 results are parked in LDS as
         // [wk][channel][pixel of the workgroup tile]; the walk below adds the WK slices in index order and stores
@@ -787,6 +832,7 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
             }
         }
         __syncthreads();
+        TDC_STAMP(5);   // output transform parked, everybody's
     } else if (p.WK > 1) {
         // Split-K across waves: park every wave's partial tile in LDS
         // ([wk][channel][pixel lane]); the walk below adds the WK slices in index order.
@@ -808,7 +854,7 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
         __syncthreads();
     }
     auto each_output = [&](auto &&sink, bool want_value) {
-        if (p.WK == 1 && TAPS != TAPS_WINO) {
+        if (p.WK == 1 && !WINO) {
             // Straight from the accumulators: each store instruction writes runs of
             // consecutive pixels of one output channel.
 #pragma unroll
@@ -953,7 +999,7 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
         return;
     }
     if (p.KS == 1) {
-        if constexpr (TAPS == TAPS_WINO) {
+        if constexpr (WINO) {
             // The parked tile rows are runs of TW (even) consecutive pixels: where image width and the output
             // address allow it, every thread finishes four (or two) consecutive pixels of one channel with one wide
             // LDS read per slice and one wide store.
@@ -989,14 +1035,20 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
             typedef float f2_t __attribute__((ext_vector_type(2)));
             if (((p.TW | p.Wo) & 3) == 0 && (stride_bits & 3) == 0 && (addr_bits & 15ull) == 0) {
                 walk(f4_t{});
+                TDC_STAMP(6);   // stores issued
+                TDC_STAMP_FLUSH(p, logical, wave, lane);
                 return;
             }
             if ((p.Wo & 1) == 0 && (stride_bits & 1) == 0 && (addr_bits & 7ull) == 0) {
                 walk(f2_t{});
+                TDC_STAMP(6);
+                TDC_STAMP_FLUSH(p, logical, wave, lane);
                 return;
             }
         }
         each_output(finish, true);
+        TDC_STAMP(6);
+        TDC_STAMP_FLUSH(p, logical, wave, lane);
         return;
     }
 
@@ -1122,18 +1174,7 @@ template <int NQ, bool AFF, int MODE>
 __global__ void __launch_bounds__(NQ == 8 ? 512 : 1024) tdc_conv1x1_stream_kernel(const ConvKParams p) {
     constexpr bool SPLIT = MODE == 1, STRIDED = MODE == 2;
     extern __shared__ __align__(16) float lds[];
-    if constexpr (TDC_TOUCH_KERNARGS) {
-        static_assert(sizeof(ConvKParams) <= 8 * 64, "touch more lines");
-        const auto kargs = __builtin_amdgcn_kernarg_segment_ptr();
-        unsigned t0, t1, t2, t3, t4, t5, t6, t7;
-        asm volatile(
-            "s_load_dword %0, %8, 0x0\n\ts_load_dword %1, %8, 0x40\n\ts_load_dword %2, %8, 0x80\n\t"
-            "s_load_dword %3, %8, 0xc0\n\ts_load_dword %4, %8, 0x100\n\ts_load_dword %5, %8, 0x140\n\t"
-            "s_load_dword %6, %8, 0x180\n\ts_load_dword %7, %8, 0x1c0\n\ts_waitcnt lgkmcnt(0)"
-            : "=&s"(t0), "=&s"(t1), "=&s"(t2), "=&s"(t3), "=&s"(t4), "=&s"(t5), "=&s"(t6), "=&s"(t7)
-            : "s"(kargs)
-            : "memory");
-    }
+    touch_kernel_arguments();
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // = this wave's slice of the input channels
@@ -1256,17 +1297,7 @@ template <int CG, bool ROW, int MODE>
 __global__ void __launch_bounds__(1024) tdc_conv3x3_stream_kernel(const ConvKParams p) {
     constexpr bool SPLIT = MODE == 1, TAIL = MODE == 2 || MODE == 3, HEAD = MODE == 3;
     extern __shared__ __align__(16) float lds[];
-    if constexpr (TDC_TOUCH_KERNARGS) {
-        const auto kargs = __builtin_amdgcn_kernarg_segment_ptr();
-        unsigned t0, t1, t2, t3, t4, t5, t6, t7;
-        asm volatile(
-            "s_load_dword %0, %8, 0x0\n\ts_load_dword %1, %8, 0x40\n\ts_load_dword %2, %8, 0x80\n\t"
-            "s_load_dword %3, %8, 0xc0\n\ts_load_dword %4, %8, 0x100\n\ts_load_dword %5, %8, 0x140\n\t"
-            "s_load_dword %6, %8, 0x180\n\ts_load_dword %7, %8, 0x1c0\n\ts_waitcnt lgkmcnt(0)"
-            : "=&s"(t0), "=&s"(t1), "=&s"(t2), "=&s"(t3), "=&s"(t4), "=&s"(t5), "=&s"(t6), "=&s"(t7)
-            : "s"(kargs)
-            : "memory");
-    }
+    touch_kernel_arguments();
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1525,6 +1556,154 @@ __global__ void __launch_bounds__(1024) tdc_conv3x3_stream_kernel(const ConvKPar
 }
 
 // ---------------------------------------------------------------------------
+// The streamed 3x3 kernel with NB pixel blocks per wave (tile.alg = 4, tile.nb = 2 or 4; stride 1, rows of 14 pixels).
+// The 16 x 16 block of the plain kernel reads the weights of its 16 channels once per 16 pixels and moves 30 times the
+// algorithmic bytes through the L2s on the mid-size layers (64 -> 64 @56x56: 54 MB for 1.75 MB), which is what bounds
+// them.  Here a workgroup owns NB horizontally adjacent 14-pixel row tiles: a wave still takes CG groups of four input
+// channels and requests everything up front, but every weight operand it holds feeds NB MFMAs, one per pixel block,
+// so the weights cross the L2 -> CU path NB times less often.  Per group and block a lane requests three values (one
+// per filter row; the three taps of a row are lane shifts, as in the plain kernel's row mode).  The partial blocks
+// of the WK waves meet in LDS as [wave][block][register][lane] and ALL threads share the final sum (in wave order, so
+// the result does not depend on timing) and the store.
+// ---------------------------------------------------------------------------
+template <int CG, int NB>
+__global__ void __launch_bounds__(1024) tdc_conv3x3_stream_rownb_kernel(const ConvKParams p) {
+    extern __shared__ __align__(16) float lds[];
+    TDC_STAMP_DECL;
+    TDC_STAMP(0);   // entry
+    touch_kernel_arguments();
+    TDC_STAMP(7);   // every line of the kernel arguments is in the scalar cache
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int logical = (int)(blockIdx.x & 7u) * p.xcd_chunk + (int)(blockIdx.x >> 3);
+    if (logical >= p.n_wg) return;
+    const int q1 = fdiv(logical, p.fd_g1);
+    const int r1 = logical - q1 * p.fd_g1.d;
+    const int img = fdiv(q1, p.fd_g2);
+    const int r2 = q1 - img * p.fd_g2.d;
+    const int bx = p.channel_major ? r1 : r2;  // pixel tile of the workgroup: NB blocks side by side
+    const int by = p.channel_major ? r2 : r1;  // channel tile
+    const int tile_y = fdiv(bx, p.fd_ntx);     // = output row (tiles are one row high)
+    const int tile_x = bx - tile_y * p.ntx;
+    const float *__restrict__ in = p.in + (long long)img * p.in_bstride;
+    float *__restrict__ out = p.out + (long long)img * p.out_bstride;
+    const float *__restrict__ resid = p.resid ? p.resid + (long long)img * p.resid_bstride : nullptr;
+    const __amdgpu_buffer_rsrc_t in_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(in), (short)0, (int)p.in_image_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t w_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.wpk), (short)0, (int)p.wpk_bytes, 0x00020000);
+
+    // wave = (channel block of the workgroup) * WK + (slice of the input channels)
+    const int wmi = fdiv(wave, p.fd_wk);
+    const int wki = wave - wmi * p.WK;
+    // weights first: they depend on nothing but the channel block and the wave (packed as for the plain kernel)
+    const int a_soff = (((by * p.WM + wmi) * (p.CCH >> 2)) + wki * CG) * 2304;
+    f4_t a0[CG], a1[CG];
+    float a8[CG];
+#pragma unroll
+    for (int g = 0; g < CG; ++g) {
+        a0[g] = __builtin_bit_cast(f4_t, __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, lane * 16, a_soff + g * 2304, 0));
+        a1[g] = __builtin_bit_cast(f4_t, __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, lane * 16, a_soff + g * 2304 + 1024, 0));
+        a8[g] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(w_rsrc, lane * 4, a_soff + g * 2304 + 2048, 0));
+    }
+    __builtin_amdgcn_sched_barrier(0);
+
+    const int k = lane >> 4, n = lane & 15;
+    const unsigned chan_bytes = (unsigned)(p.H * p.W) * 4u;
+    const unsigned base = (unsigned)(wki * (4 * CG) + k) * chan_bytes;   // this lane's first channel
+    // lane n of a quarter: input column (block's first column - pad + n) of the three input rows under the output row
+    const int iyr = tile_y - p.pad;
+    unsigned roff[NB][3];
+#pragma unroll
+    for (int blk = 0; blk < NB; ++blk) {
+        const int ixr = (tile_x * NB + blk) * 14 - p.pad + n;
+#pragma unroll
+        for (int r = 0; r < 3; ++r) {
+            const bool ok = (unsigned)(iyr + r) < (unsigned)p.H && (unsigned)ixr < (unsigned)p.W;
+            const unsigned m = ok ? 0xffffffffu : 0u;
+            roff[blk][r] = ((unsigned)((iyr + r) * p.W + ixr) * 4u & m) | ((unsigned)OOB_OFFSET & ~m);
+        }
+    }
+    float rowv[CG][NB][3];
+#pragma unroll
+    for (int g = 0; g < CG; ++g) {
+#pragma unroll
+        for (int blk = 0; blk < NB; ++blk)
+#pragma unroll
+            for (int r = 0; r < 3; ++r)
+                rowv[g][blk][r] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                    in_rsrc, (int)(roff[blk][r] + base + (unsigned)(4 * g) * chan_bytes), 0, 0));
+        __builtin_amdgcn_sched_barrier(0);   // requests in the order the MFMAs consume them
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    TDC_STAMP(1);   // every request issued
+    f4_t acc[NB];
+#pragma unroll
+    for (int blk = 0; blk < NB; ++blk) acc[blk] = (f4_t){0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int g = 0; g < CG; ++g) {
+#pragma unroll
+        for (int r = 0; r < 3; ++r) {
+#pragma unroll
+            for (int c = 0; c < 3; ++c) {
+                const int t = r * 3 + c;
+                const float av = t < 4 ? a0[g][t] : t < 8 ? a1[g][t - 4] : a8[g];
+#pragma unroll
+                for (int blk = 0; blk < NB; ++blk) {
+                    const int v = __builtin_bit_cast(int, rowv[g][blk][r]);
+                    // row_shl:c within the 16 lanes of a quarter: lane n takes the value of lane n + c
+                    const float bv = c == 0 ? rowv[g][blk][r]
+                                   : c == 1 ? __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, v, 0x101, 0xf, 0xf, true))
+                                            : __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, v, 0x102, 0xf, 0xf, true));
+                    acc[blk] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, bv, acc[blk], 0, 0, 0);
+                }
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);   // group by group, as the data arrives
+    }
+    TDC_STAMP(4);   // MFMAs issued (the last results may still be in the pipe)
+    // lane l of block blk holds rows 4*(l/16) .. +3 (output channels) of column l%16 (pixel)
+#pragma unroll
+    for (int blk = 0; blk < NB; ++blk)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) lds[((wave * NB + blk) * 4 + i) * 64 + lane] = acc[blk][i];
+    __syncthreads();
+    TDC_STAMP(5);   // everybody's partial blocks are in LDS
+    const int nthreads = blockDim.x;
+    const int total = p.WM * NB * 256;
+    for (int idx = tid; idx < total; idx += nthreads) {
+        const int l = idx & 63, i = (idx >> 6) & 3;
+        const int rest = idx >> 8;                     // = channel block of the workgroup * NB + pixel block
+        const int cb = rest / NB, blk = rest - cb * NB;
+        const float *src = lds + (((cb * p.WK) * NB + blk) * 4 + i) * 64 + l;
+        const int wstride = NB * 256;
+        float val = 0.0f;
+        // four reads in flight at a time; the additions stay in wave order
+        for (int w0 = 0; w0 < p.WK; w0 += 4) {
+            float part[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) part[u] = src[min(w0 + u, p.WK - 1) * wstride];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                if (w0 + u < p.WK) val += part[u];
+        }
+        const int ch = (by * p.WM + cb) * 16 + 4 * (l >> 4) + i;
+        const int px = l & 15;
+        const int ox = (tile_x * NB + blk) * 14 + px;
+        if (ch < p.N && px < 14 && ox < p.Wo) {
+            if (p.bias) val += p.bias[ch];
+            const long long o = (long long)ch * p.P + tile_y * p.Wo + ox;
+            if (resid) val += resid[o];
+            if (p.relu) val = fmaxf(val, 0.0f);
+            out[o] = val;
+        }
+    }
+    TDC_STAMP(6);   // stores issued
+    TDC_STAMP_FLUSH(p, logical, wave, lane);
+}
+
+// ---------------------------------------------------------------------------
 // Instantiation table: KernelId (worked out on the host from tile and filter, see kernel_id_for) -> function.
 // A 2x2 block grid of MFMAs per wave is built for at most 8 waves per workgroup (256 registers per lane), the
 // Winograd loop for 12, everything else for 16.
@@ -1590,6 +1769,17 @@ const void *kernel_function(const KernelId &k) {
         const int nq = k.p[0], mode = k.p[2];
         if (k.p[1]) fn = mode == 2 ? pick_stream<true, 2>(nq) : mode == 1 ? pick_stream<true, 1>(nq) : mode == 0 ? pick_stream<true, 0>(nq) : nullptr;
         else fn = mode == 2 ? pick_stream<false, 2>(nq) : mode == 1 ? pick_stream<false, 1>(nq) : mode == 0 ? pick_stream<false, 0>(nq) : nullptr;
+    } else if (k.family == KernelId::STREAM_3x3 && k.p[3] > 1) {
+        // NB pixel blocks per wave: rows of 14 pixels, plain mode only
+        const int cg = k.p[0], nb = k.p[3];
+        if (k.p[1] && k.p[2] == 0) {
+            if (nb == 2) fn = cg == 1 ? static_cast<kernel_fn>(tdc_conv3x3_stream_rownb_kernel<1, 2>)
+                            : cg == 2 ? static_cast<kernel_fn>(tdc_conv3x3_stream_rownb_kernel<2, 2>)
+                            : cg == 4 ? static_cast<kernel_fn>(tdc_conv3x3_stream_rownb_kernel<4, 2>) : nullptr;
+            if (nb == 4) fn = cg == 1 ? static_cast<kernel_fn>(tdc_conv3x3_stream_rownb_kernel<1, 4>)
+                            : cg == 2 ? static_cast<kernel_fn>(tdc_conv3x3_stream_rownb_kernel<2, 4>)
+                            : cg == 4 ? static_cast<kernel_fn>(tdc_conv3x3_stream_rownb_kernel<4, 4>) : nullptr;
+        }
     } else if (k.family == KernelId::STREAM_3x3) {
         const int cg = k.p[0], mode = k.p[2];
         if (k.p[1]) fn = mode == 2 ? pick_stream3<true, 2>(cg) : mode == 1 ? pick_stream3<true, 1>(cg) : mode == 0 ? pick_stream3<true, 0>(cg) : nullptr;

@@ -61,9 +61,29 @@ struct tdc_conv_plan {
     bool have_tail_weights = false;
     int in_relu = 0;
     bool have_weights = false;
+#if defined(TDC_STAMPS) && TDC_STAMPS
+    unsigned long long *d_stamps = nullptr;   // profiling build: per-wave time stamps of the last launch
+    size_t stamp_words = 0;
+#endif
 };
 
+#if defined(TDC_STAMPS) && TDC_STAMPS
+// Profiling build only: copy the time stamps of the plan's last launch to the host, [workgroup][16 waves][8]
+// values of the 100 MHz constant clock (0 = that wave wrote nothing); *words_out = how many were written.
+extern "C" int tdc_debug_read_stamps(tdc_conv_plan *plan, unsigned long long *host_out, uint64_t cap, uint64_t *words_out) {
+    if (!plan || !host_out || !words_out) return (int)TDC_ERR_INVALID;
+    const size_t n = std::min<size_t>(plan->stamp_words, (size_t)cap);
+    if (hipMemcpy(host_out, plan->d_stamps, n * 8, hipMemcpyDeviceToHost) != hipSuccess) return (int)TDC_ERR_HIP;
+    *words_out = n;
+    return TDC_OK;
+}
+#endif
+
 static void free_plan_buffers(tdc_conv_plan *p) {
+#if defined(TDC_STAMPS) && TDC_STAMPS
+    if (p->d_stamps) (void)hipFree(p->d_stamps);
+    p->d_stamps = nullptr;
+#endif
     if (p->d_wpk) (void)hipFree(p->d_wpk);
     if (p->d_bias) (void)hipFree(p->d_bias);
     if (p->d_ws) (void)hipFree(p->d_ws);
@@ -367,6 +387,15 @@ int tdc_conv_plan_create_with_tail(const tdc_conv_desc *desc, int32_t tail_N, in
             return hip_fail("hipMalloc(split-K workspace)", e);
         }
     }
+#if defined(TDC_STAMPS) && TDC_STAMPS
+    p->stamp_words = (size_t)p->geo.grid_x * p->geo.grid_y * p->geo.grid_z * 16 * 8;
+    e = hipMalloc((void **)&p->d_stamps, p->stamp_words * 8);
+    if (e == hipSuccess) e = hipMemset(p->d_stamps, 0, p->stamp_words * 8);
+    if (e != hipSuccess) {
+        free_plan_buffers(p.get());
+        return hip_fail("hipMalloc(time stamps)", e);
+    }
+#endif
     *plan_out = p.release();
     return TDC_OK;
 }
@@ -613,6 +642,9 @@ static int forward_impl(tdc_conv_plan *plan, const float *d_in, int64_t in_batch
     kp.fd_g1 = make_fastdiv(g.channel_major ? g.grid_x : g.grid_y);
     kp.fd_g2 = make_fastdiv(g.channel_major ? g.grid_y : g.grid_x);
     kp.wpk_bytes = (unsigned)(packed_weight_floats(g) * sizeof(float));
+#if defined(TDC_STAMPS) && TDC_STAMPS
+    kp.stamps = plan->d_stamps;
+#endif
     int he = launch_conv(plan->kernel, g, kp, stream);
     if (he) return hip_fail("kernel launch", he);
     return TDC_OK;

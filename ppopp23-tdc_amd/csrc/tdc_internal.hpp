@@ -146,6 +146,9 @@ struct ConvKParams {
     long long in_bstride;      // floats between consecutive images of the input (C*H*W when dense)
     long long out_bstride;     // ... of the output (N*P when dense)
     long long resid_bstride;   // ... of the residual
+#if defined(TDC_STAMPS) && TDC_STAMPS
+    unsigned long long *stamps;   // profiling build: [workgroup][16 waves][8] time stamps, or null
+#endif
 };
 
 // Inner loop of the staged kernel (its TAPS template argument).
@@ -155,7 +158,8 @@ enum : int { TAPS_GENERIC = 0, TAPS_1x1 = 1, TAPS_3x3 = 9, TAPS_3x3G = 10, TAPS_
 // launcher and the occupancy probe all speak of the same function.
 //   STAGED      tdc_conv_mfma_kernel<MF, MB, NB, TAPS, MAXW, EXT>     p = {MF, MB, NB, TAPS, MAXW, EXT}
 //   STREAM_1x1  tdc_conv1x1_stream_kernel<NQ, AFF, MODE>              p = {NQ, AFF, MODE}
-//   STREAM_3x3  tdc_conv3x3_stream_kernel<CG, ROW, MODE>              p = {CG, ROW, MODE}
+//   STREAM_3x3  tdc_conv3x3_stream_kernel<CG, ROW, MODE>              p = {CG, ROW, MODE, 1}
+//               tdc_conv3x3_stream_rownb_kernel<CG, NB>               p = {CG, 1, 0, NB}   (NB = 2 or 4 pixel blocks per wave)
 struct KernelId {
     enum Family : int { NONE = 0, STAGED = 1, STREAM_1x1 = 2, STREAM_3x3 = 3 };
     int family = NONE;

@@ -112,7 +112,8 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
     };
     if (!check_desc(d, why)) return false;
     if (t.mf != 32 && t.mf != 16) return fail("tile.mf must be 16 or 32");
-    if (t.mb < 1 || t.mb > 2 || t.nb < 1 || t.nb > 2) return fail("tile.mb / tile.nb must be 1 or 2");
+    if (t.mb < 1 || t.mb > 2 || t.nb < 1 || (t.nb > 2 && !(t.alg == 4 && t.nb == 4)))
+        return fail("tile.mb / tile.nb must be 1 or 2 (tile.nb may be 4 for tile.alg = 4)");
     if (t.wm < 1 || t.wn < 1 || t.wk < 1) return fail("tile.wm / wn / wk must be >= 1");
     g = Geometry();
     // (256 registers per lane for the 2x2 block grid, 168 for the Winograd path)
@@ -138,7 +139,13 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
         // 3x3 convolution streamed from global memory: 16 channels x 16 pixels per workgroup, the input channels
         // split over wk waves in groups of four, everything in one pass
         if (d.KH != 3 || d.KW != 3 || d.dilation != 1) return fail("tile.alg = 4 needs a 3x3 / dilation 1 convolution");
-        if (t.mf != 16 || t.mb != 1 || t.nb != 1 || t.wn != 1) return fail("tile.alg = 4 needs mf = 16 and one pixel block per workgroup");
+        if (t.mf != 16 || t.mb != 1 || t.wn != 1) return fail("tile.alg = 4 needs mf = 16, mb = 1, wn = 1");
+        if (t.nb != 1) {
+            // nb pixel blocks per wave (the weights a wave holds feed nb MFMAs each): rows of 14 pixels, stride 1
+            if (d.stride != 1 || t.tw != 14) return fail("tile.alg = 4 with nb > 1 needs stride 1 and tw = 14");
+            if (t.nb > ceil_div(g.Wo, 14)) return fail("tile.alg = 4: more pixel blocks per wave than an image row has 14-pixel tiles");
+            if (tail_N > 0 || t.ks != 1) return fail("tile.alg = 4 with nb > 1 has no fused tail and no split across workgroups");
+        }
         if (t.wm * t.wk > 16) return fail("tile.alg = 4: at most 16 waves (wm channel blocks x wk channel slices)");
         if (t.wl != 0) return fail("tile.alg = 4 has no loader waves");
         const int groups = (t.cch % (4 * t.wk) == 0) ? t.cch / (4 * t.wk) : 0;
@@ -190,8 +197,10 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
         if (t.tw < 1 || t.tw > g.PT || (!runs && t.tw > g.Wo)) return fail("tile.tw must be in [1, min(Wo, pixel lanes)]");
         g.TW = t.tw;
         g.TH = runs ? 1 : std::min(g.PT / t.tw, g.Ho);
+        if (t.alg == 4) g.TH = std::min(16 / t.tw, g.Ho);   // (a block is 16 pixel lanes, whatever nb is)
     }
     g.ntx = ceil_div(g.Wo, g.TW);
+    if (t.alg == 4 && t.nb > 1) g.ntx = ceil_div(g.ntx, t.nb);   // a workgroup takes nb neighbouring tiles of a row
     g.nty = ceil_div(g.Ho, g.TH);
     if (t.alg == 3 && !flat) {
         g.ntx = ceil_div(g.P, 16);
@@ -245,7 +254,8 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
     g.nstage = g.cps > 1 ? 2 : 1;
     const long long stage_bytes = (long long)g.nstage * g.stage_floats * 4;
     // (the Winograd path always parks its output tiles in LDS, also without a split over waves)
-    const long long red_bytes = (t.wk > 1 || t.alg == 1) ? (long long)t.wk * g.MT * g.PT * 4 : 0;
+    // (... and so does the streamed 3x3 kernel with several pixel blocks per wave: all its threads share the final store)
+    const long long red_bytes = (t.wk > 1 || t.alg == 1 || (t.alg == 4 && t.nb > 1)) ? (long long)t.wk * g.MT * g.PT * 4 : 0;
     long long lds = std::max(stage_bytes, red_bytes);
     if (tail_N > 0) {
         // A fused 1x1 tail needs every output channel of the convolution in one workgroup; its tile is parked
@@ -431,7 +441,7 @@ KernelId kernel_id_with_head(const tdc_tile &t) {
     const int cg = t.cch / (4 * t.wk);
     if (cg != 1 && cg != 2 && cg != 4) return k;
     k.family = KernelId::STREAM_3x3;
-    k.p[0] = cg; k.p[1] = 0; k.p[2] = 3;
+    k.p[0] = cg; k.p[1] = 0; k.p[2] = 3; k.p[3] = 1;
     return k;
 }
 
@@ -439,15 +449,21 @@ KernelId kernel_id_for(const tdc_tile &t, int KH, int KW, int dilation, int stri
     KernelId k;
     if (t.alg == 4) {
         // (`extras` can only mean a fused tail here, which the one kernel carries)
-        if (KH != 3 || KW != 3 || dilation != 1 || t.mf != 16 || t.mb != 1 || t.nb != 1 || t.wm < 1 || t.wn != 1 || t.wk < 1 ||
+        if (KH != 3 || KW != 3 || dilation != 1 || t.mf != 16 || t.mb != 1 || t.wm < 1 || t.wn != 1 || t.wk < 1 ||
             t.wm * t.wk > 16 || t.cch % (4 * t.wk) != 0)
             return k;
         const int cg = t.cch / (4 * t.wk);
         if ((cg != 1 && cg != 2 && cg != 4) || (extras && t.ks > 1)) return k;
+        const bool row = stride == 1 && t.tw == 14;   // one row of 14 pixels: the taps of a filter row are lane shifts
+        if (t.nb != 1) {
+            // several pixel blocks per wave: row tiles, no extras, no split across workgroups
+            if ((t.nb != 2 && t.nb != 4) || !row || extras || t.ks > 1) return k;
+        }
         k.family = KernelId::STREAM_3x3;
         k.p[0] = cg;
-        k.p[1] = stride == 1 && t.tw == 14;   // one row of 14 pixels: the taps of a filter row are lane shifts
+        k.p[1] = row;
         k.p[2] = extras ? 2 : t.ks > 1 ? 1 : 0;
+        k.p[3] = t.nb;
         return k;
     }
     if (t.alg == 3) {
@@ -493,7 +509,8 @@ std::string kernel_name(const KernelId &k) {
             std::snprintf(buf, sizeof buf, "tdc_conv1x1_stream_kernel<%d, %s, %d>", k.p[0], tf[k.p[1] != 0], k.p[2]);
             break;
         case KernelId::STREAM_3x3:
-            std::snprintf(buf, sizeof buf, "tdc_conv3x3_stream_kernel<%d, %s, %d>", k.p[0], tf[k.p[1] != 0], k.p[2]);
+            if (k.p[3] > 1) std::snprintf(buf, sizeof buf, "tdc_conv3x3_stream_rownb_kernel<%d, %d>", k.p[0], k.p[3]);
+            else std::snprintf(buf, sizeof buf, "tdc_conv3x3_stream_kernel<%d, %s, %d>", k.p[0], tf[k.p[1] != 0], k.p[2]);
             break;
         default: return "";
     }
@@ -510,6 +527,10 @@ int kernel_vgprs(const KernelId &k) {
         if (aff) return nq == 1 ? (mode == 1 ? 72 : 40) : nq == 2 ? (mode == 1 ? 72 : 48) : nq == 4 ? 80 : 144;
         if (mode == 1) return nq == 8 ? 96 : 72;
         return nq == 1 ? 40 : nq == 2 ? 40 : nq == 4 ? 48 : 80;
+    }
+    if (k.family == KernelId::STREAM_3x3 && k.p[3] > 1) {
+        const int cg = k.p[0], nb = k.p[3];
+        return nb == 2 ? (cg == 1 ? 32 : cg == 2 ? 40 : 72) : (cg == 1 ? 40 : cg == 2 ? 64 : 104);
     }
     if (k.family == KernelId::STREAM_3x3) {
         const int cg = k.p[0], row = k.p[1], mode = k.p[2];
@@ -616,12 +637,15 @@ bool model_evaluate(const tdc_conv_desc &d, const tdc_tile &t, tdc_tile_info &in
             //  shifts where a tile is one row of 14 pixels)
             const double rate = std::min(0.59 * MC.copy_bytes_per_clk, chip_share);
             const bool row_mode = d.stride == 1 && t.tw == 14;
-            const double bytes = (double)t.cch * t.wm * (576.0 + (row_mode ? 0.28 : 0.66) * 576.0) * r;
+            // (nb pixel blocks per wave: the input rows of every block, the weights once)
+            const double bytes = (double)t.cch * t.wm * (576.0 + t.nb * (row_mode ? 0.28 : 0.66) * 576.0) * r;
             const double groups = (double)t.cch / (4.0 * t.wk);
             const double waves_simd = std::ceil((double)g.waves * r / m.simds_per_cu);
             // a wave issues its requests one after the other (about 21 cycles each): fewer groups per wave start sooner
             double clk = MC.stream_setup_clk + MC.stream_latency_clk + 288.0 + 65.0 * (waves_simd - 1.0) + bytes / rate +
-                         groups * (3.0 + (row_mode ? 3.0 : 9.0)) * 21.4;
+                         groups * (3.0 + t.nb * (row_mode ? 3.0 : 9.0)) * 21.4;
+            // the MFMAs of the extra blocks no longer hide under the requests: the matrix pipe of a SIMD serves its waves in turn
+            if (t.nb > 1) clk += waves_simd * groups * 9.0 * (t.nb - 1) * mfma_clk;
             if (t.wk > 1) clk += 1.6 * MC.sync_clk;
             if (tail_N > 0) {
                 // park the columns, a barrier, the first touch of the tail's weights, its blocks dealt over the waves
@@ -761,6 +785,16 @@ std::vector<tdc_tile> model_enumerate(const tdc_conv_desc &d, int tail_N) {
                     if (!make_geometry(d, t, g, nullptr, tail_N)) continue;
                     if (ks > 1 && (long long)g.grid_x * g.grid_y * g.grid_z > 2LL * machine().cus) continue;
                     out.push_back(t);
+                    // the same tile with 2 or 4 neighbouring 14-pixel row tiles per workgroup, sharing the weights in
+                    // registers (where the image row has that many)
+                    if (tw == 14 && d.stride == 1 && ks == 1 && tail_N == 0 && !std::getenv("TDC_EXPERIMENT_NO_STREAMED_NB"))
+                        for (int nb : {2, 4}) {
+                            if (ceil_div(Wo, 14) < nb) continue;
+                            t.nb = nb;
+                            if (make_geometry(d, t, g, nullptr, 0) &&
+                                kernel_id_for(t, 3, 3, 1, 1, false).family != KernelId::NONE)
+                                out.push_back(t);
+                        }
                 }
             }
         }

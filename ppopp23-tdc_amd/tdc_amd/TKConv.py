@@ -123,29 +123,56 @@ class TKConv2dC(nn.Module):
             self.last_kernel.copy_(last)
             if bias is not None:
                 self.bias.copy_(bias)
+        self.invalidate()
         return self
+
+    MAX_CACHED_SHAPES = 8   # native operators (packed weights + intermediates) kept per module, least recently used first out
+
+    def invalidate(self):
+        """Drop the native operators, so that the next forward re-packs the weights from the parameters.  Needed after
+        writing parameters in a way autograd's version counters do not see (``module.core_kernel.data.copy_(w)``,
+        ``.data = w``); ``load_kernels``, ``load_state_dict`` and ``.to()`` / ``.float()`` call it themselves."""
+        for op in self._ops.values():
+            op.close()
+        self._ops.clear()
+        self._stamp = None
+
+    def _load_from_state_dict(self, *args, **kwargs):
+        super()._load_from_state_dict(*args, **kwargs)
+        self.invalidate()
+
+    def _apply(self, fn, *args, **kwargs):
+        out = super()._apply(fn, *args, **kwargs)
+        self.invalidate()
+        return out
 
     def _versions(self):
         ps = [self.first_kernel, self.core_kernel, self.last_kernel] + ([self.bias] if self.bias is not None else [])
-        return tuple((p.data_ptr(), p._version) for p in ps)
+        # (storage address and version counter; writes through .data bump neither, hence the first/last elements as a
+        #  cheap additional check — a full comparison would cost more than the convolution)
+        stamp = []
+        for p in ps:
+            flat = p.detach().reshape(-1)
+            stamp.append((p.data_ptr(), p._version, float(flat[0]), float(flat[-1])))
+        return tuple(stamp)
 
     def _op_for(self, x):
         if x.dim() != 4 or x.shape[1] != self.in_channels:
             raise ValueError(f"expected input [B,{self.in_channels},H,W], got {tuple(x.shape)}")
         stamp = self._versions()
         if stamp != self._stamp:      # parameters changed: re-pack on next use
-            for op in self._ops.values():
-                op.close()
-            self._ops.clear()
+            self.invalidate()
             self._stamp = stamp
         key = (x.shape[0], x.shape[2], x.shape[3])
-        op = self._ops.get(key)
+        op = self._ops.pop(key, None)
         if op is None:
             op = TKConvOp(x.shape[0], self.in_channels, self.in_rank, self.out_rank, self.out_channels,
                           x.shape[2], x.shape[3], self.kernel_size[0], self.stride[0], self.padding[0],
                           self.dilation[0], bias=self.bias is not None)
             op.set_weights(self.first_kernel, self.core_kernel, self.last_kernel, self.bias)
-            self._ops[key] = op
+            while len(self._ops) >= self.MAX_CACHED_SHAPES:     # (dicts keep insertion order: the first key is the oldest use)
+                self._ops.pop(next(iter(self._ops))).close()
+        self._ops[key] = op      # most recently used last
         return op
 
     @torch.no_grad()

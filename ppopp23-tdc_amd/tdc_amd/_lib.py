@@ -10,7 +10,8 @@ import os
 from ctypes import POINTER, Structure, byref, c_char_p, c_double, c_int, c_int32, c_void_p
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libtdc_amd.so")
+# (TDC_AMD_LIBRARY in the environment points at another build of the same library, e.g. the profiling build with time stamps)
+LIB_PATH = os.environ.get("TDC_AMD_LIBRARY") or os.path.join(_HERE, "libtdc_amd.so")
 
 TDC_OK, TDC_ERR_INVALID, TDC_ERR_UNSUPPORTED, TDC_ERR_HIP, TDC_ERR_NOMEM, TDC_ERR_STATE = range(6)
 

@@ -180,11 +180,14 @@ def test_streamed_1x1_with_stride(shape, stride):
 
 @pytest.mark.parametrize("shape,stride,pad", [((1, 16, 16, 7, 7), 1, 1), ((2, 13, 20, 9, 11), 1, 1), ((1, 40, 24, 13, 13), 2, 1),
                                               ((1, 16, 16, 12, 12), 1, 2), ((1, 128, 48, 7, 7), 1, 1), ((1, 64, 32, 28, 28), 1, 1),
-                                              ((3, 5, 3, 4, 3), 1, 0), ((1, 250, 17, 5, 5), 2, 1)])
+                                              ((3, 5, 3, 4, 3), 1, 0), ((1, 250, 17, 5, 5), 2, 1), ((2, 20, 33, 9, 58), 1, 1),
+                                              ((1, 96, 40, 6, 30), 1, 1), ((1, 64, 48, 5, 56), 1, 0), ((1, 16, 20, 4, 44), 1, 1)])
 def test_every_streamed_3x3_tile(shape, stride, pad):
     """The 3x3 path that streams both operands from global memory into registers (tile.alg = 4): every launchable tile
-    (1, 2 or 4 channel groups per wave, 1 to 16 waves, every shape of the 16-pixel tile), stride 2, wide and no padding,
-    ragged channel counts, batches; plain, and with bias + residual + ReLU written into a channel slice."""
+    (1, 2 or 4 channel groups per wave, 1 to 16 waves, every shape of the 16-pixel tile; 2 or 4 neighbouring 14-pixel row
+    tiles per workgroup where the rows are wide enough, including rows whose last workgroup has blocks past the image),
+    stride 2, wide and no padding, ragged channel counts, batches; plain, and with bias + residual + ReLU written into a
+    channel slice."""
     from ctypes import c_void_p
     B, C, N, H, W = shape
     x, w = case(2500 + C * N + H, B, C, N, H, W, 3)
@@ -196,6 +199,8 @@ def test_every_streamed_3x3_tile(shape, stride, pad):
     want_full = (torch.from_numpy(want) + bias.view(1, -1, 1, 1) + resid).clamp_min(0).numpy()
     tiles = [t for t in tdc_amd.model_enumerate(tdc_amd.conv_desc(B, C, N, H, W, 3, 3, stride, pad)) if t.alg == 4]
     assert tiles
+    if stride == 1 and Wo > 14:
+        assert {t.nb for t in tiles} == ({1, 2, 4} if Wo > 42 else {1, 2})
     for t in tiles:
         announce("streamed 3x3", shape, stride, pad, t)
         assert_close(run_conv(x, w, stride=stride, pad=pad, tile=t), want, f"{shape} s{stride} p{pad} {t}")

@@ -67,11 +67,21 @@ def test_streamed_tiles_only_where_they_apply():
                  (d3, tdc_amd.Tile(16, 1, 1, 1, 1, 4, 32, 14, 1, 0, 4)),       # not all channels in one pass
                  (d3, tdc_amd.Tile(16, 1, 1, 1, 1, 4, 64, 14, 1, 2, 4)),       # loader waves
                  (d3, tdc_amd.Tile(16, 1, 1, 8, 1, 4, 64, 14, 1, 0, 4)),       # 32 waves
-                 (d3, tdc_amd.Tile(16, 1, 2, 1, 1, 4, 64, 14, 1, 0, 4)),       # one pixel block per wave
+                 (d3, tdc_amd.Tile(16, 1, 2, 1, 1, 4, 64, 14, 1, 0, 4)),       # two pixel blocks per wave, one 14-pixel tile per row
+                 (conv3(64, 64, 56), tdc_amd.Tile(16, 1, 2, 1, 1, 4, 64, 16, 1, 0, 4)),   # several blocks need rows of 14 pixels
+                 (conv3(64, 64, 56), tdc_amd.Tile(16, 1, 2, 1, 1, 4, 32, 14, 2, 0, 4)),   # ... and no split across workgroups
+                 (conv3(64, 64, 56, stride=2), tdc_amd.Tile(16, 1, 2, 1, 1, 4, 64, 14, 1, 0, 4)),   # ... and stride 1
                  (tdc_amd.conv_desc(1, 64, 64, 14, 14, 3, 3, 1, 2, 2), tdc_amd.Tile(16, 1, 1, 1, 1, 4, 64, 14, 1, 0, 4)),  # dilation 2
                  (d1, tdc_amd.Tile(16, 1, 1, 1, 1, 4, 256, 16, 1, 0, 4))]:
         with pytest.raises(tdc_amd.TdcError):
             tdc_amd.model_evaluate(d, t)
+    # nb = 2 or 4 neighbouring 14-pixel row tiles per workgroup (the weights a wave holds feed nb MFMAs each)
+    nb4 = tdc_amd.model_evaluate(conv3(64, 64, 56), tdc_amd.Tile(16, 1, 4, 1, 1, 8, 64, 14, 1, 0, 4))
+    assert (nb4.grid_x, nb4.grid_y, nb4.th, nb4.block_threads, nb4.lds_bytes) == (56, 4, 1, 512, 8 * 4 * 1024)
+    nb2 = tdc_amd.model_evaluate(conv3(64, 64, 28), tdc_amd.Tile(16, 1, 2, 1, 1, 16, 64, 14, 1, 0, 4))
+    assert (nb2.grid_x, nb2.grid_y, nb2.block_threads) == (28, 4, 1024)
+    assert any(t.alg == 4 and t.nb == 4 for t in tdc_amd.model_enumerate(conv3(64, 64, 56)))
+    assert not any(t.alg == 4 and t.nb > 1 for t in tdc_amd.model_enumerate(conv3(64, 64, 14)))
     # the enumeration offers them for every 1x1 / 3x3 shape they fit, and only there
     assert any(t.alg == 3 for t in tdc_amd.model_enumerate(d1)) and not any(t.alg == 4 for t in tdc_amd.model_enumerate(d1))
     assert any(t.alg == 4 for t in tdc_amd.model_enumerate(d3)) and not any(t.alg == 3 for t in tdc_amd.model_enumerate(d3))

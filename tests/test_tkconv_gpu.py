@@ -112,6 +112,20 @@ def test_module_forward_matches_reference_forward():
     want2 = ref.tkconv_torch(x2, m.first_kernel.detach(), m.core_kernel.detach(), m.last_kernel.detach(), m.bias.detach(),
                              1, 1, 1)
     assert_close(m(x2.cuda()).cpu().numpy(), want2.numpy(), "module after update")
+    # writes through .data do not bump the version counter: invalidate() (or load_state_dict / load_kernels) re-packs
+    m.last_kernel.data[1:-1].mul_(-2.0)          # (first and last element untouched: the cheap stamp cannot see it)
+    m.invalidate()
+    want3 = ref.tkconv_torch(x2, m.first_kernel.detach(), m.core_kernel.detach(), m.last_kernel.detach(), m.bias.detach(),
+                             1, 1, 1)
+    assert_close(m(x2.cuda()).cpu().numpy(), want3.numpy(), "module after invalidate()")
+    sd = {k: v.clone() * 0.5 for k, v in m.state_dict().items()}
+    m.load_state_dict(sd)
+    want4 = ref.tkconv_torch(x2, sd["first_kernel"], sd["core_kernel"], sd["last_kernel"], sd["bias"], 1, 1, 1)
+    assert_close(m(x2.cuda()).cpu().numpy(), want4.numpy(), "module after load_state_dict")
+    # the per-shape operator cache is bounded
+    for hw in range(5, 5 + m.MAX_CACHED_SHAPES + 3):
+        m(torch.randn(1, 40, hw, hw).cuda())
+    assert len(m._ops) == m.MAX_CACHED_SHAPES
 
 
 def test_module_stride2_no_bias_and_load_kernels():
