@@ -134,6 +134,31 @@ __device__ __forceinline__ int fdiv(int n, const FastDiv &f) {
     return (int)(__umulhi((unsigned)n, f.m) + ((unsigned)n & f.pass));
 }
 
+// Epilogue of a lane that holds four consecutive output channels (from ch0) of one pixel: + bias, + residual, ReLU,
+// store.  All eight loads are requested before the first value is needed — one memory round trip for the lane
+// instead of one per load (written naively, every load sits behind the previous channel's store, which it might alias).
+__device__ __forceinline__ void finish_four_channels(const f4_t &acc, int ch0, int N, long long P, long long pix,
+                                                     const float *__restrict__ bias, const float *__restrict__ resid,
+                                                     int relu, float *__restrict__ out) {
+    float bv[4] = {0.0f, 0.0f, 0.0f, 0.0f}, rv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (bias) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) bv[i] = bias[min(ch0 + i, N - 1)];
+    }
+    if (resid) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) rv[i] = resid[(long long)min(ch0 + i, N - 1) * P + pix];
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        if (ch0 + i >= N) continue;
+        float val = acc[i] + bv[i];
+        val += rv[i];
+        if (relu) val = fmaxf(val, 0.0f);
+        out[(long long)(ch0 + i) * P + pix] = val;
+    }
+}
+
 // The kernel arguments (about 400 bytes) are read through the scalar cache.  Left alone, the compiler fetches them in
 // several dependent batches, and every batch that touches a cache line for the first time costs a round trip to L2
 // before the first request can go out.  Touch every line of the argument block at once: whatever order the compiler
@@ -853,7 +878,12 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
         }
         __syncthreads();
     }
-    auto each_output = [&](auto &&sink, bool want_value) {
+    // With `want_addends` the bias and the residual value of every output are requested before its value is
+    // assembled (all of a pixel block's at once, or ahead of the partial sums' LDS reads) and handed to the sink,
+    // so that the lane pays one memory round trip and not one per load.
+    auto each_output = [&](auto &&sink, bool want_value, bool want_addends) {
+        const bool load_bias = want_addends && p.bias != nullptr;
+        const bool load_resid = want_addends && resid != nullptr;
         if (p.WK == 1 && !WINO) {
             // Straight from the accumulators: each store instruction writes runs of
             // consecutive pixels of one output channel.
@@ -864,13 +894,23 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
                 const int jx = j - jy * p.TW;
                 const int oy = oy0 + jy, ox = ox0 + jx;
                 const bool pix_ok = jy < p.TH && oy < p.Ho && ox < p.Wo && !loader;
-                const int pp = oy * p.Wo + ox;
+                const int pp = pix_ok ? oy * p.Wo + ox : 0;
 #pragma unroll
                 for (int mb = 0; mb < MB; ++mb) {
 #pragma unroll
-                    for (int v = 0; v < NACC; ++v) {
-                        const int n = m0 + (wm * MB + mb) * MF + M::row(v, lane);
-                        if (n < p.N && pix_ok) sink(n, pp, acc[mb][nb][v]);
+                    for (int v0 = 0; v0 < NACC; v0 += 4) {
+                        float bv[4], rv[4];
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) {
+                            const int n = min(m0 + (wm * MB + mb) * MF + M::row(v0 + u, lane), p.N - 1);
+                            bv[u] = load_bias ? p.bias[n] : 0.0f;
+                            rv[u] = load_resid ? resid[(long long)n * p.P + pp] : 0.0f;
+                        }
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) {
+                            const int n = m0 + (wm * MB + mb) * MF + M::row(v0 + u, lane);
+                            if (n < p.N && pix_ok) sink(n, pp, acc[mb][nb][v0 + u], bv[u], rv[u]);
+                        }
                     }
                 }
             }
@@ -884,6 +924,8 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
                 const int n = m0 + ml;
                 const int oy = oy0 + jy, ox = ox0 + jx;
                 if (n < p.N && jy < p.TH && oy < p.Ho && ox < p.Wo) {
+                    const float bv = load_bias ? p.bias[n] : 0.0f;
+                    const float rv = load_resid ? resid[(long long)n * p.P + oy * p.Wo + ox] : 0.0f;
                     float val = 0.0f;
                     if (want_value) {
                         // four reads in flight at a time; the additions stay in slice order
@@ -896,17 +938,16 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
                                 if (k0 + u < p.WK) val += part[u];
                         }
                     }
-                    sink(n, oy * p.Wo + ox, val);
+                    sink(n, oy * p.Wo + ox, val, bv, rv);
                 }
             }
         }
     };
-    auto finish = [&](int n, int pp, float val) {
-        if (p.bias) val += p.bias[n];
-        const long long o = (long long)n * p.P + pp;
-        if (resid) val += resid[o];
+    auto finish = [&](int n, int pp, float val, float bv, float rv) {
+        val += bv;
+        val += rv;
         if (p.relu) val = fmaxf(val, 0.0f);
-        out[o] = val;
+        out[(long long)n * p.P + pp] = val;
     };
     if constexpr (EXT) if (p.tail_w) {
         // Fused tail: a 1x1 convolution over the output channels of this one, out2 = W2 * act(conv + bias), in the
@@ -940,6 +981,7 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
             for (int idx = tid; idx < total; idx += nthreads) {
                 const int ml = fdiv(idx, p.fd_pt);
                 const int pl = idx - ml * PT;
+                const float b1 = (p.bias && ml < p.N) ? p.bias[ml] : 0.0f;
                 float val = 0.0f;
                 for (int k0 = 0; k0 < p.WK; k0 += 4) {
                     float part[4];
@@ -949,7 +991,7 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
                     for (int u = 0; u < 4; ++u)
                         if (k0 + u < p.WK) val += part[u];
                 }
-                if (p.bias && ml < p.N) val += p.bias[ml];
+                val += b1;
                 if (p.relu) val = fmaxf(val, 0.0f);
                 f[ml * LD + pl] = val;
             }
@@ -963,6 +1005,23 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
             const int pxblk = blk - mblk * npx;
             const float *wa = p.tail_w + (size_t)mblk * p.tail_ng * 64 + lane;
             const float *fb = f + ksub16 * LD + pxblk * 16 + px16;
+            const int j = pxblk * 16 + px16;
+            const int jy = fdiv(j, p.fd_tw);
+            const int jx = j - jy * p.TW;
+            const int oy = oy0 + jy, ox = ox0 + jx;
+            const bool pix_ok = jy < p.TH && oy < p.Ho && ox < p.Wo;
+            const int pp = pix_ok ? oy * p.Wo + ox : 0;
+            // (bias and residual of this block are requested before the small GEMM and arrive under it)
+            const int n20 = mblk * 16 + 4 * ksub16;
+            float tbv[4] = {0.0f, 0.0f, 0.0f, 0.0f}, trv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+            if (p.tail_bias) {
+#pragma unroll
+                for (int v = 0; v < 4; ++v) tbv[v] = p.tail_bias[min(n20 + v, p.tail_N - 1)];
+            }
+            if (resid) {
+#pragma unroll
+                for (int v = 0; v < 4; ++v) trv[v] = resid[(long long)min(n20 + v, p.tail_N - 1) * p.P + pp];
+            }
             f4_t acc2 = {0.0f, 0.0f, 0.0f, 0.0f};
             for (int g0 = 0; g0 < p.tail_ng; g0 += 4) {
                 float a[4], b[4];
@@ -976,22 +1035,15 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
                 for (int u = 0; u < 4; ++u)
                     if (g0 + u < p.tail_ng) acc2 = __builtin_amdgcn_mfma_f32_16x16x4f32(a[u], b[u], acc2, 0, 0, 0);
             }
-            const int j = pxblk * 16 + px16;
-            const int jy = fdiv(j, p.fd_tw);
-            const int jx = j - jy * p.TW;
-            const int oy = oy0 + jy, ox = ox0 + jx;
-            if (jy < p.TH && oy < p.Ho && ox < p.Wo) {
-                const int pp = oy * p.Wo + ox;
+            if (pix_ok) {
 #pragma unroll
                 for (int v = 0; v < 4; ++v) {
-                    const int n2 = mblk * 16 + 4 * ksub16 + v;
+                    const int n2 = n20 + v;
                     if (n2 < p.tail_N) {
-                        float val = acc2[v];
-                        if (p.tail_bias) val += p.tail_bias[n2];
-                        const long long o = (long long)n2 * p.P + pp;
-                        if (resid) val += resid[o];
+                        float val = acc2[v] + tbv[v];
+                        val += trv[v];
                         if (p.tail_relu) val = fmaxf(val, 0.0f);
-                        out[o] = val;
+                        out[(long long)n2 * p.P + pp] = val;
                     }
                 }
             }
@@ -1019,11 +1071,15 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
                     const int n = m0 + ml;
                     const int oy = oy0 + jy, ox = ox0 + jx;
                     if (n < p.N && jy < p.TH && oy < p.Ho && ox < p.Wo) {
+                        // (bias and residual are requested first and arrive under the LDS reads)
+                        const long long o = (long long)n * p.P + oy * p.Wo + ox;
+                        const float bv = p.bias ? p.bias[n] : 0.0f;
+                        vec_t rv = vec_tag;
+                        if (resid) rv = *reinterpret_cast<const vec_t *>(resid + o);
                         vec_t val = *reinterpret_cast<const vec_t *>(lds + idx);
                         for (int k = 1; k < p.WK; ++k) val += *reinterpret_cast<const vec_t *>(lds + k * (MT * PT) + idx);
-                        const long long o = (long long)n * p.P + oy * p.Wo + ox;
-                        if (p.bias) val += p.bias[n];
-                        if (resid) val += *reinterpret_cast<const vec_t *>(resid + o);
+                        val += bv;
+                        val += rv;
                         if (p.relu) {
 #pragma unroll
                             for (int e = 0; e < V; ++e) val[e] = fmaxf(val[e], 0.0f);
@@ -1046,7 +1102,7 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
                 return;
             }
         }
-        each_output(finish, true);
+        each_output(finish, true, true);
         TDC_STAMP(6);
         TDC_STAMP_FLUSH(p, logical, wave, lane);
         return;
@@ -1061,10 +1117,10 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
     const long long NP = (long long)p.N * p.P;
     float *wsz = p.ws + (long long)bz * NP;
     each_output(
-        [&](int n, int pp, float val) {
+        [&](int n, int pp, float val, float, float) {
             __hip_atomic_store(wsz + (long long)n * p.P + pp, val, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         },
-        true);
+        true, false);
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
     unsigned *ticket = p.ctr + ((unsigned)img * p.grid_y + by) * p.grid_x + bx;
@@ -1078,7 +1134,7 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
     if (tid == 0) __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
     const float *ws0 = p.ws + (long long)img * p.KS * NP;
     each_output(
-        [&](int n, int pp, float) {
+        [&](int n, int pp, float, float bv, float rv) {
             const long long o = (long long)n * p.P + pp;
             // Four loads in flight at a time; the additions stay in slice order.
             float val = 0.0f;
@@ -1093,9 +1149,9 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
                 for (int u = 0; u < 4; ++u)
                     if (k0 + u < p.KS) val += part[u];
             }
-            finish(n, pp, val);
+            finish(n, pp, val, bv, rv);
         },
-        false);
+        false, true);
 }
 
 // ---------------------------------------------------------------------------
@@ -1266,17 +1322,7 @@ __global__ void __launch_bounds__(NQ == 8 ? 512 : 1024) tdc_conv1x1_stream_kerne
         if (!stream_join_slices(p, lds, acc, wave == 0 && px < p.P, by * 16 + 4 * k, px, img, slice, by, bx)) return;
     }
     if (wave != 0 || px >= p.P) return;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int ch = by * 16 + 4 * k + i;
-        if (ch >= p.N) continue;
-        float val = acc[i];
-        if (p.bias) val += p.bias[ch];
-        const long long o = (long long)ch * p.P + px;
-        if (resid) val += resid[o];
-        if (p.relu) val = fmaxf(val, 0.0f);
-        out[o] = val;
-    }
+    finish_four_channels(acc, by * 16 + 4 * k, p.N, p.P, px, p.bias, resid, p.relu, out);
 }
 
 // ---------------------------------------------------------------------------
@@ -1508,6 +1554,18 @@ __global__ void __launch_bounds__(1024) tdc_conv3x3_stream_kernel(const ConvKPar
         for (int blk = wave; blk < p.tail_mblk; blk += nwaves) {
             const float *wa = p.tail_w + (size_t)blk * p.tail_ng * 64 + lane;
             const float *fb = f + k * LD + n;
+            // (bias and residual of this block are requested before the small GEMM and arrive under it)
+            const int n20 = blk * 16 + 4 * k;
+            const long long ppc = live ? pp : 0;
+            float tbv[4] = {0.0f, 0.0f, 0.0f, 0.0f}, trv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+            if (p.tail_bias) {
+#pragma unroll
+                for (int v = 0; v < 4; ++v) tbv[v] = p.tail_bias[min(n20 + v, p.tail_N - 1)];
+            }
+            if (resid) {
+#pragma unroll
+                for (int v = 0; v < 4; ++v) trv[v] = resid[(long long)min(n20 + v, p.tail_N - 1) * p.P + ppc];
+            }
             f4_t acc2 = {0.0f, 0.0f, 0.0f, 0.0f};
             for (int g0 = 0; g0 < p.tail_ng; g0 += 4) {
                 float ta[4], tb[4];
@@ -1524,14 +1582,12 @@ __global__ void __launch_bounds__(1024) tdc_conv3x3_stream_kernel(const ConvKPar
             if (live) {
 #pragma unroll
                 for (int v = 0; v < 4; ++v) {
-                    const int n2 = blk * 16 + 4 * k + v;
+                    const int n2 = n20 + v;
                     if (n2 < p.tail_N) {
-                        float val = acc2[v];
-                        if (p.tail_bias) val += p.tail_bias[n2];
-                        const long long o = (long long)n2 * p.P + pp;
-                        if (resid) val += resid[o];
+                        float val = acc2[v] + tbv[v];
+                        val += trv[v];
                         if (p.tail_relu) val = fmaxf(val, 0.0f);
-                        out[o] = val;
+                        out[(long long)n2 * p.P + pp] = val;
                     }
                 }
             }
@@ -1542,17 +1598,7 @@ __global__ void __launch_bounds__(1024) tdc_conv3x3_stream_kernel(const ConvKPar
         if (!stream_join_slices(p, lds, acc, wki == 0 && live, mblk * 16 + 4 * k, pp, img, slice, by, bx)) return;
     }
     if (wki != 0 || !live) return;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int ch = mblk * 16 + 4 * k + i;
-        if (ch >= p.N) continue;
-        float val = acc[i];
-        if (p.bias) val += p.bias[ch];
-        const long long o = (long long)ch * p.P + pp;
-        if (resid) val += resid[o];
-        if (p.relu) val = fmaxf(val, 0.0f);
-        out[o] = val;
-    }
+    finish_four_channels(acc, mblk * 16 + 4 * k, p.N, p.P, pp, p.bias, resid, p.relu, out);
 }
 
 // ---------------------------------------------------------------------------
@@ -1678,6 +1724,14 @@ __global__ void __launch_bounds__(1024) tdc_conv3x3_stream_rownb_kernel(const Co
         const int cb = rest / NB, blk = rest - cb * NB;
         const float *src = lds + (((cb * p.WK) * NB + blk) * 4 + i) * 64 + l;
         const int wstride = NB * 256;
+        const int ch = (by * p.WM + cb) * 16 + 4 * (l >> 4) + i;
+        const int px = l & 15;
+        const int ox = (tile_x * NB + blk) * 14 + px;
+        const bool ok = ch < p.N && px < 14 && ox < p.Wo;
+        const long long o = ok ? (long long)ch * p.P + tile_y * p.Wo + ox : 0;
+        // (bias and residual are requested before the partial sums are read and arrive under those reads)
+        const float bv = p.bias ? p.bias[min(ch, p.N - 1)] : 0.0f;
+        const float rv = resid ? resid[o] : 0.0f;
         float val = 0.0f;
         // four reads in flight at a time; the additions stay in wave order
         for (int w0 = 0; w0 < p.WK; w0 += 4) {
@@ -1688,13 +1742,9 @@ __global__ void __launch_bounds__(1024) tdc_conv3x3_stream_rownb_kernel(const Co
             for (int u = 0; u < 4; ++u)
                 if (w0 + u < p.WK) val += part[u];
         }
-        const int ch = (by * p.WM + cb) * 16 + 4 * (l >> 4) + i;
-        const int px = l & 15;
-        const int ox = (tile_x * NB + blk) * 14 + px;
-        if (ch < p.N && px < 14 && ox < p.Wo) {
-            if (p.bias) val += p.bias[ch];
-            const long long o = (long long)ch * p.P + tile_y * p.Wo + ox;
-            if (resid) val += resid[o];
+        if (ok) {
+            val += bv;
+            val += rv;
             if (p.relu) val = fmaxf(val, 0.0f);
             out[o] = val;
         }

@@ -423,16 +423,35 @@ double *mc_field(int i) {
 
 }  // namespace
 
-// Waves of this kernel that fit one SIMD: 512 vector registers per lane shared by its waves, at most 8 waves, and
-// 800 scalar registers handed out in blocks of 16 — the staged kernel needs 106 (112 allocated), which leaves room
-// for 7 waves, not 8, so a 1024-thread workgroup of it is alone on its compute unit however few vector registers it
-// uses (the HIP runtime's occupancy query says the same).  The streamed kernels stay under 96 scalar registers.
+struct CompiledKernel { const char *name; int regs, sgprs, waves; };
+// hipcc's resource report for the convolution kernels of this build (written by the Makefile from the compile of
+// conv_mfma.hip): name, VGPRs + AGPRs per lane, scalar registers, waves per SIMD.
+static const CompiledKernel compiled_kernels[] = {
+#include "kernel_registers.inc"
+};
+
+static const CompiledKernel *compiled_kernel(const KernelId &k) {
+    static const std::map<std::string, const CompiledKernel *> by_name = [] {
+        std::map<std::string, const CompiledKernel *> m;
+        for (const CompiledKernel &c : compiled_kernels) m[c.name] = &c;
+        return m;
+    }();
+    const auto it = by_name.find(kernel_name(k));
+    return it == by_name.end() ? nullptr : it->second;
+}
+
+// Waves of this kernel that fit one SIMD, as the compiler works it out from the registers of the compiled kernel:
+// 512 vector registers per lane shared by a SIMD's waves (handed out in blocks of 8), at most 8 waves, and 800 scalar
+// registers in blocks of 16 — the staged kernel needs 106 (112 allocated), which leaves room for 7 waves, not 8, so
+// a 1024-thread workgroup of it is alone on its compute unit however few vector registers it uses (the HIP runtime's
+// occupancy query says the same).
 int kernel_waves_per_simd(const KernelId &k) {
-    const int regs = kernel_vgprs(k);
-    if (regs <= 0) return 0;
+    const CompiledKernel *c = compiled_kernel(k);
+    if (!c) return 0;
     const Machine &m = machine();
-    const int by_sgpr = k.family == KernelId::STAGED ? 800 / 112 : 800 / 96;
-    return std::min(std::min(m.max_waves_per_simd, m.vgprs_per_simd_lane / regs), by_sgpr);
+    const int by_vgpr = m.vgprs_per_simd_lane / ((c->regs + 7) / 8 * 8);
+    const int by_sgpr = 800 / ((c->sgprs + 15) / 16 * 16);
+    return std::min(std::min(m.max_waves_per_simd, by_vgpr), std::min(by_sgpr, c->waves));
 }
 
 KernelId kernel_id_with_head(const tdc_tile &t) {
@@ -517,44 +536,13 @@ std::string kernel_name(const KernelId &k) {
     return buf;
 }
 
-// Registers per lane of the compiled instantiations (hipcc's kernel-resource-usage report: VGPRs + AGPRs), rounded
-// up to the allocation granule of 8.  The reference measures occupancy per candidate by compiling and probing each
-// (2080Ti-evaluation/Gen-occupancy/template.cu:277-284); here the candidates share a few dozen instantiations, so
-// the table is short, and a test compares it with the report of the build at hand.
+// Registers per lane of the compiled instantiation (hipcc's kernel-resource-usage report: VGPRs + AGPRs), rounded up
+// to the allocation granule of 8; 0 for a kernel the library does not hold.  The reference measures occupancy per
+// candidate by compiling and probing each (2080Ti-evaluation/Gen-occupancy/template.cu:277-284); here the candidates
+// share about a hundred instantiations, whose report the build compiles into this file.
 int kernel_vgprs(const KernelId &k) {
-    if (k.family == KernelId::STREAM_1x1) {
-        const int nq = k.p[0], aff = k.p[1], mode = k.p[2];
-        if (aff) return nq == 1 ? (mode == 1 ? 72 : 40) : nq == 2 ? (mode == 1 ? 72 : 48) : nq == 4 ? 80 : 144;
-        if (mode == 1) return nq == 8 ? 96 : 72;
-        return nq == 1 ? 40 : nq == 2 ? 40 : nq == 4 ? 48 : 80;
-    }
-    if (k.family == KernelId::STREAM_3x3 && k.p[3] > 1) {
-        const int cg = k.p[0], nb = k.p[3];
-        return nb == 2 ? (cg == 1 ? 32 : cg == 2 ? 40 : 72) : (cg == 1 ? 40 : cg == 2 ? 64 : 104);
-    }
-    if (k.family == KernelId::STREAM_3x3) {
-        const int cg = k.p[0], row = k.p[1], mode = k.p[2];
-        if (cg == 4) return 88;
-        if (mode == 1) return 64;
-        if (mode == 3) return cg == 1 ? 56 : 64;
-        if (cg == 1) return row && mode == 0 ? 40 : 48;
-        return row ? 48 : 56;
-    }
-    if (k.family != KernelId::STAGED) return 0;
-    const int mf = k.p[0], mb = k.p[1], nb = k.p[2], taps = k.p[3], ext = k.p[5];
-    if (taps == TAPS_WINO) return 128;
-    if (taps == TAPS_3x3G) return mf == 16 ? 104 : 120;
-    const int blk = (mb - 1) * 2 + (nb - 1);   // 1x1, 1x2, 2x1, 2x2 blocks per wave
-    // [mf 16/32][taps generic/1x1/3x3][blocks][plain/extras]
-    static const int tab[2][3][4][2] = {
-        {{{32, 32}, {48, 48}, {40, 40}, {64, 64}},
-         {{48, 72}, {56, 80}, {64, 80}, {80, 88}},
-         {{64, 64}, {88, 88}, {96, 96}, {120, 120}}},
-        {{{48, 48}, {80, 80}, {64, 64}, {128, 128}},
-         {{56, 80}, {88, 104}, {88, 104}, {128, 144}},
-         {{80, 80}, {112, 112}, {112, 112}, {168, 168}}}};
-    const int ti = taps == TAPS_GENERIC ? 0 : taps == TAPS_1x1 ? 1 : 2;
-    return tab[mf == 32][ti][blk][ext != 0];
+    const CompiledKernel *c = compiled_kernel(k);
+    return c ? (c->regs + 7) / 8 * 8 : 0;
 }
 
 bool model_evaluate(const tdc_conv_desc &d, const tdc_tile &t, tdc_tile_info &info, std::string *why, int tail_N) {
