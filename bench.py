@@ -92,6 +92,8 @@ def main():
                     help="profiling aid: launch every layer of the sweep (and of the reference's 18 shapes) `steps` times, "
                          "each launch followed by a stream synchronisation, and exit; under rocprofv3 --kernel-trace the "
                          "kernel durations are then those of isolated launches, not launch-to-launch times")
+    ap.add_argument("--tiles-from", default=None, metavar="FILE",
+                    help="profiling aid: force the tiles recorded in this file, the output of a plain run of this benchmark")
     ap.add_argument("--tile", default=None, metavar="mf,mb,nb,wm,wn,wk,cch,tw,ks,wl,alg",
                     help="with --only-dominant / --only-conv: force this tile instead of selecting one")
     ap.add_argument("--tune", type=int, default=16, metavar="CLASSES",
@@ -163,9 +165,17 @@ def main():
                           "roof_us": round(info.roof_us, 4), "timing": "hipEvents around the launches of this run"}))
         return
 
+    # --tiles-from: the tiles a plain run of this benchmark timed (its JSON line), so that a profiled run launches
+    # the same kernels (measured selection under a profiler times the candidates with the profiler's overhead).
+    forced_tiles = {}
+    if a.tiles_from:
+        prev = json.loads(open(a.tiles_from).read().strip().splitlines()[-1])
+        for row in prev["layers"] + prev["reference_layer_shapes"]["layers"]:
+            forced_tiles[(row["R1"], row["R2"], row["H"])] = tdc_amd.Tile(*row["tile"])
+
     def make_layer(hw, r1, r2):
         x, w = ref.make_core_case(hw, r1, r2)
-        plan = Conv2dPlan(1, r1, r2, hw, hw, 3, 3, 1, 1).set_weights(w)
+        plan = Conv2dPlan(1, r1, r2, hw, hw, 3, 3, 1, 1, tile=forced_tiles.get((r1, r2, hw))).set_weights(w)
         return {"hw": hw, "r1": r1, "r2": r2, "plan": plan, "x": x.cuda(), "out": torch.empty(1, r2, hw, hw, device="cuda"),
                 "xc": x, "wc": w}
 
