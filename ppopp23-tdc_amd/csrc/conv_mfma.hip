@@ -808,6 +808,41 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
 #pragma unroll
                     for (int nb = 0; nb < NB; ++nb) acc[mb][nb] = M::run(a[mb], b[nb], acc[mb][nb]);
             }
+        } else if constexpr (TAPS == TAPS_7x7) {
+            // 7x7, dilation 1 (the stems of the networks): the 49 K-steps of a channel group fully unrolled, the
+            // operands of filter row r+1 read while the MFMAs of row r run (two register sets of seven K-steps).
+            for (int g = 0; g < ncgw; ++g) {
+                const float *lgrp = sin + g * KC * p.CS;
+                float a[2][7][MB], b[2][7][NB];
+                auto load_row = [&](int r, float(&ar)[7][MB], float(&br)[7][NB]) {
+#pragma unroll
+                    for (int s7 = 0; s7 < 7; ++s7) {
+#pragma unroll
+                        for (int mb = 0; mb < MB; ++mb) ar[s7][mb] = sw[mb][(g * 49 + r * 7 + s7) * 64];
+#pragma unroll
+                        for (int nb = 0; nb < NB; ++nb) br[s7][nb] = lgrp[boff[nb] + r * p.RS + s7];
+                    }
+                };
+                load_row(0, a[0], b[0]);
+#pragma unroll
+                for (int r = 0; r < 7; ++r) {
+                    if (r + 1 < 7) load_row(r + 1, a[(r + 1) & 1], b[(r + 1) & 1]);
+#pragma unroll
+                    for (int s7 = 0; s7 < 7; ++s7)
+#pragma unroll
+                        for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                            for (int nb = 0; nb < NB; ++nb)
+                                acc[mb][nb] = M::run(a[r & 1][s7][mb], b[r & 1][s7][nb], acc[mb][nb]);
+                    if (r + 1 < 7) {
+#pragma unroll
+                        for (int s7 = 0; s7 < 7; ++s7) {
+                            __builtin_amdgcn_sched_group_barrier(0x008, MB * NB, 0);  // MFMA
+                            __builtin_amdgcn_sched_group_barrier(0x100, MB + NB, 0);  // LDS reads of the next row
+                        }
+                    }
+                }
+            }
         } else {
             // Any filter size / dilation: taps walked at run time.
             for (int g = 0; g < ncgw; ++g) {
@@ -1812,6 +1847,7 @@ const void *kernel_function(const KernelId &k) {
                 break;
             case TAPS_3x3: fn = ext ? pick_mf<TAPS_3x3, true>(k.p[0], k.p[1], k.p[2]) : pick_mf<TAPS_3x3, false>(k.p[0], k.p[1], k.p[2]); break;
             case TAPS_1x1: fn = ext ? pick_mf<TAPS_1x1, true>(k.p[0], k.p[1], k.p[2]) : pick_mf<TAPS_1x1, false>(k.p[0], k.p[1], k.p[2]); break;
+            case TAPS_7x7: fn = ext ? nullptr : pick_mf<TAPS_7x7, false>(k.p[0], k.p[1], k.p[2]); break;
             case TAPS_GENERIC: fn = ext ? pick_mf<TAPS_GENERIC, true>(k.p[0], k.p[1], k.p[2]) : pick_mf<TAPS_GENERIC, false>(k.p[0], k.p[1], k.p[2]); break;
             default: break;
         }

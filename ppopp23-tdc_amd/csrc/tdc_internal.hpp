@@ -152,7 +152,7 @@ struct ConvKParams {
 };
 
 // Inner loop of the staged kernel (its TAPS template argument).
-enum : int { TAPS_GENERIC = 0, TAPS_1x1 = 1, TAPS_3x3 = 9, TAPS_3x3G = 10, TAPS_WINO = 16 };
+enum : int { TAPS_GENERIC = 0, TAPS_1x1 = 1, TAPS_3x3 = 9, TAPS_3x3G = 10, TAPS_WINO = 16, TAPS_7x7 = 49 };
 
 // Which kernel instantiation serves a tile: worked out on the host (no device needed), so that the tile model, the
 // launcher and the occupancy probe all speak of the same function.

@@ -506,7 +506,9 @@ KernelId kernel_id_for(const tdc_tile &t, int KH, int KW, int dilation, int stri
         if (extras || KH != 3 || KW != 3 || dilation != 1 || t.mb != 1 || t.nb != 1) return k;
         taps = TAPS_3x3G;
     } else if (t.alg == 0) {
-        taps = (KH == 3 && KW == 3 && dilation == 1) ? TAPS_3x3 : (KH == 1 && KW == 1) ? TAPS_1x1 : TAPS_GENERIC;
+        taps = (KH == 3 && KW == 3 && dilation == 1) ? TAPS_3x3 : (KH == 1 && KW == 1) ? TAPS_1x1
+             : (KH == 7 && KW == 7 && dilation == 1 && !extras) ? TAPS_7x7   // (the network stems; built without the extras)
+                                                                : TAPS_GENERIC;
     } else {
         return k;
     }

@@ -294,6 +294,33 @@ def test_general_filters(K, stride, pad, dil):
         assert_close(run_conv(x, w, stride=stride, pad=pad, dil=dil, tile=t), want, f"K{K} s{stride} p{pad} d{dil} {t}")
 
 
+@pytest.mark.parametrize("C,stride", [(3, 2), (9, 1)])
+def test_seven_by_seven_instantiations(C, stride):
+    """The unrolled 7x7 loop (the network stems) in all its register-block variants: 16- and 32-row MFMAs, one or two
+    channel and pixel blocks per wave, one and three channel groups, stride 1 and 2; and the same filter with a
+    dilation, which falls back to the run-time tap walker."""
+    N, H, W = 64, 30, 27
+    x, w = case(3100 + C, 1, C, N, H, W, 7)
+    want = ref.conv2d_c(x.numpy(), w.numpy(), stride=stride, pad=3)
+    d = tdc_amd.conv_desc(1, C, N, H, W, 7, 7, stride, 3, 1)
+    seen = set()
+    for t in tdc_amd.model_enumerate(d):
+        key = (t.mf, t.mb, t.nb)
+        if t.alg != 0 or key in seen:
+            continue
+        seen.add(key)
+        name, _, _ = tdc_amd._lib.model_kernel_info(d, t)
+        assert ", 49, " in name, name
+        announce("7x7", C, stride, t)
+        assert_close(run_conv(x, w, stride=stride, pad=3, tile=t), want, f"7x7 C{C} s{stride} {t}")
+    assert len(seen) >= 6, seen
+    dd = tdc_amd.conv_desc(1, C, N, H, W, 7, 7, stride, 6, 2)
+    t = tdc_amd.model_select(dd).tile
+    assert ", 0, " in tdc_amd._lib.model_kernel_info(dd, t)[0]
+    want = ref.conv2d_c(x.numpy(), w.numpy(), stride=stride, pad=6, dil=2)
+    assert_close(run_conv(x, w, stride=stride, pad=6, dil=2, tile=t), want, f"7x7 dilated C{C} s{stride}")
+
+
 def test_random_shapes_model_tile():
     """Forty seeded random problems (ragged sizes, batch, stride, padding, dilation, rectangular images, every
     epilogue combination) with the tile the model picks, against F.conv2d on the host."""
