@@ -339,8 +339,10 @@ int tdc_model_kernel_info(const tdc_conv_desc *desc, const tdc_tile *tile, int32
                           int32_t *vgprs_out, int32_t *waves_per_simd_out);
 /* Calibration constants of the latency model (launch floor, copy latency and rate, barrier cost, ...;
  * the counterpart of num_sm / num_threads / a,b,c / ratio in the reference's model.py:265-266,278).
- * get: writes up to `cap` values, *count_out = how many there are.  set: all of them, all > 0;
- * process-wide, not thread-safe against concurrent model calls. */
+ * get: writes up to `cap` values, *count_out = how many there are.  set: all of them, all > 0; process-wide.
+ * The constants only steer the CHOICE of a tile: they are read while a plan is created (or a tdc_model_* call
+ * runs) and never afterwards, so existing plans keep their tile, their kernels and their results whatever is set
+ * later.  set may be called while other threads create plans: evaluations in flight finish with the old values. */
 int tdc_model_get_constants(double *values_out, int32_t cap, int32_t *count_out);
 int tdc_model_set_constants(const double *values, int32_t count);
 /* Measured tile selection, process-wide.  With classes > 0 every plan created WITHOUT a forced tile (single

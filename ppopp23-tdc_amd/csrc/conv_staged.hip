@@ -45,138 +45,9 @@
 //   * tiles are two-dimensional (TH x TW), so the halo is paid on a short
 //     perimeter instead of on whole image rows;
 //   * bias, residual add and ReLU are fused into the store.
-#include <hip/hip_runtime.h>
-
-#include <mutex>
-
-#include "tdc_internal.hpp"
-
-#ifndef TDC_TOUCH_KERNARGS
-#define TDC_TOUCH_KERNARGS 1
-#endif
-
-// Profiling build only (make STAMPS=1): every wave records s_memrealtime (the 100 MHz constant clock, comparable
-// across compute units and dies) at the boundaries of its phases and leaves the eight values in a plan-owned buffer,
-// [workgroup][wave][8].  The product build compiles none of it.
-#ifndef TDC_STAMPS
-#define TDC_STAMPS 0
-#endif
-#if TDC_STAMPS
-#define TDC_STAMP_DECL unsigned long long tdc_stamp_[8] = {0, 0, 0, 0, 0, 0, 0, 0}
-#define TDC_STAMP(i) tdc_stamp_[i] = __builtin_amdgcn_s_memrealtime()
-#define TDC_STAMP_FLUSH(p, wg, wave, lane)                                                             \
-    do {                                                                                               \
-        if ((p).stamps && (lane) == 0) {                                                               \
-            unsigned long long *dst_ = (p).stamps + ((size_t)(wg) * 16 + (wave)) * 8;                   \
-            for (int i_ = 0; i_ < 8; ++i_) dst_[i_] = tdc_stamp_[i_];                                   \
-        }                                                                                              \
-    } while (0)
-#else
-#define TDC_STAMP_DECL
-#define TDC_STAMP(i)
-#define TDC_STAMP_FLUSH(p, wg, wave, lane)
-#endif
+#include "conv_device.hpp"
 
 namespace tdc {
-
-typedef float f4_t __attribute__((ext_vector_type(4)));
-typedef float f16_t __attribute__((ext_vector_type(16)));
-typedef __attribute__((address_space(3))) void *lds_ptr_t;
-
-template <int MF>
-struct Mfma;
-
-// v_mfma_f32_32x32x2_f32: A lane l = A[l%32][l/32], B lane l = B[l/32][l%32],
-// D vgpr v lane l = D[8*(v/4) + 4*(l/32) + v%4][l%32].
-template <>
-struct Mfma<32> {
-    using acc_t = f16_t;
-    static constexpr int NACC = 16;
-    static constexpr int KC = 2;
-    static __device__ __forceinline__ acc_t run(float a, float b, acc_t c) {
-        return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
-    }
-    static __device__ __forceinline__ int row(int v, int lane) {
-        return 8 * (v >> 2) + 4 * (lane >> 5) + (v & 3);
-    }
-    static __device__ __forceinline__ int col(int lane) { return lane & 31; }
-    static __device__ __forceinline__ int ksub(int lane) { return lane >> 5; }
-};
-
-// v_mfma_f32_16x16x4_f32: A lane l = A[l%16][l/16], B lane l = B[l/16][l%16],
-// D vgpr v lane l = D[4*(l/16) + v][l%16].
-template <>
-struct Mfma<16> {
-    using acc_t = f4_t;
-    static constexpr int NACC = 4;
-    static constexpr int KC = 4;
-    static __device__ __forceinline__ acc_t run(float a, float b, acc_t c) {
-        return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
-    }
-    static __device__ __forceinline__ int row(int v, int lane) { return 4 * (lane >> 4) + v; }
-    static __device__ __forceinline__ int col(int lane) { return lane & 15; }
-    static __device__ __forceinline__ int ksub(int lane) { return lane >> 4; }
-};
-
-// TAPS_WINO: 3x3 / stride 1 as Winograd F(2x2,3x3).  A pixel lane holds one 2x2 output tile; per four input
-// channels a wave reads the 4x4 input patch of its tile from the SAME zero-haloed LDS window the direct path
-// uses, transforms it in registers (V = B^T d B, 32 additions), and feeds 16 MFMAs — one per position of the
-// transformed domain, against weights U = G g G^T prepared on the host — where the direct path needs 36 for
-// the same four pixels.  The 16 accumulators of a lane are combined at the end (Y = A^T M A, in registers:
-// every lane holds all 16 positions of its tile) into the 2x2 outputs.
-// TAPS_3x3G: the direct 3x3 loop with its weights read from global memory straight into registers (like the
-// Winograd path) instead of being staged in LDS: the LDS then holds input only and a pass can take all input channels.
-// (the TAPS_* values themselves are declared next to KernelId)
-
-constexpr int OOB_OFFSET = 0x7ffffff0;  // beyond any buffer: the load returns zero
-
-__device__ __forceinline__ int fdiv(int n, const FastDiv &f) {
-    return (int)(__umulhi((unsigned)n, f.m) + ((unsigned)n & f.pass));
-}
-
-// Epilogue of a lane that holds four consecutive output channels (from ch0) of one pixel: + bias, + residual, ReLU,
-// store.  All eight loads are requested before the first value is needed — one memory round trip for the lane
-// instead of one per load (written naively, every load sits behind the previous channel's store, which it might alias).
-__device__ __forceinline__ void finish_four_channels(const f4_t &acc, int ch0, int N, long long P, long long pix,
-                                                     const float *__restrict__ bias, const float *__restrict__ resid,
-                                                     int relu, float *__restrict__ out) {
-    float bv[4] = {0.0f, 0.0f, 0.0f, 0.0f}, rv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-    if (bias) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) bv[i] = bias[min(ch0 + i, N - 1)];
-    }
-    if (resid) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) rv[i] = resid[(long long)min(ch0 + i, N - 1) * P + pix];
-    }
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        if (ch0 + i >= N) continue;
-        float val = acc[i] + bv[i];
-        val += rv[i];
-        if (relu) val = fmaxf(val, 0.0f);
-        out[(long long)(ch0 + i) * P + pix] = val;
-    }
-}
-
-// The kernel arguments (about 400 bytes) are read through the scalar cache.  Left alone, the compiler fetches them in
-// several dependent batches, and every batch that touches a cache line for the first time costs a round trip to L2
-// before the first request can go out.  Touch every line of the argument block at once: whatever order the compiler
-// then loads the values in, it hits the scalar cache.
-__device__ __forceinline__ void touch_kernel_arguments() {
-    if constexpr (TDC_TOUCH_KERNARGS) {
-        static_assert(sizeof(ConvKParams) <= 8 * 64, "touch more lines");
-        const auto kargs = __builtin_amdgcn_kernarg_segment_ptr();
-        unsigned t0, t1, t2, t3, t4, t5, t6, t7;
-        asm volatile(
-            "s_load_dword %0, %8, 0x0\n\ts_load_dword %1, %8, 0x40\n\ts_load_dword %2, %8, 0x80\n\t"
-            "s_load_dword %3, %8, 0xc0\n\ts_load_dword %4, %8, 0x100\n\ts_load_dword %5, %8, 0x140\n\t"
-            "s_load_dword %6, %8, 0x180\n\ts_load_dword %7, %8, 0x1c0\n\ts_waitcnt lgkmcnt(0)"
-            : "=&s"(t0), "=&s"(t1), "=&s"(t2), "=&s"(t3), "=&s"(t4), "=&s"(t5), "=&s"(t6), "=&s"(t7)
-            : "s"(kargs)
-            : "memory");
-    }
-}
 
 // Copy planning.  A pass moves the input window of CCH channels and the weight
 // slab of those channels into one LDS stage.  The stage is cut into blocks of
@@ -1190,605 +1061,6 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
 }
 
 // ---------------------------------------------------------------------------
-// Streamed kernels whose input channels are split over KS workgroups: the lanes that hold a finished partial block
-// (`holder`: four consecutive channels from `ch0` of pixel `pp`) leave it in the workspace ws[image][slice][N][P]; the
-// workgroup that draws the last ticket of its (image, channel tile, pixel tile) reads all KS partials back and adds
-// them in slice order, so the result does not depend on which workgroup that is.  Same protocol as the staged
-// kernel: every workspace access is a relaxed device-scope atomic (written through, read past the die-local L2).
-// Returns false in the workgroups that are done; every thread of the workgroup must call it.
-// ---------------------------------------------------------------------------
-__device__ __forceinline__ bool stream_join_slices(const ConvKParams &p, float *lds, f4_t &acc, bool holder, int ch0,
-                                                   int pp, int img, int slice, int by, int bx) {
-    const long long NP = (long long)p.N * p.P;
-    if (holder) {
-        float *wsz = p.ws + ((long long)img * p.KS + slice) * NP;
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-            if (ch0 + i < p.N)
-                __hip_atomic_store(wsz + (long long)(ch0 + i) * p.P + pp, acc[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    __builtin_amdgcn_s_waitcnt(0);
-    __syncthreads();
-    unsigned *ticket = p.ctr + ((unsigned)img * p.grid_y + by) * p.grid_x + bx;
-    if (threadIdx.x == 0) {
-        const unsigned d = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        reinterpret_cast<unsigned *>(lds)[0] = d;
-    }
-    __syncthreads();
-    const unsigned drawn = reinterpret_cast<const unsigned *>(lds)[0];
-    if (drawn != (unsigned)p.KS - 1u) return false;
-    if (threadIdx.x == 0) __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // for the next launch
-    if (holder) {
-        const float *ws0 = p.ws + (long long)img * p.KS * NP;
-        float part[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) part[i] = 0.0f;
-        // (these loads go past the L2 and take a microsecond: eight slices are requested at once, then added in order)
-        for (int s0 = 0; s0 < p.KS; s0 += 8) {
-            float v[8][4];
-#pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                const float *src = ws0 + (long long)min(s0 + u, p.KS - 1) * NP + pp;
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    v[u][i] = __hip_atomic_load(src + (long long)min(ch0 + i, p.N - 1) * p.P, __ATOMIC_RELAXED,
-                                                __HIP_MEMORY_SCOPE_AGENT);
-            }
-#pragma unroll
-            for (int u = 0; u < 8; ++u)
-                if (s0 + u < p.KS) {
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) part[i] += v[u][i];
-                }
-        }
-#pragma unroll
-        for (int i = 0; i < 4; ++i) acc[i] = part[i];
-    }
-    return true;
-}
-
-// ---------------------------------------------------------------------------
-// 1x1 convolution with many input channels over few pixels (tile.alg = 3): no LDS stage, no passes, no barrier
-// before the reduction.  One workgroup owns a 16-channel x 16-pixel block of the output; its WK waves split the
-// input channels, NQ runs of 16 channels each.  A wave requests ALL its operands up front, straight into
-// registers (per run: one 128-bit load of packed weights, four 32-bit loads of the input, and two 128-bit loads of
-// the input affine if there is one), then issues its 4*NQ MFMAs as the data arrives and leaves its 16x16 partial
-// in LDS for wave 0 to add up in a fixed order.  Within a run lane (k, n) takes channels 16q + 4k + s over the four
-// K-steps s, so that its weights and its scale/shift pairs are contiguous.
-// Channels past C read as zero (range-checked vector offsets) and meet zero weights; pixel lanes past the image
-// re-read its last pixel and are never stored.
-// ---------------------------------------------------------------------------
-// (eight runs per wave: 72 registers of operands, 136 with the affine; that variant is built for at most 8 waves)
-// MODE 1: the instantiation whose input channels are dealt to p.KS workgroups.  MODE 2: stride > 1 (ResNet's downsampling
-// shortcuts): output pixel (oy, ox) reads input pixel (oy * stride, ox * stride).  The plain one pays for neither.
-template <int NQ, bool AFF, int MODE>
-__global__ void __launch_bounds__(NQ == 8 ? 512 : 1024) tdc_conv1x1_stream_kernel(const ConvKParams p) {
-    constexpr bool SPLIT = MODE == 1, STRIDED = MODE == 2;
-    extern __shared__ __align__(16) float lds[];
-    touch_kernel_arguments();
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // = this wave's slice of the input channels
-    // same die-aware decoding of the one-dimensional launch as the staged kernel
-    const int logical = (int)(blockIdx.x & 7u) * p.xcd_chunk + (int)(blockIdx.x >> 3);
-    if (logical >= p.n_wg) return;
-    const int q1 = fdiv(logical, p.fd_g1);
-    const int r1 = logical - q1 * p.fd_g1.d;
-    const int bz = fdiv(q1, p.fd_g2);          // image * KS + slice of the input channels
-    const int r2 = q1 - bz * p.fd_g2.d;
-    const int img = SPLIT ? fdiv(bz, p.fd_ks) : bz;
-    const int slice = SPLIT ? bz - img * p.KS : 0;
-    const int KS = SPLIT ? p.KS : 1;
-    const int bx = p.channel_major ? r1 : r2;  // pixel block
-    const int by = p.channel_major ? r2 : r1;  // channel block
-    const float *__restrict__ in = p.in + (long long)img * p.in_bstride;
-    float *__restrict__ out = p.out + (long long)img * p.out_bstride;
-    const float *__restrict__ resid = p.resid ? p.resid + (long long)img * p.resid_bstride : nullptr;
-    const __amdgpu_buffer_rsrc_t in_rsrc =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(in), (short)0, (int)p.in_image_bytes, 0x00020000);
-    const __amdgpu_buffer_rsrc_t w_rsrc =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.wpk), (short)0, (int)p.wpk_bytes, 0x00020000);
-
-    const int k = lane >> 4, n = lane & 15;
-    const int px = bx * 16 + n;
-    const int pxr = min(px, p.P - 1);
-    const int cl = wave * (16 * NQ) + 4 * k;   // this lane's first channel inside the workgroup's slice
-    const int c0 = slice * p.CCH + cl;         // ... and in the image
-    // bytes between channels (with stride 1 the host presents the image as one row of H*W pixels)
-    const unsigned HW4 = STRIDED ? (unsigned)(p.H * p.W) * 4u : (unsigned)p.W * 4u;
-    unsigned pix4 = (unsigned)pxr * 4u;        // this lane's input pixel, in bytes from the start of a channel
-    if constexpr (STRIDED) {
-        const int oy = fdiv(pxr, p.fd_wtw);    // (fd_wtw holds the output row length here)
-        const int ox = pxr - oy * p.Wo;
-        pix4 = (unsigned)((oy * p.W + ox) * p.stride) * 4u;
-    }
-
-    f4_t a[NQ], sc[NQ], sh[NQ];
-    float b[NQ][4];
-    const int a_soff = ((by * KS + slice) * (p.CCH >> 4) + wave * NQ) * 1024;
-    const unsigned b_voff = (unsigned)c0 * HW4 + pix4;
-#pragma unroll
-    for (int q = 0; q < NQ; ++q) {
-        a[q] = __builtin_bit_cast(f4_t, __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, lane * 16, a_soff + q * 1024, 0));
-#pragma unroll
-        for (int s4 = 0; s4 < 4; ++s4)   // (the whole offset goes through the range-checked vector operand)
-            b[q][s4] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(in_rsrc, (int)(b_voff + (unsigned)(16 * q + s4) * HW4), 0, 0));
-        if constexpr (AFF) {
-            const __amdgpu_buffer_rsrc_t aff_rsrc =
-                __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.in_aff + slice * 2 * p.CCH), (short)0, p.CCH * 8, 0x00020000);
-            sc[q] = __builtin_bit_cast(f4_t, __builtin_amdgcn_raw_buffer_load_b128(aff_rsrc, (cl + 16 * q) * 4, 0, 0));
-            sh[q] = __builtin_bit_cast(f4_t, __builtin_amdgcn_raw_buffer_load_b128(aff_rsrc, (p.CCH + cl + 16 * q) * 4, 0, 0));
-        }
-        __builtin_amdgcn_sched_barrier(0);   // requests in the order the MFMAs consume them
-    }
-    // (every request is issued before the first MFMA: the scheduler must not sink loads into the MFMA sequence)
-    __builtin_amdgcn_sched_barrier(0);
-    // two accumulator chains: consecutive MFMAs do not wait for each other's result
-    f4_t acc0 = (f4_t){0.0f, 0.0f, 0.0f, 0.0f}, acc1 = (f4_t){0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-    for (int q = 0; q < NQ; ++q) {
-#pragma unroll
-        for (int s4 = 0; s4 < 4; ++s4) {
-            float v = b[q][s4];
-            if constexpr (AFF) {
-                v = v * sc[q][s4] + sh[q][s4];
-                if (p.in_relu) v = fmaxf(v, 0.0f);
-            }
-            if (s4 & 1) acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(a[q][s4], v, acc1, 0, 0, 0);
-            else acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(a[q][s4], v, acc0, 0, 0, 0);
-        }
-        __builtin_amdgcn_sched_barrier(0);   // run by run, as the data arrives
-    }
-    f4_t acc = acc0 + acc1;
-    // lane l holds rows 4*(l/16) .. +3 (output channels) of column l%16 (pixel)
-    if (p.WK > 1) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) lds[(wave * 4 + i) * 64 + lane] = acc[i];
-        __syncthreads();
-        if (wave == 0) {
-            acc = (f4_t){0.0f, 0.0f, 0.0f, 0.0f};
-            for (int w = 0; w < p.WK; ++w)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) acc[i] += lds[(w * 4 + i) * 64 + lane];
-        }
-    }
-    if constexpr (SPLIT) {
-        // the input channels are split over KS workgroups: whoever finishes last adds the partial blocks in slice order
-        if (!stream_join_slices(p, lds, acc, wave == 0 && px < p.P, by * 16 + 4 * k, px, img, slice, by, bx)) return;
-    }
-    if (wave != 0 || px >= p.P) return;
-    finish_four_channels(acc, by * 16 + 4 * k, p.N, p.P, px, p.bias, resid, p.relu, out);
-}
-
-// ---------------------------------------------------------------------------
-// 3x3 convolution streamed the same way (tile.alg = 4): one workgroup owns 16 output channels of a TH x TW tile of 16
-// pixels, its WK waves split the input channels, CG groups of four channels each.  Per group a lane requests its nine
-// input values (one per tap, four channels across the lane quarters) and its nine weights (packed as for
-// tile.alg = 2: two 128-bit loads and one 32-bit load); padding, channels past C and lanes past the tile present an
-// out-of-range offset and read zero without a memory access.
-// ---------------------------------------------------------------------------
-// ROW (stride 1 and a tile of one row of 14 pixels): the 16 lanes of a quarter load the 16 consecutive input pixels
-// that the row of outputs touches, once per filter row, and the three taps of a row are lane shifts of that value
-// (three requests per group of channels instead of nine).
-// MODE: 0 = plain, 1 = input channels dealt to p.KS workgroups, 2 = with the fused 1x1 tail, 3 = with a fused 1x1 head in
-// front as well (a whole Tucker convolution in one launch: the workgroup first computes the first factor on its window of
-// (TH + 2) x (TW + 2) pixels into LDS, which the core loop then reads instead of global memory).  Separate instantiations:
-// code a launch never runs still costs it (0.13 us per launch measured for the split's code inside the plain kernel).
-template <int CG, bool ROW, int MODE>
-__global__ void __launch_bounds__(1024) tdc_conv3x3_stream_kernel(const ConvKParams p) {
-    constexpr bool SPLIT = MODE == 1, TAIL = MODE == 2 || MODE == 3, HEAD = MODE == 3;
-    extern __shared__ __align__(16) float lds[];
-    touch_kernel_arguments();
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int logical = (int)(blockIdx.x & 7u) * p.xcd_chunk + (int)(blockIdx.x >> 3);
-    if (logical >= p.n_wg) return;
-    const int q1 = fdiv(logical, p.fd_g1);
-    const int r1 = logical - q1 * p.fd_g1.d;
-    const int bz = fdiv(q1, p.fd_g2);          // image * KS + slice of the input channels
-    const int r2 = q1 - bz * p.fd_g2.d;
-    const int img = SPLIT ? fdiv(bz, p.fd_ks) : bz;
-    const int slice = SPLIT ? bz - img * p.KS : 0;
-    const int KS = SPLIT ? p.KS : 1;
-    const int bx = p.channel_major ? r1 : r2;  // pixel tile
-    const int by = p.channel_major ? r2 : r1;  // channel block
-    const int tile_y = fdiv(bx, p.fd_ntx);
-    const int tile_x = bx - tile_y * p.ntx;
-    const float *__restrict__ in = p.in + (long long)img * p.in_bstride;
-    float *__restrict__ out = p.out + (long long)img * p.out_bstride;
-    const float *__restrict__ resid = p.resid ? p.resid + (long long)img * p.resid_bstride : nullptr;
-    const __amdgpu_buffer_rsrc_t in_rsrc =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(in), (short)0, (int)p.in_image_bytes, 0x00020000);
-    const __amdgpu_buffer_rsrc_t w_rsrc =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.wpk), (short)0, (int)p.wpk_bytes, 0x00020000);
-
-    // wave = (channel block of the workgroup) * WK + (slice of the input channels)
-    const int wmi = fdiv(wave, p.fd_wk);
-    const int wki = wave - wmi * p.WK;
-    const int mblk = by * p.WM + wmi;   // this wave's block of 16 output channels
-    // The weights depend on nothing but the channel block and the wave: request them before any pixel arithmetic.
-    // packed as [channel tile][slice][block of the workgroup][group]: nine taps x 64 lanes x 4 bytes per group
-    const int a_soff = ((((by * KS + slice) * p.WM + wmi) * (p.CCH >> 2)) + wki * CG) * 2304;
-    f4_t a0[CG], a1[CG];
-    float a8[CG], b[CG][9];
-#pragma unroll
-    for (int g = 0; g < CG; ++g) {
-        a0[g] = __builtin_bit_cast(f4_t, __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, lane * 16, a_soff + g * 2304, 0));
-        a1[g] = __builtin_bit_cast(f4_t, __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, lane * 16, a_soff + g * 2304 + 1024, 0));
-        a8[g] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(w_rsrc, lane * 4, a_soff + g * 2304 + 2048, 0));
-    }
-    __builtin_amdgcn_sched_barrier(0);
-
-    const int k = lane >> 4, n = lane & 15;
-    const int jy = fdiv(n, p.fd_tw);
-    const int jx = n - jy * p.TW;
-    const int oy = tile_y * p.TH + jy, ox = tile_x * p.TW + jx;
-    const bool live = jy < p.TH && oy < p.Ho && ox < p.Wo;
-    const int iy0 = oy * p.stride - p.pad, ix0 = ox * p.stride - p.pad;
-    const unsigned rowb = (unsigned)p.W * 4u;
-    const unsigned chan_bytes = (unsigned)(p.H * p.W) * 4u;
-    const unsigned base = (unsigned)(slice * p.CCH + wki * (4 * CG) + k) * chan_bytes;   // this lane's first channel
-    if constexpr (HEAD) {
-        // First factor on the window: 16 x 16 blocks (channels x window pixels) dealt to the waves, both operands
-        // streamed from global memory four runs of 16 input channels at a time; pixels outside the image read zero,
-        // which is the core's zero padding (the factor has no bias).
-        float *F = lds + p.head_f_off;
-        const __amdgpu_buffer_rsrc_t hw_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-            const_cast<float *>(p.head_w), (short)0, p.head_mblk * p.head_runs * 1024, 0x00020000);
-        const int nwaves = p.WM * p.WK;
-        const int nblk = p.head_mblk * p.head_npb;
-        for (int blk = wave; blk < nblk; blk += nwaves) {
-            const int cb = fdiv(blk, p.fd_hnpb);
-            const int pb = blk - cb * p.head_npb;
-            const int wq = pb * 16 + n;
-            const int wy = fdiv(wq, p.fd_hww);
-            const int wx = wq - wy * p.head_ww;
-            const int iy = tile_y * p.TH - p.pad + wy, ix = tile_x * p.TW - p.pad + wx;
-            const bool ok = wq < p.head_wq && (unsigned)iy < (unsigned)p.H && (unsigned)ix < (unsigned)p.W;
-            const unsigned pix = ok ? (unsigned)(iy * p.W + ix) * 4u + (unsigned)(4 * k) * chan_bytes : (unsigned)OOB_OFFSET;
-            f4_t h0 = (f4_t){0.0f, 0.0f, 0.0f, 0.0f}, h1 = (f4_t){0.0f, 0.0f, 0.0f, 0.0f};
-            // (four runs per round trip: eight at once measured slower, the workgroup is bound by its compute unit's fill rate)
-            for (int q0 = 0; q0 < p.head_runs; q0 += 4) {
-                f4_t ha[4];
-                float hb[4][4];
-#pragma unroll
-                for (int u = 0; u < 4; ++u) {
-                    ha[u] = __builtin_bit_cast(f4_t, __builtin_amdgcn_raw_buffer_load_b128(
-                                                         hw_rsrc, lane * 16, (cb * p.head_runs + q0 + u) * 1024, 0));
-#pragma unroll
-                    for (int s4 = 0; s4 < 4; ++s4)
-                        hb[u][s4] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
-                            in_rsrc, (int)(pix + (unsigned)(16 * (q0 + u) + s4) * chan_bytes), 0, 0));
-                }
-#pragma unroll
-                for (int u = 0; u < 4; ++u)
-#pragma unroll
-                    for (int s4 = 0; s4 < 4; ++s4) {
-                        if (s4 & 1) h1 = __builtin_amdgcn_mfma_f32_16x16x4f32(ha[u][s4], hb[u][s4], h1, 0, 0, 0);
-                        else h0 = __builtin_amdgcn_mfma_f32_16x16x4f32(ha[u][s4], hb[u][s4], h0, 0, 0, 0);
-                    }
-            }
-            const f4_t h = h0 + h1;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) F[(cb * 16 + 4 * k + i) * p.head_ld + wq] = h[i];
-        }
-        __syncthreads();
-        // the core's pixel operand comes from that window: output pixel (jy, jx), tap (r, c) = window pixel (jy + r, jx + c)
-        const float *Fk = F + (wki * (4 * CG) + k) * p.head_ld;
-        const int wmax = p.head_npb * 16 - 1;
-#pragma unroll
-        for (int g = 0; g < CG; ++g)
-#pragma unroll
-            for (int t = 0; t < 9; ++t)
-                b[g][t] = Fk[4 * g * p.head_ld + min((jy + t / 3) * p.head_ww + jx + t % 3, wmax)];
-    } else
-    if constexpr (ROW) {
-        // lane n of a quarter: input column (tile's first column - pad + n) of the three input rows
-        const int iyr = tile_y - p.pad, ixr = tile_x * 14 - p.pad + n;
-        unsigned roff[3];
-#pragma unroll
-        for (int r = 0; r < 3; ++r) {
-            const bool ok = (unsigned)(iyr + r) < (unsigned)p.H && (unsigned)ixr < (unsigned)p.W;
-            const unsigned m = ok ? 0xffffffffu : 0u;
-            roff[r] = ((unsigned)((iyr + r) * p.W + ixr) * 4u & m) | ((unsigned)OOB_OFFSET & ~m);
-        }
-        float rowv[CG][3];
-#pragma unroll
-        for (int g = 0; g < CG; ++g) {
-#pragma unroll
-            for (int r = 0; r < 3; ++r)
-                rowv[g][r] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
-                    in_rsrc, (int)(roff[r] + base + (unsigned)(4 * g) * chan_bytes), 0, 0));
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int g = 0; g < CG; ++g)
-#pragma unroll
-            for (int r = 0; r < 3; ++r) {
-                const int v = __builtin_bit_cast(int, rowv[g][r]);
-                b[g][r * 3 + 0] = rowv[g][r];
-                // row_shl:1 / row_shl:2 within the 16 lanes of a quarter: lane n takes the value of lane n+1 / n+2
-                b[g][r * 3 + 1] = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, v, 0x101, 0xf, 0xf, true));
-                b[g][r * 3 + 2] = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, v, 0x102, 0xf, 0xf, true));
-            }
-    } else {
-        // byte offset of every tap inside one channel, or the out-of-range offset (branch-free: row and column tests apart)
-        const unsigned off0 = (unsigned)(iy0 * p.W + ix0) * 4u;
-        unsigned rmask[3], cmask[3];
-#pragma unroll
-        for (int r = 0; r < 3; ++r) {
-            rmask[r] = ((unsigned)(iy0 + r) < (unsigned)p.H && live) ? 0xffffffffu : 0u;
-            cmask[r] = ((unsigned)(ix0 + r) < (unsigned)p.W) ? 0xffffffffu : 0u;
-        }
-        unsigned toff[9];
-#pragma unroll
-        for (int r = 0; r < 3; ++r)
-#pragma unroll
-            for (int c = 0; c < 3; ++c) {
-                const unsigned m = rmask[r] & cmask[c];
-                toff[r * 3 + c] = ((off0 + (unsigned)r * rowb + (unsigned)c * 4u) & m) | ((unsigned)OOB_OFFSET & ~m);
-            }
-#pragma unroll
-        for (int g = 0; g < CG; ++g) {
-#pragma unroll
-            for (int t = 0; t < 9; ++t)   // (the whole offset goes through the range-checked vector operand)
-                b[g][t] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
-                    in_rsrc, (int)(toff[t] + base + (unsigned)(4 * g) * chan_bytes), 0, 0));
-            __builtin_amdgcn_sched_barrier(0);   // requests in the order the MFMAs consume them
-        }
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    f4_t acc0 = (f4_t){0.0f, 0.0f, 0.0f, 0.0f}, acc1 = (f4_t){0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-    for (int g = 0; g < CG; ++g) {
-#pragma unroll
-        for (int t = 0; t < 9; ++t) {
-            const float av = t < 4 ? a0[g][t] : t < 8 ? a1[g][t - 4] : a8[g];
-            if (t & 1) acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(av, b[g][t], acc1, 0, 0, 0);
-            else acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(av, b[g][t], acc0, 0, 0, 0);
-        }
-        __builtin_amdgcn_sched_barrier(0);   // group by group, as the data arrives
-    }
-    f4_t acc = acc0 + acc1;
-    // lane l holds rows 4*(l/16) .. +3 (output channels) of column l%16 (pixel); the slices of a channel block are
-    // added by its first wave, in slice order
-    if (p.WK > 1) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) lds[(wave * 4 + i) * 64 + lane] = acc[i];
-        __syncthreads();
-        if (wki == 0) {
-            acc = (f4_t){0.0f, 0.0f, 0.0f, 0.0f};
-            for (int w = 0; w < p.WK; ++w)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) acc[i] += lds[((wave + w) * 4 + i) * 64 + lane];
-        }
-    }
-    const int pp = oy * p.Wo + ox;
-    if constexpr (TAIL) {
-        // Fused 1x1 tail, out2 = W2 * act(conv + bias): the workgroup owns every output channel of the convolution
-        // (the host guarantees it).  The finished 16-pixel columns are parked in LDS as f[channel][pixel] — the B operand
-        // of a second small GEMM whose A operand, the tail's packed weights, comes from global memory — and its
-        // 16x16 output blocks are dealt to all waves.
-        float *f = lds + p.tail_f_off;
-        const int LD = p.tail_ld;
-        if (wki == 0) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int ml = wmi * 16 + 4 * k + i;
-                const int ch = by * 16 * p.WM + ml;
-                float val = acc[i];
-                if (p.bias && ch < p.N) val += p.bias[ch];
-                if (p.relu) val = fmaxf(val, 0.0f);
-                f[ml * LD + n] = val;
-            }
-        }
-        __syncthreads();
-        const int nwaves = p.WM * p.WK;
-        for (int blk = wave; blk < p.tail_mblk; blk += nwaves) {
-            const float *wa = p.tail_w + (size_t)blk * p.tail_ng * 64 + lane;
-            const float *fb = f + k * LD + n;
-            // (bias and residual of this block are requested before the small GEMM and arrive under it)
-            const int n20 = blk * 16 + 4 * k;
-            const long long ppc = live ? pp : 0;
-            float tbv[4] = {0.0f, 0.0f, 0.0f, 0.0f}, trv[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-            if (p.tail_bias) {
-#pragma unroll
-                for (int v = 0; v < 4; ++v) tbv[v] = p.tail_bias[min(n20 + v, p.tail_N - 1)];
-            }
-            if (resid) {
-#pragma unroll
-                for (int v = 0; v < 4; ++v) trv[v] = resid[(long long)min(n20 + v, p.tail_N - 1) * p.P + ppc];
-            }
-            f4_t acc2 = {0.0f, 0.0f, 0.0f, 0.0f};
-            for (int g0 = 0; g0 < p.tail_ng; g0 += 4) {
-                float ta[4], tb[4];
-#pragma unroll
-                for (int u = 0; u < 4; ++u) {
-                    const int g = min(g0 + u, p.tail_ng - 1);
-                    ta[u] = wa[g * 64];
-                    tb[u] = fb[g * 4 * LD];
-                }
-#pragma unroll
-                for (int u = 0; u < 4; ++u)
-                    if (g0 + u < p.tail_ng) acc2 = __builtin_amdgcn_mfma_f32_16x16x4f32(ta[u], tb[u], acc2, 0, 0, 0);
-            }
-            if (live) {
-#pragma unroll
-                for (int v = 0; v < 4; ++v) {
-                    const int n2 = n20 + v;
-                    if (n2 < p.tail_N) {
-                        float val = acc2[v] + tbv[v];
-                        val += trv[v];
-                        if (p.tail_relu) val = fmaxf(val, 0.0f);
-                        out[(long long)n2 * p.P + pp] = val;
-                    }
-                }
-            }
-        }
-        return;
-    }
-    if constexpr (SPLIT) {
-        if (!stream_join_slices(p, lds, acc, wki == 0 && live, mblk * 16 + 4 * k, pp, img, slice, by, bx)) return;
-    }
-    if (wki != 0 || !live) return;
-    finish_four_channels(acc, mblk * 16 + 4 * k, p.N, p.P, pp, p.bias, resid, p.relu, out);
-}
-
-// ---------------------------------------------------------------------------
-// The streamed 3x3 kernel with NB pixel blocks per wave (tile.alg = 4, tile.nb = 2 or 4; stride 1, rows of 14 pixels).
-// The 16 x 16 block of the plain kernel reads the weights of its 16 channels once per 16 pixels and moves 30 times the
-// algorithmic bytes through the L2s on the mid-size layers (64 -> 64 @56x56: 54 MB for 1.75 MB), which is what bounds
-// them.  Here a workgroup owns NB horizontally adjacent 14-pixel row tiles: a wave still takes CG groups of four input
-// channels and requests everything up front, but every weight operand it holds feeds NB MFMAs, one per pixel block,
-// so the weights cross the L2 -> CU path NB times less often.  Per group and block a lane requests three values (one
-// per filter row; the three taps of a row are lane shifts, as in the plain kernel's row mode).  The partial blocks
-// of the WK waves meet in LDS as [wave][block][register][lane] and ALL threads share the final sum (in wave order, so
-// the result does not depend on timing) and the store.
-// ---------------------------------------------------------------------------
-template <int CG, int NB>
-__global__ void __launch_bounds__(1024) tdc_conv3x3_stream_rownb_kernel(const ConvKParams p) {
-    extern __shared__ __align__(16) float lds[];
-    TDC_STAMP_DECL;
-    TDC_STAMP(0);   // entry
-    touch_kernel_arguments();
-    TDC_STAMP(7);   // every line of the kernel arguments is in the scalar cache
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int logical = (int)(blockIdx.x & 7u) * p.xcd_chunk + (int)(blockIdx.x >> 3);
-    if (logical >= p.n_wg) return;
-    const int q1 = fdiv(logical, p.fd_g1);
-    const int r1 = logical - q1 * p.fd_g1.d;
-    const int img = fdiv(q1, p.fd_g2);
-    const int r2 = q1 - img * p.fd_g2.d;
-    const int bx = p.channel_major ? r1 : r2;  // pixel tile of the workgroup: NB blocks side by side
-    const int by = p.channel_major ? r2 : r1;  // channel tile
-    const int tile_y = fdiv(bx, p.fd_ntx);     // = output row (tiles are one row high)
-    const int tile_x = bx - tile_y * p.ntx;
-    const float *__restrict__ in = p.in + (long long)img * p.in_bstride;
-    float *__restrict__ out = p.out + (long long)img * p.out_bstride;
-    const float *__restrict__ resid = p.resid ? p.resid + (long long)img * p.resid_bstride : nullptr;
-    const __amdgpu_buffer_rsrc_t in_rsrc =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(in), (short)0, (int)p.in_image_bytes, 0x00020000);
-    const __amdgpu_buffer_rsrc_t w_rsrc =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(p.wpk), (short)0, (int)p.wpk_bytes, 0x00020000);
-
-    // wave = (channel block of the workgroup) * WK + (slice of the input channels)
-    const int wmi = fdiv(wave, p.fd_wk);
-    const int wki = wave - wmi * p.WK;
-    // weights first: they depend on nothing but the channel block and the wave (packed as for the plain kernel)
-    const int a_soff = (((by * p.WM + wmi) * (p.CCH >> 2)) + wki * CG) * 2304;
-    f4_t a0[CG], a1[CG];
-    float a8[CG];
-#pragma unroll
-    for (int g = 0; g < CG; ++g) {
-        a0[g] = __builtin_bit_cast(f4_t, __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, lane * 16, a_soff + g * 2304, 0));
-        a1[g] = __builtin_bit_cast(f4_t, __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, lane * 16, a_soff + g * 2304 + 1024, 0));
-        a8[g] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(w_rsrc, lane * 4, a_soff + g * 2304 + 2048, 0));
-    }
-    __builtin_amdgcn_sched_barrier(0);
-
-    const int k = lane >> 4, n = lane & 15;
-    const unsigned chan_bytes = (unsigned)(p.H * p.W) * 4u;
-    const unsigned base = (unsigned)(wki * (4 * CG) + k) * chan_bytes;   // this lane's first channel
-    // lane n of a quarter: input column (block's first column - pad + n) of the three input rows under the output row
-    const int iyr = tile_y - p.pad;
-    unsigned roff[NB][3];
-#pragma unroll
-    for (int blk = 0; blk < NB; ++blk) {
-        const int ixr = (tile_x * NB + blk) * 14 - p.pad + n;
-#pragma unroll
-        for (int r = 0; r < 3; ++r) {
-            const bool ok = (unsigned)(iyr + r) < (unsigned)p.H && (unsigned)ixr < (unsigned)p.W;
-            const unsigned m = ok ? 0xffffffffu : 0u;
-            roff[blk][r] = ((unsigned)((iyr + r) * p.W + ixr) * 4u & m) | ((unsigned)OOB_OFFSET & ~m);
-        }
-    }
-    float rowv[CG][NB][3];
-#pragma unroll
-    for (int g = 0; g < CG; ++g) {
-#pragma unroll
-        for (int blk = 0; blk < NB; ++blk)
-#pragma unroll
-            for (int r = 0; r < 3; ++r)
-                rowv[g][blk][r] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
-                    in_rsrc, (int)(roff[blk][r] + base + (unsigned)(4 * g) * chan_bytes), 0, 0));
-        __builtin_amdgcn_sched_barrier(0);   // requests in the order the MFMAs consume them
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    TDC_STAMP(1);   // every request issued
-    f4_t acc[NB];
-#pragma unroll
-    for (int blk = 0; blk < NB; ++blk) acc[blk] = (f4_t){0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-    for (int g = 0; g < CG; ++g) {
-#pragma unroll
-        for (int r = 0; r < 3; ++r) {
-#pragma unroll
-            for (int c = 0; c < 3; ++c) {
-                const int t = r * 3 + c;
-                const float av = t < 4 ? a0[g][t] : t < 8 ? a1[g][t - 4] : a8[g];
-#pragma unroll
-                for (int blk = 0; blk < NB; ++blk) {
-                    const int v = __builtin_bit_cast(int, rowv[g][blk][r]);
-                    // row_shl:c within the 16 lanes of a quarter: lane n takes the value of lane n + c
-                    const float bv = c == 0 ? rowv[g][blk][r]
-                                   : c == 1 ? __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, v, 0x101, 0xf, 0xf, true))
-                                            : __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, v, 0x102, 0xf, 0xf, true));
-                    acc[blk] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, bv, acc[blk], 0, 0, 0);
-                }
-            }
-        }
-        __builtin_amdgcn_sched_barrier(0);   // group by group, as the data arrives
-    }
-    TDC_STAMP(4);   // MFMAs issued (the last results may still be in the pipe)
-    // lane l of block blk holds rows 4*(l/16) .. +3 (output channels) of column l%16 (pixel)
-#pragma unroll
-    for (int blk = 0; blk < NB; ++blk)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) lds[((wave * NB + blk) * 4 + i) * 64 + lane] = acc[blk][i];
-    __syncthreads();
-    TDC_STAMP(5);   // everybody's partial blocks are in LDS
-    const int nthreads = blockDim.x;
-    const int total = p.WM * NB * 256;
-    for (int idx = tid; idx < total; idx += nthreads) {
-        const int l = idx & 63, i = (idx >> 6) & 3;
-        const int rest = idx >> 8;                     // = channel block of the workgroup * NB + pixel block
-        const int cb = rest / NB, blk = rest - cb * NB;
-        const float *src = lds + (((cb * p.WK) * NB + blk) * 4 + i) * 64 + l;
-        const int wstride = NB * 256;
-        const int ch = (by * p.WM + cb) * 16 + 4 * (l >> 4) + i;
-        const int px = l & 15;
-        const int ox = (tile_x * NB + blk) * 14 + px;
-        const bool ok = ch < p.N && px < 14 && ox < p.Wo;
-        const long long o = ok ? (long long)ch * p.P + tile_y * p.Wo + ox : 0;
-        // (bias and residual are requested before the partial sums are read and arrive under those reads)
-        const float bv = p.bias ? p.bias[min(ch, p.N - 1)] : 0.0f;
-        const float rv = resid ? resid[o] : 0.0f;
-        float val = 0.0f;
-        // four reads in flight at a time; the additions stay in wave order
-        for (int w0 = 0; w0 < p.WK; w0 += 4) {
-            float part[4];
-#pragma unroll
-            for (int u = 0; u < 4; ++u) part[u] = src[min(w0 + u, p.WK - 1) * wstride];
-#pragma unroll
-            for (int u = 0; u < 4; ++u)
-                if (w0 + u < p.WK) val += part[u];
-        }
-        if (ok) {
-            val += bv;
-            val += rv;
-            if (p.relu) val = fmaxf(val, 0.0f);
-            out[o] = val;
-        }
-    }
-    TDC_STAMP(6);   // stores issued
-    TDC_STAMP_FLUSH(p, logical, wave, lane);
-}
-
-// ---------------------------------------------------------------------------
 // Instantiation table: KernelId (worked out on the host from tile and filter, see kernel_id_for) -> function.
 // A 2x2 block grid of MFMAs per wave is built for at most 8 waves per workgroup (256 registers per lane), the
 // Winograd loop for 12, everything else for 16.
@@ -1811,28 +1083,7 @@ static kernel_fn pick_mf(int mf, int mb, int nb) {
     return nullptr;
 }
 
-template <bool AFF, int MODE>
-static kernel_fn pick_stream(int nq) {
-    switch (nq) {
-        case 1: return tdc_conv1x1_stream_kernel<1, AFF, MODE>;
-        case 2: return tdc_conv1x1_stream_kernel<2, AFF, MODE>;
-        case 4: return tdc_conv1x1_stream_kernel<4, AFF, MODE>;
-        case 8: return tdc_conv1x1_stream_kernel<8, AFF, MODE>;
-        default: return nullptr;
-    }
-}
-
-template <bool ROW, int MODE>
-static kernel_fn pick_stream3(int groups) {
-    switch (groups) {
-        case 1: return tdc_conv3x3_stream_kernel<1, ROW, MODE>;
-        case 2: return tdc_conv3x3_stream_kernel<2, ROW, MODE>;
-        case 4: return tdc_conv3x3_stream_kernel<4, ROW, MODE>;
-        default: return nullptr;
-    }
-}
-
-const void *kernel_function(const KernelId &k) {
+const void *staged_kernel_function(const KernelId &k) {
     kernel_fn fn = nullptr;
     if (k.family == KernelId::STAGED) {
         const bool ext = k.p[5] != 0;
@@ -1851,109 +1102,8 @@ const void *kernel_function(const KernelId &k) {
             case TAPS_GENERIC: fn = ext ? pick_mf<TAPS_GENERIC, true>(k.p[0], k.p[1], k.p[2]) : pick_mf<TAPS_GENERIC, false>(k.p[0], k.p[1], k.p[2]); break;
             default: break;
         }
-    } else if (k.family == KernelId::STREAM_1x1) {
-        const int nq = k.p[0], mode = k.p[2];
-        if (k.p[1]) fn = mode == 2 ? pick_stream<true, 2>(nq) : mode == 1 ? pick_stream<true, 1>(nq) : mode == 0 ? pick_stream<true, 0>(nq) : nullptr;
-        else fn = mode == 2 ? pick_stream<false, 2>(nq) : mode == 1 ? pick_stream<false, 1>(nq) : mode == 0 ? pick_stream<false, 0>(nq) : nullptr;
-    } else if (k.family == KernelId::STREAM_3x3 && k.p[3] > 1) {
-        // NB pixel blocks per wave: rows of 14 pixels, plain mode only
-        const int cg = k.p[0], nb = k.p[3];
-        if (k.p[1] && k.p[2] == 0) {
-            if (nb == 2) fn = cg == 1 ? static_cast<kernel_fn>(tdc_conv3x3_stream_rownb_kernel<1, 2>)
-                            : cg == 2 ? static_cast<kernel_fn>(tdc_conv3x3_stream_rownb_kernel<2, 2>)
-                            : cg == 4 ? static_cast<kernel_fn>(tdc_conv3x3_stream_rownb_kernel<4, 2>) : nullptr;
-            if (nb == 4) fn = cg == 1 ? static_cast<kernel_fn>(tdc_conv3x3_stream_rownb_kernel<1, 4>)
-                            : cg == 2 ? static_cast<kernel_fn>(tdc_conv3x3_stream_rownb_kernel<2, 4>)
-                            : cg == 4 ? static_cast<kernel_fn>(tdc_conv3x3_stream_rownb_kernel<4, 4>) : nullptr;
-        }
-    } else if (k.family == KernelId::STREAM_3x3) {
-        const int cg = k.p[0], mode = k.p[2];
-        if (k.p[1]) fn = mode == 2 ? pick_stream3<true, 2>(cg) : mode == 1 ? pick_stream3<true, 1>(cg) : mode == 0 ? pick_stream3<true, 0>(cg) : nullptr;
-        else fn = mode == 3 ? pick_stream3<false, 3>(cg) : mode == 2 ? pick_stream3<false, 2>(cg) : mode == 1 ? pick_stream3<false, 1>(cg)
-                : mode == 0 ? pick_stream3<false, 0>(cg) : nullptr;
     }
     return reinterpret_cast<const void *>(fn);
-}
-
-// ---------------------------------------------------------------------------
-// Static scratch for callers that cannot allocate (HIP graph capture, serving loops whose harness forbids
-// hipMalloc): the partial tiles and ticket counters of a split across workgroups (tile.ks > 1) in a device array
-// that exists from module load to process exit, one copy per GPU.  4 MiB of partial tiles (256 -> 256 @7x7 with four
-// slices needs 0.2 MiB, 2048 -> 256 @7x7 with eight 0.4 MiB) and 64 KiB of counters.
-// In host code the array's NAME is not a device address; its address on the current device comes from
-// hipGetSymbolAddress and is kept per device.
-// ---------------------------------------------------------------------------
-constexpr size_t kScratchWsBytes = 4u << 20;
-constexpr size_t kScratchCtrBytes = 64u << 10;
-static __device__ __align__(256) unsigned char scratch[kScratchWsBytes + kScratchCtrBytes];
-
-size_t static_scratch_ws_bytes() { return kScratchWsBytes; }
-size_t static_scratch_ctr_bytes() { return kScratchCtrBytes; }
-
-int static_scratch_address(void **ptr_out) {
-    constexpr int kMaxDevices = 64;
-    static void *per_device[kMaxDevices] = {};
-    static std::mutex mtx;
-    int dev = 0;
-    hipError_t e = hipGetDevice(&dev);
-    if (e != hipSuccess) return (int)e;
-    if (dev < 0 || dev >= kMaxDevices) return (int)hipErrorInvalidDevice;
-    std::lock_guard<std::mutex> lock(mtx);
-    if (!per_device[dev]) {
-        void *p = nullptr;
-        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));   // the address of this device's copy
-        if (e != hipSuccess) return (int)e;
-        if (!p) return (int)hipErrorInvalidSymbol;
-        per_device[dev] = p;
-    }
-    *ptr_out = per_device[dev];
-    return 0;
-}
-
-__global__ void __launch_bounds__(256) tdc_zero_words_kernel(unsigned *dst, int n) {
-    const int i = blockIdx.x * 256 + threadIdx.x;
-    if (i < n) dst[i] = 0u;
-}
-
-int launch_zero_words(unsigned *dst, int n, void *stream) {
-    if (n <= 0) return 0;
-    hipLaunchKernelGGL(tdc_zero_words_kernel, dim3((n + 255) / 256), dim3(256), 0, (hipStream_t)stream, dst, n);
-    return (int)hipGetLastError();
-}
-
-int kernel_resources(const void *fn, int block_threads, int dynamic_lds_bytes, int *vgprs, int *static_lds, int *max_threads,
-                     int *max_wg_per_cu) {
-    hipFuncAttributes attr{};
-    hipError_t e = hipFuncGetAttributes(&attr, fn);
-    if (e != hipSuccess) return (int)e;
-    int blocks = 0;
-    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, fn, block_threads, (size_t)dynamic_lds_bytes);
-    if (e != hipSuccess) return (int)e;
-    *vgprs = attr.numRegs;
-    *static_lds = (int)attr.sharedSizeBytes;
-    *max_threads = attr.maxThreadsPerBlock;
-    *max_wg_per_cu = blocks;
-    return 0;
-}
-
-int prepare_conv_kernel(const void *fn, const Geometry &g) {
-    if (!fn) return (int)hipErrorInvalidValue;
-    // Dynamic LDS above the 64 KiB default has to be opted into per kernel function.  The attribute belongs to
-    // the function, not to the plan, and several plans share one instantiation: always raise it to the whole
-    // LDS, so that a later plan with a smaller request cannot lower it under an earlier plan's feet.
-    if (g.lds_bytes > 64 * 1024) {
-        hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, machine().lds_bytes_per_cu);
-        if (e != hipSuccess) return (int)e;
-    }
-    return 0;
-}
-
-int launch_conv(const void *fn, const Geometry &g, const ConvKParams &kp, void *stream) {
-    if (!fn) return (int)hipErrorInvalidValue;
-    dim3 grid(8 * kp.xcd_chunk), block(g.threads);
-    hipLaunchKernelGGL(reinterpret_cast<kernel_fn>(const_cast<void *>(fn)), grid, block,
-                       (size_t)g.lds_bytes, (hipStream_t)stream, kp);
-    return (int)hipGetLastError();
 }
 
 }  // namespace tdc

@@ -59,7 +59,7 @@ struct Geometry {
     int nstage = 1;
     int lds_bytes = 0;
     int max_waves_kernel = 0;        // launch bound of the instantiated kernel
-    int channel_major = 0;           // which logical workgroup order costs fewer L2 fills (see conv_mfma.hip)
+    int channel_major = 0;           // which logical workgroup order costs fewer L2 fills (see conv_staged.hip)
     double b_ways = 1.0;             // serialisation of the B-operand LDS read by bank conflicts (1 = none)
 };
 
@@ -178,6 +178,9 @@ int kernel_vgprs(const KernelId &k);
 int kernel_waves_per_simd(const KernelId &k);
 // The function itself (nullptr if not instantiated).
 const void *kernel_function(const KernelId &k);
+// (its two halves, one per translation unit that holds kernels: conv_staged.hip and conv_stream.hip)
+const void *staged_kernel_function(const KernelId &k);
+const void *stream_kernel_function(const KernelId &k);
 inline const void *conv_kernel_for(const tdc_tile &t, int KH, int KW, int dilation, int stride, bool extras) {
     return kernel_function(kernel_id_for(t, KH, KW, dilation, stride, extras));
 }

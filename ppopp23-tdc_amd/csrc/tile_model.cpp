@@ -12,6 +12,8 @@
 #include <algorithm>
 #include <array>
 #include <map>
+#include <mutex>
+#include <shared_mutex>
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
@@ -395,6 +397,7 @@ struct ModelConst {
     double stream_latency_clk = 645;    // alg 3: round trip of the first request, global memory -> registers
 };
 ModelConst MC;
+std::shared_mutex MC_mutex;   // readers: every model evaluation; writer: tdc_model_set_constants
 constexpr int kNumModelConst = 18;
 
 double *mc_field(int i) {
@@ -425,7 +428,7 @@ double *mc_field(int i) {
 
 struct CompiledKernel { const char *name; int regs, sgprs, waves; };
 // hipcc's resource report for the convolution kernels of this build (written by the Makefile from the compile of
-// conv_mfma.hip): name, VGPRs + AGPRs per lane, scalar registers, waves per SIMD.
+// conv_staged.hip and conv_stream.hip): name, VGPRs + AGPRs per lane, scalar registers, waves per SIMD.
 static const CompiledKernel compiled_kernels[] = {
 #include "kernel_registers.inc"
 };
@@ -551,6 +554,7 @@ bool model_evaluate(const tdc_conv_desc &d, const tdc_tile &t, tdc_tile_info &in
     Geometry g;
     if (!make_geometry(d, t, g, why, tail_N)) return false;
     const Machine &m = machine();
+    std::shared_lock<std::shared_mutex> constants_lock(MC_mutex);
     std::memset(&info, 0, sizeof(info));
     info.tile = t;
     info.grid_x = g.grid_x;
@@ -896,6 +900,7 @@ std::vector<tdc_tile> model_enumerate(const tdc_conv_desc &d, int tail_N) {
 }
 
 int model_constants(double *out, int cap) {
+    std::shared_lock<std::shared_mutex> lock(MC_mutex);
     for (int i = 0; i < kNumModelConst && i < cap; ++i) out[i] = *mc_field(i);
     return kNumModelConst;
 }
@@ -904,6 +909,7 @@ bool model_set_constants(const double *in, int n) {
     if (n != kNumModelConst) return false;
     for (int i = 0; i < n; ++i)
         if (!(in[i] > 0.0)) return false;
+    std::unique_lock<std::shared_mutex> lock(MC_mutex);
     for (int i = 0; i < n; ++i) *mc_field(i) = in[i];
     return true;
 }
