@@ -8,6 +8,7 @@ geometry (grid, workgroup, LDS) is what tells the layers apart.
     python -m tdc_amd.profsum pmc    <dir-with-*_counter_collection.csv> [--copy-bytes N]
     python -m tdc_amd.profsum timeline <dir-with-*_kernel_trace.csv> --last N
     python -m tdc_amd.profsum isolated <dir-with-*_kernel_trace.csv> --layers <output of bench.py --isolated-layers>
+    python -m tdc_amd.profsum isolated-pmc <dir,dir,...> --layers <output of bench.py --isolated-layers> [--copy-bytes N]
 
 ``kernel``: count / mean / min / max duration in microseconds per (kernel, grid, workgroup, LDS).
 ``pmc``: mean counter value per (kernel, grid, workgroup); with ``--copy-bytes N`` the FETCH_SIZE /
@@ -16,6 +17,7 @@ copy kernel in the same run, which is known to read and write N bytes.
 ``timeline``: the last N dispatches of the trace in launch order (one forward of a network of N kernels):
 start offset, duration, and the idle gap since the previous kernel ended.
 ``isolated``: median / p10 kernel duration per benchmark layer from a trace of ``bench.py --isolated-layers``.
+``isolated-pmc``: counters per benchmark layer from ``--pmc`` runs of the same command (one directory per counter set).
 """
 from __future__ import annotations
 
@@ -139,15 +141,87 @@ def isolated(path, layers_json, out=sys.stdout):
             r1, r2, hw, ",".join(str(v) for v in tile), d[len(d) // 2], d[len(d) // 10], names.pop(), len(d), d[0], d[-1]))
 
 
+def isolated_pmc(paths, layers_json, copy_bytes=None, out=sys.stdout):
+    """Counters per benchmark layer from ``rocprofv3 --pmc`` runs of ``bench.py --isolated-layers`` (one run per counter
+    set; `paths` = their output directories): the last (layers x launches) convolution dispatches of each run, in
+    dispatch order, against the layer list the run printed; mean over the launches of a layer.  FETCH_SIZE and
+    WRITE_SIZE are scaled by what the run's calibration copy of `copy_bytes` bytes reads."""
+    import json
+    info = None
+    for line in open(layers_json):
+        line = line.strip()
+        if line.startswith("{") and "isolated_layers" in line:
+            info = json.loads(line)
+    if info is None:
+        raise SystemExit(f"no --isolated-layers result line in {layers_json}")
+    per = info["launches_per_layer"]      # (one of them is the layer's parity launch, which comes before all isolated launches)
+    nl = len(info["layers"])
+    means = [dict() for _ in range(nl)]
+    kernels = [None] * nl
+    scale = {}
+    for path in paths:
+        files = sorted(glob.glob(os.path.join(path, "**", "*counter_collection.csv"), recursive=True))
+        if not files:
+            raise SystemExit(f"no *counter_collection.csv under {path}")
+        disp = collections.OrderedDict()
+        copies = collections.defaultdict(float)
+        for f in files:
+            for r in csv.DictReader(open(f)):
+                name = _short(r["Kernel_Name"])
+                if "tdc_conv" in name:
+                    disp.setdefault(int(r["Dispatch_Id"]), (name, {}))[1][r["Counter_Name"]] = float(r["Counter_Value"])
+                elif "copy" in name.lower() and r["Counter_Name"] in ("FETCH_SIZE", "WRITE_SIZE"):
+                    copies[r["Counter_Name"]] = max(copies[r["Counter_Name"]], float(r["Counter_Value"]))
+        if copy_bytes:
+            for cname, best in copies.items():
+                if best > 0:
+                    scale[cname] = copy_bytes / (best * 1024.0)
+        ids = sorted(disp)
+        # every layer: one parity launch (all of them first), then `per - 1` isolated launches, layer after layer
+        need = (per - 1) * nl
+        if len(ids) < need:
+            raise SystemExit(f"{path}: {len(ids)} convolution dispatches, expected at least {need}")
+        ids = ids[-need:]
+        for i in range(nl):
+            chunk = [disp[d] for d in ids[i * (per - 1):(i + 1) * (per - 1)]]
+            names = {c[0] for c in chunk}
+            if len(names) != 1:
+                raise SystemExit(f"{path}: layer {i}: the dispatches do not line up with the layer list ({names})")
+            kernels[i] = names.pop()
+            for cname in chunk[0][1]:
+                means[i][cname] = sum(c[1][cname] for c in chunk) / len(chunk)
+    for cname, sc in sorted(scale.items()):
+        out.write("# %s: 1 counted KiB = %.4f KiB moved (from the calibration copy of %d bytes)\n" % (cname, sc, copy_bytes))
+    out.write("# per layer: R1 R2 H=W tile | kernel | waves, MFMA instructions, MFMA-busy cycles per SIMD (1024 SIMDs), share of wave "
+              "cycles waiting on any instruction, LDS bank-conflict share of LDS-active cycles | L2 read bytes (sectors x 32) "
+              "and their ratio to the algorithmic bytes, L2 hit rate | HBM traffic (FETCH_SIZE + WRITE_SIZE, scaled) and its ratio\n")
+    for i, (r1, r2, hw, tile) in enumerate(info["layers"]):
+        m = means[i]
+        alg = 4.0 * (r1 * hw * hw + r2 * hw * hw + 9 * r1 * r2)
+        g = lambda k: m.get(k, float("nan"))
+        l2 = g("TCC_READ_SECTORS_sum") * 32.0
+        hbm = g("FETCH_SIZE") * 1024.0 * scale.get("FETCH_SIZE", 1.0) + g("WRITE_SIZE") * 1024.0 * scale.get("WRITE_SIZE", 1.0)
+        out.write("layer_counters: %d %d %d %s | %s | waves %d mfma %d busy/simd %.0f wait %.0f%% lds_conflict %.0f%% | "
+                  "l2_read %.2f MB x%.1f hit %.0f%% | hbm %.2f MB x%.2f\n" % (
+                      r1, r2, hw, ",".join(str(v) for v in tile), kernels[i], g("SQ_WAVES"), g("SQ_INSTS_MFMA"),
+                      g("SQ_VALU_MFMA_BUSY_CYCLES") / 1024.0, 100.0 * g("SQ_WAIT_INST_ANY") / max(g("SQ_WAVE_CYCLES"), 1.0),
+                      100.0 * g("SQ_LDS_BANK_CONFLICT") / max(g("SQ_LDS_IDX_ACTIVE"), 1.0) if g("SQ_LDS_IDX_ACTIVE") > 0 else 0.0,
+                      l2 * 1e-6, l2 / alg, 100.0 * g("TCC_HIT_sum") / max(g("TCC_REQ_sum"), 1.0), hbm * 1e-6, hbm / alg))
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser()
-    ap.add_argument("mode", choices=["kernel", "pmc", "timeline", "isolated"])
+    ap.add_argument("mode", choices=["kernel", "pmc", "timeline", "isolated", "isolated-pmc"])
     ap.add_argument("path")
     ap.add_argument("--copy-bytes", type=int, default=None)
     ap.add_argument("--layers", default=None, help="isolated: file holding the JSON line bench.py --isolated-layers printed")
     ap.add_argument("--last", type=int, default=64, help="timeline: how many dispatches from the end of the trace")
     a = ap.parse_args(argv)
-    if a.mode == "isolated":
+    if a.mode == "isolated-pmc":
+        if not a.layers:
+            raise SystemExit("isolated-pmc: --layers <file with the output of bench.py --isolated-layers> is required")
+        isolated_pmc(a.path.split(","), a.layers, a.copy_bytes)
+    elif a.mode == "isolated":
         if not a.layers:
             raise SystemExit("isolated: --layers <file with the output of bench.py --isolated-layers> is required")
         isolated(a.path, a.layers)
