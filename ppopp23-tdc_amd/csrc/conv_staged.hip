@@ -114,7 +114,7 @@ __device__ __forceinline__ void issue_inputs(const ConvKParams &p, __amdgpu_buff
                                              int iy0, int ix0a, int dw, int dn, int lane) {
     const int VW = p.VW;
     const int blk_floats = 64 * VW;
-    const int nblk = p.in_stage_floats / blk_floats;
+    const int nblk = p.in_nblk;
     // This pass starts chunk*CCH channels further on.  The shift goes through the vector offset on
     // purpose: only that one is range-checked, and channels past C must read as zero.
     const int pass_bytes = chunk * p.CCH * p.H * p.W * 4;
@@ -217,7 +217,7 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
     // waves the first pass is dealt differently and computes its offsets on the fly, so the table is only
     // filled afterwards, by the loaders, while the first copies are in flight.
     int pre[MAXPRE];
-    const int in_nblk = p.in_stage_floats / (64 * p.VW);
+    const int in_nblk = p.in_nblk;
     auto fill_pre = [&]() {
 #pragma unroll
         for (int i = 0; i < MAXPRE; ++i) {

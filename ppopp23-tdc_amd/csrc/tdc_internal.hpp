@@ -127,6 +127,7 @@ struct ConvKParams {
     FastDiv fd_g1, fd_g2;      // the fastest / second extent of the logical order
     int RS, CS, VW, nrows;
     int in_stage_floats, wslab_floats, stage_floats, nstage;
+    int in_nblk;                     // in_stage_floats / (64 * VW): copy blocks of the input window per pass
     int relu;
     int in_relu;               // ReLU after the input affine
     int tail_N, tail_mblk, tail_ng, tail_relu;   // tail outputs, their 16-row blocks, K-steps (ceil(N/4)), ReLU after it
