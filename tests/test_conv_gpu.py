@@ -321,6 +321,44 @@ def test_seven_by_seven_instantiations(C, stride):
     assert_close(run_conv(x, w, stride=stride, pad=6, dil=2, tile=t), want, f"7x7 dilated C{C} s{stride}")
 
 
+def _epilogue_tiles(d):
+    """One tile of every kernel family the enumeration offers for `d` (staged direct with one and several register
+    blocks, Winograd, global weights, streamed with 1 / 2 / 4 row blocks, and the variants split across workgroups)."""
+    seen, out = set(), []
+    for t in tdc_amd.model_enumerate(d):
+        key = (t.alg, t.mf, t.mb, t.nb, t.wk > 1, t.ks > 1)
+        if key not in seen:
+            seen.add(key)
+            out.append(t)
+    return out
+
+
+@pytest.mark.parametrize("shape,K", [((2, 24, 40, 10, 30), 3), ((1, 64, 48, 9, 56), 3), ((2, 96, 40, 6, 7), 1), ((1, 16, 20, 11, 13), 5)])
+def test_epilogue_on_every_kernel_family(shape, K):
+    """+ bias, + residual, ReLU on one tile of every kernel family: against the oracle, with the residual in its own
+    buffer and IN PLACE (the residual buffer is the output buffer), where every lane must have read its residual
+    values before it stores."""
+    B, C, N, H, W = shape
+    x, w = case(8800 + C + N, B, C, N, H, W, K)
+    g = seeded(8801 + H)
+    bias = torch.randn(N, generator=g)
+    resid = torch.randn(B, N, H, W, generator=g)
+    want = ref.conv2d_c(x.numpy(), w.numpy(), bias.numpy(), resid.numpy(), pad=K // 2, relu=True)
+    d = tdc_amd.conv_desc(B, C, N, H, W, K, K, 1, K // 2)
+    tiles = _epilogue_tiles(d)
+    assert len({t.alg for t in tiles}) >= (2 if K in (1, 3) else 1)
+    xd = x.cuda()
+    for t in tiles:
+        announce("epilogue", shape, K, t)
+        assert_close(run_conv(x, w, bias, resid, pad=K // 2, relu=True, tile=t), want, f"epilogue {shape} {t}")
+        plan = tdc_amd.Conv2dPlan(B, C, N, H, W, K, K, 1, K // 2, 1, True, True, tile=t).set_weights(w, bias)
+        buf = resid.cuda().clone()
+        plan.forward(xd, buf, out=buf)
+        torch.cuda.synchronize()
+        plan.close()
+        assert_close(buf.cpu().numpy(), want, f"in-place epilogue {shape} {t}")
+
+
 def test_random_shapes_model_tile():
     """Forty seeded random problems (ragged sizes, batch, stride, padding, dilation, rectangular images, every
     epilogue combination) with the tile the model picks, against F.conv2d on the host."""
