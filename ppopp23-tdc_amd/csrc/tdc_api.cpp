@@ -624,7 +624,7 @@ static int forward_impl(tdc_conv_plan *plan, const float *d_in, int64_t in_batch
     const bool aligned = reinterpret_cast<uintptr_t>(d_in) % 16 == 0 && kp.in_bstride % 4 == 0;
     kp.VW = (g.VW == 4 && aligned) ? 4 : 1;
     kp.in_stage_floats = g.in_stage_floats; kp.wslab_floats = g.wslab_floats;
-    kp.in_nblk = g.in_stage_floats / (64 * std::max(g.VW, 1));
+    kp.in_nblk = g.in_stage_floats / (64 * kp.VW);   // (kp.VW: the element width this launch really copies with)
     kp.stage_floats = g.stage_floats; kp.nstage = g.nstage;
     kp.relu = d.relu;
     kp.fd_csv = make_fastdiv(g.CS / kp.VW);

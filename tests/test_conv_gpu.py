@@ -359,6 +359,30 @@ def test_epilogue_on_every_kernel_family(shape, K):
         assert_close(buf.cpu().numpy(), want, f"in-place epilogue {shape} {t}")
 
 
+@pytest.mark.parametrize("shape,K", [((1, 24, 32, 12, 16), 3), ((2, 40, 20, 8, 28), 3), ((1, 48, 16, 6, 8), 1), ((1, 12, 16, 9, 12), 5)])
+def test_input_not_aligned_to_16_bytes(shape, K):
+    """Image rows that are a multiple of four floats are staged with 16-byte copy elements; an input pointer that is
+    only 4-byte aligned (a view one float into its buffer) makes the launch fall back to 4-byte elements, four times
+    as many copy blocks.  One tile of every kernel family, input and output both one float off."""
+    B, C, N, H, W = shape
+    x, w = case(8900 + C + N, B, C, N, H, W, K)
+    want = ref.conv2d_c(x.numpy(), w.numpy(), pad=K // 2)
+    d = tdc_amd.conv_desc(B, C, N, H, W, K, K, 1, K // 2)
+    xbuf = torch.zeros(x.numel() + 1, device="cuda")
+    xv = xbuf[1:].view(B, C, H, W)
+    xv.copy_(x)
+    assert xv.data_ptr() % 16 == 4
+    for t in _epilogue_tiles(d):
+        announce("unaligned input", shape, K, t)
+        plan = tdc_amd.Conv2dPlan(B, C, N, H, W, K, K, 1, K // 2, tile=t).set_weights(w)
+        obuf = torch.full((B * N * H * W + 1,), float("nan"), device="cuda")
+        ov = obuf[1:].view(B, N, H, W)
+        plan.forward(xv, out=ov)
+        torch.cuda.synchronize()
+        plan.close()
+        assert_close(ov.cpu().numpy(), want, f"unaligned input {shape} {t}")
+
+
 def test_random_shapes_model_tile():
     """Forty seeded random problems (ragged sizes, batch, stride, padding, dilation, rectangular images, every
     epilogue combination) with the tile the model picks, against F.conv2d on the host."""
