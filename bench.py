@@ -56,6 +56,17 @@ REFERENCE_LAYERS = (
 )
 
 
+def cpu_model():
+    """The host processor's name as /proc/cpuinfo gives it (reported beside the CPU baseline)."""
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 def kernel_only_durations():
     """{(R1, R2, H): (median us, p10 us, tile)} of isolated launches from the committed rocprofv3 kernel-trace summary
     (lines `kernel_only_us: R1 R2 H tile median p10`)."""
@@ -447,7 +458,7 @@ def main():
                 passes += 1
             cpu_s = time.perf_counter() - t0
         out["cpu_baseline"] = {"value": round(cpu_s * 1e6 / (passes * len(layers)), 2), "unit": "us/layer",
-                               "cores": torch.get_num_threads(), "kind": "port",
+                               "cores": torch.get_num_threads(), "cpu_model": cpu_model(), "kind": "port",
                                "sample": "%d passes over the same 28 layers with torch.nn.functional.conv2d fp32 on "
                                          "the host (the call the reference operator makes on CPU), ~10 s" % passes}
         if e2e_params is not None:
