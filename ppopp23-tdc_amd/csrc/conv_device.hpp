@@ -85,6 +85,34 @@ struct Mfma<16> {
 
 constexpr int OOB_OFFSET = 0x7ffffff0;  // beyond any buffer: the load returns zero
 
+// Output stores.  TDC_STORE_WT (experiment builds): written through the die's L2 at once (device-scope store) instead
+// of staying dirty there until the kernel ends.
+#ifndef TDC_STORE_WT
+#define TDC_STORE_WT 0
+#endif
+__device__ __forceinline__ void store_out(float *p, float v) {
+#if TDC_STORE_WT
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#else
+    *p = v;
+#endif
+}
+__device__ __forceinline__ void store_out(float *p, f4_t v) {
+#if TDC_STORE_WT
+    asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
+#else
+    *reinterpret_cast<f4_t *>(p) = v;
+#endif
+}
+typedef float f2_store_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void store_out(float *p, f2_store_t v) {
+#if TDC_STORE_WT
+    asm volatile("global_store_dwordx2 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
+#else
+    *reinterpret_cast<f2_store_t *>(p) = v;
+#endif
+}
+
 __device__ __forceinline__ int fdiv(int n, const FastDiv &f) {
     return (int)(__umulhi((unsigned)n, f.m) + ((unsigned)n & f.pass));
 }
@@ -110,7 +138,7 @@ __device__ __forceinline__ void finish_four_channels(const f4_t &acc, int ch0, i
         float val = acc[i] + bv[i];
         val += rv[i];
         if (relu) val = fmaxf(val, 0.0f);
-        out[(long long)(ch0 + i) * P + pix] = val;
+        store_out(out + ((long long)(ch0 + i) * P + pix), val);
     }
 }
 

@@ -853,7 +853,7 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
         val += bv;
         val += rv;
         if (p.relu) val = fmaxf(val, 0.0f);
-        out[(long long)n * p.P + pp] = val;
+        store_out(out + ((long long)n * p.P + pp), val);
     };
     if constexpr (EXT) if (p.tail_w) {
         // Fused tail: a 1x1 convolution over the output channels of this one, out2 = W2 * act(conv + bias), in the
@@ -949,7 +949,7 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
                         float val = acc2[v] + tbv[v];
                         val += trv[v];
                         if (p.tail_relu) val = fmaxf(val, 0.0f);
-                        out[(long long)n2 * p.P + pp] = val;
+                        store_out(out + ((long long)n2 * p.P + pp), val);
                     }
                 }
             }
@@ -990,7 +990,7 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
 #pragma unroll
                             for (int e = 0; e < V; ++e) val[e] = fmaxf(val[e], 0.0f);
                         }
-                        *reinterpret_cast<vec_t *>(out + o) = val;
+                        store_out(out + o, val);
                     }
                 }
             };

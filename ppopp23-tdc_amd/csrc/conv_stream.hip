@@ -439,7 +439,7 @@ __global__ void __launch_bounds__(1024) tdc_conv3x3_stream_kernel(const ConvKPar
                         float val = acc2[v] + tbv[v];
                         val += trv[v];
                         if (p.tail_relu) val = fmaxf(val, 0.0f);
-                        out[(long long)n2 * p.P + pp] = val;
+                        store_out(out + ((long long)n2 * p.P + pp), val);
                     }
                 }
             }
@@ -598,7 +598,7 @@ __global__ void __launch_bounds__(1024) tdc_conv3x3_stream_rownb_kernel(const Co
             val += bv;
             val += rv;
             if (p.relu) val = fmaxf(val, 0.0f);
-            out[o] = val;
+            store_out(out + o, val);
         }
     }
     TDC_STAMP(6);   // stores issued
