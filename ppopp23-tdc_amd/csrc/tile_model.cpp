@@ -378,23 +378,23 @@ namespace {
 // (2080Ti-evaluation/TDC-LAYERS-MODELING/model.py:265-266,278).
 struct ModelConst {
     double launch_us = 1.474;           // device time of an empty kernel in a back-to-back stream
-    double setup_clk = 1740;          // kernel arguments and index arithmetic before the first copy is issued
-    double copy_latency_clk = 665.1;   // first byte of a global->LDS copy (L2 / memory-side cache)
-    double copy_bytes_per_clk = 41.18;   // sustained global->LDS rate of one CU
-    double l2_bytes_per_clk = 8347;   // whole-chip L2->CU rate when every CU copies at once
-    double lds_bytes_per_clk = 22.86;   // LDS traffic of the split-K reduction
+    double setup_clk = 1479;          // kernel arguments and index arithmetic before the first copy is issued
+    double copy_latency_clk = 798.12;   // first byte of a global->LDS copy (L2 / memory-side cache)
+    double copy_bytes_per_clk = 42.0036;   // sustained global->LDS rate of one CU
+    double l2_bytes_per_clk = 12019.7;   // whole-chip L2->CU rate when every CU copies at once
+    double lds_bytes_per_clk = 41.148;   // LDS traffic of the split-K reduction
     double sync_clk = 275.2;            // one workgroup barrier
     double store_bytes_per_clk = 2.827;  // per CU, short runs per channel
-    double kstep_issue_clk = 6.044;      // vector-ALU / LDS-issue cycles per operand read, not hidden under MFMAs
-    double pass_overhead_clk = 491.9;   // per wave and pass: copy issue, pointer set-up, pipeline fill
-    double wave_setup_clk = 540.5;      // prologue cycles added per extra wave sharing a SIMD
-    double ksplit_clk = 4604;         // split across workgroups: write-through, ticket round trip, read-back
+    double kstep_issue_clk = 4.36679;      // vector-ALU / LDS-issue cycles per operand read, not hidden under MFMAs
+    double pass_overhead_clk = 371.876;   // per wave and pass: copy issue, pointer set-up, pipeline fill
+    double wave_setup_clk = 778.32;      // prologue cycles added per extra wave sharing a SIMD
+    double ksplit_clk = 3381.18;         // split across workgroups: write-through, ticket round trip, read-back
     double copy_issue_clk = 100.5;      // a wave is held this long by every global->LDS copy instruction it issues
-    double lds_read_clk = 2.88;        // LDS busy cycles per conflict-free operand read of one wave
-    double wino_kstep_clk = 13.99;      // Winograd: cycles per MFMA that the input transform adds on top of the operand reads
-    double gw_latency_clk = 1457;       // alg 2: the first weights come from L2 into registers after the input copy is under way
-    double stream_setup_clk = 250;      // alg 3: index arithmetic before the requests go out (no copy tables, no stages)
-    double stream_latency_clk = 645;    // alg 3: round trip of the first request, global memory -> registers
+    double lds_read_clk = 1.44;        // LDS busy cycles per conflict-free operand read of one wave
+    double wino_kstep_clk = 16.788;      // Winograd: cycles per MFMA that the input transform adds on top of the operand reads
+    double gw_latency_clk = 1040.3;       // alg 2: the first weights come from L2 into registers after the input copy is under way
+    double stream_setup_clk = 459;      // alg 3: index arithmetic before the requests go out (no copy tables, no stages)
+    double stream_latency_clk = 774;    // alg 3: round trip of the first request, global memory -> registers
 };
 ModelConst MC;
 std::shared_mutex MC_mutex;   // readers: every model evaluation; writer: tdc_model_set_constants
@@ -636,10 +636,16 @@ bool model_evaluate(const tdc_conv_desc &d, const tdc_tile &t, tdc_tile_info &in
             const double groups = (double)t.cch / (4.0 * t.wk);
             const double waves_simd = std::ceil((double)g.waves * r / m.simds_per_cu);
             // a wave issues its requests one after the other (about 21 cycles each): fewer groups per wave start sooner
-            double clk = MC.stream_setup_clk + MC.stream_latency_clk + 288.0 + 65.0 * (waves_simd - 1.0) + bytes / rate +
+            // (288 cycles per group: a wave's own nine MFMAs per block run one after the other)
+            double clk = MC.stream_setup_clk + MC.stream_latency_clk + 288.0 * groups + 65.0 * (waves_simd - 1.0) + bytes / rate +
                          groups * (3.0 + t.nb * (row_mode ? 3.0 : 9.0)) * 21.4;
             // the MFMAs of the extra blocks no longer hide under the requests: the matrix pipe of a SIMD serves its waves in turn
-            if (t.nb > 1) clk += waves_simd * groups * 9.0 * (t.nb - 1) * mfma_clk;
+            if (t.nb > 1) {
+                clk += waves_simd * groups * 9.0 * (t.nb - 1) * mfma_clk;
+                // all threads share the final sum and store; a workgroup of few waves walks its blocks in several rounds
+                const double rounds = std::ceil((double)t.wm * t.nb * 256.0 / g.threads);
+                clk += (rounds - 1.0) * (110.0 + 8.0 * t.wk);
+            }
             if (t.wk > 1) clk += 1.6 * MC.sync_clk;
             if (tail_N > 0) {
                 // park the columns, a barrier, the first touch of the tail's weights, its blocks dealt over the waves
