@@ -94,6 +94,7 @@ def main():
                     help="profiling aid: launch only the dominant layer (128->128 @56), `steps` times, and exit")
     ap.add_argument("--only-e2e", action="store_true",
                     help="profiling aid: run only the end-to-end Tucker ResNet-18 forward, `steps` times, and exit")
+    ap.add_argument("--e2e-batch", type=int, default=1, help="with --only-e2e: images per forward")
     ap.add_argument("--e2e-net", choices=["resnet18", "densenet121"], default="resnet18",
                     help="which Tucker network --only-e2e runs (batch 1)")
     ap.add_argument("--only-conv", default=None, metavar="C,N,H,K[,stride]",
@@ -139,11 +140,11 @@ def main():
     if a.only_e2e:
         from tdc_amd import nets
         if a.e2e_net == "densenet121":
-            net = nets.build_tucker_densenet121(nets.densenet121_params(seed=121), batch=1)
+            net = nets.build_tucker_densenet121(nets.densenet121_params(seed=121), batch=a.e2e_batch)
         else:
-            net = nets.build_tucker_resnet18(nets.resnet18_params(seed=18), batch=1)
+            net = nets.build_tucker_resnet18(nets.resnet18_params(seed=18), batch=a.e2e_batch)
         ms = net.time_ms(iters=a.steps, graph=graph)
-        print(json.dumps({"only_e2e": True, "net": a.e2e_net, "forwards": a.steps, "ms": ms,
+        print(json.dumps({"only_e2e": True, "net": a.e2e_net, "batch": a.e2e_batch, "forwards": a.steps, "ms": ms,
                           "kernels": net.num_kernels}))
         return
 
