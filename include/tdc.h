@@ -99,7 +99,14 @@ typedef struct tdc_tile {
                          the input channels in groups of four; cch = 4 * wk * {1, 2, 4}, ceil(C / cch) = ks.  With stride 1 and
                          tw = 14 the three taps of a filter row are lane shifts of one request.  Carries a fused 1x1
                          tail when wm covers every output channel (and ks = 1).
-                     The model offers 3 and 4 where launch and latency dominate (few channels or few pixels); the
+                     5 = Winograd F(2x2,3x3) with BOTH operands read from global memory straight into registers
+                         (3x3 / stride 1 / pad 1 / dilation 1, even image width): a workgroup owns 16 * wm channels of
+                         one tile-row block (2 output rows x 28 columns, tw = 28), its wk waves split the input
+                         channels in groups of four, cch = 4 * wk * {1, 2, 3, 4} >= C (one pass; at most 16 / 16 / 16 / 12
+                         waves per workgroup); the input rows are loaded as column pairs, once per lane, and the
+                         patch columns a tile shares with its neighbours are lane shifts; mf = 16, mb = nb = wn = 1,
+                         ks = 1, wl = 0.  No fused tail.
+                     The model offers 3, 4 and 5 where launch and latency dominate (few channels or few pixels); the
                      staged paths keep the layers whose operands are worth sharing through the LDS. */
 } tdc_tile;
 

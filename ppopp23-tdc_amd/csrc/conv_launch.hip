@@ -8,10 +8,12 @@
 
 namespace tdc {
 
-// The kernels live in two translation units (conv_staged.hip, conv_stream.hip); each maps the KernelIds of its
-// family to its instantiations.
+// The kernels live in three translation units (conv_staged.hip, conv_stream.hip, conv_wino_stream.hip); each maps the
+// KernelIds of its families to its instantiations.
 const void *kernel_function(const KernelId &k) {
-    return k.family == KernelId::STAGED ? staged_kernel_function(k) : stream_kernel_function(k);
+    return k.family == KernelId::STAGED        ? staged_kernel_function(k)
+           : k.family == KernelId::STREAM_WINO ? wino_stream_kernel_function(k)
+                                               : stream_kernel_function(k);
 }
 
 // ---------------------------------------------------------------------------

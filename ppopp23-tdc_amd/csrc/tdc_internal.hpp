@@ -80,7 +80,7 @@ bool model_set_constants(const double *in, int n);
 // in MFMA A-operand order: lane l of an entry holds
 // w[tile*MT + mblk*mf + l%mf][pass*cch + cg*kc + l/mf][tap], zero outside N x C.
 // tile.alg = 2 regroups the nine taps of a channel group as [taps 0-3][lane][4] [taps 4-7][lane][4] [tap 8][lane];
-// tile.alg = 1 stores the 16 Winograd-domain values U = G g G^T of every (n, c) as [quarter][lane][4].
+// tile.alg = 1 and 5 store the 16 Winograd-domain values U = G g G^T of every (n, c) as [quarter][lane][4].
 size_t packed_weight_floats(const Geometry &g);
 void pack_weights(const tdc_conv_desc &d, const tdc_tile &t, const Geometry &g, const float *w_oihw, float *packed);
 
@@ -161,14 +161,17 @@ enum : int { TAPS_GENERIC = 0, TAPS_1x1 = 1, TAPS_3x3 = 9, TAPS_3x3G = 10, TAPS_
 //   STREAM_1x1  tdc_conv1x1_stream_kernel<NQ, AFF, MODE>              p = {NQ, AFF, MODE}
 //   STREAM_3x3  tdc_conv3x3_stream_kernel<CG, ROW, MODE>              p = {CG, ROW, MODE, 1}
 //               tdc_conv3x3_stream_rownb_kernel<CG, NB>               p = {CG, 1, 0, NB}   (NB = 2 or 4 pixel blocks per wave)
+//   STREAM_WINO tdc_wino3x3_stream_kernel<CG, MAXW>                   p = {CG, MAXW}
 struct KernelId {
-    enum Family : int { NONE = 0, STAGED = 1, STREAM_1x1 = 2, STREAM_3x3 = 3 };
+    enum Family : int { NONE = 0, STAGED = 1, STREAM_1x1 = 2, STREAM_3x3 = 3, STREAM_WINO = 4 };
     int family = NONE;
     int p[6] = {0, 0, 0, 0, 0, 0};
 };
 // `extras`: the instantiation that also carries the input affine and the fused 1x1 tail.  family == NONE: no kernel.
 KernelId kernel_id_for(const tdc_tile &t, int KH, int KW, int dilation, int stride, bool extras);
-KernelId kernel_id_with_head(const tdc_tile &t);   // streamed 3x3 with fused 1x1 head and tail
+KernelId kernel_id_with_head(const tdc_tile &t);
+// Streamed Winograd kernel (tile.alg = 5): waves per workgroup it is built for, by groups of four channels per wave (0 = none).
+int wino_stream_max_waves(int groups);   // streamed 3x3 with fused 1x1 head and tail
 // The kernel's name as the compiler's resource report and the profiler print it, e.g.
 // "tdc_conv_mfma_kernel<16, 1, 1, 9, 16, false>".
 std::string kernel_name(const KernelId &k);
@@ -179,9 +182,10 @@ int kernel_vgprs(const KernelId &k);
 int kernel_waves_per_simd(const KernelId &k);
 // The function itself (nullptr if not instantiated).
 const void *kernel_function(const KernelId &k);
-// (its two halves, one per translation unit that holds kernels: conv_staged.hip and conv_stream.hip)
+// (its parts, one per translation unit that holds kernels: conv_staged.hip, conv_stream.hip, conv_wino_stream.hip)
 const void *staged_kernel_function(const KernelId &k);
 const void *stream_kernel_function(const KernelId &k);
+const void *wino_stream_kernel_function(const KernelId &k);
 inline const void *conv_kernel_for(const tdc_tile &t, int KH, int KW, int dilation, int stride, bool extras) {
     return kernel_function(kernel_id_for(t, KH, KW, dilation, stride, extras));
 }

@@ -120,6 +120,12 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
     g = Geometry();
     // (256 registers per lane for the 2x2 block grid, 168 for the Winograd path)
     g.max_waves_kernel = (t.mb == 2 && t.nb == 2) ? 8 : t.alg == 1 ? 12 : 16;
+    if (t.alg == 5) {
+        // streamed Winograd: the launch bound follows the groups of four channels a wave keeps in registers
+        const int groups = (t.wk >= 1 && t.cch % (4 * t.wk) == 0) ? t.cch / (4 * t.wk) : 0;
+        g.max_waves_kernel = wino_stream_max_waves(groups);
+        if (!g.max_waves_kernel) return fail("tile.alg = 5 needs cch = 4 * wk * {1, 2, 3, 4}");
+    }
     if (t.wl < 0 || t.wl > 8) return fail("tile.wl must be in [0, 8]");
     if ((long long)t.wm * t.wn * t.wk + t.wl > g.max_waves_kernel) return fail("too many waves per workgroup for this tile");
     g.waves = t.wm * t.wn * t.wk + t.wl;
@@ -136,7 +142,20 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
     g.taps = d.KH * d.KW;
     g.ktaps = g.taps;
     g.MT = t.mf * t.mb * t.wm;
-    if (t.alg < 0 || t.alg > 4) return fail("tile.alg must be in [0, 4]");
+    if (t.alg < 0 || t.alg > 5) return fail("tile.alg must be in [0, 5]");
+    if (t.alg == 5) {
+        // Winograd F(2x2,3x3) streamed from global memory: 16*wm channels of one tile row block (2 rows x 28 columns) per
+        // workgroup, the input channels split over wk waves in groups of four, everything in one pass
+        if (d.KH != 3 || d.KW != 3 || d.stride != 1 || d.dilation != 1 || d.pad != 1)
+            return fail("tile.alg = 5 needs a 3x3 / stride 1 / pad 1 / dilation 1 convolution");
+        if (d.W % 2 != 0) return fail("tile.alg = 5 needs an even image width");
+        if (t.mf != 16 || t.mb != 1 || t.nb != 1 || t.wn != 1) return fail("tile.alg = 5 needs mf = 16, mb = nb = wn = 1");
+        if (t.wl != 0 || t.ks != 1) return fail("tile.alg = 5 has no loader waves and no split across workgroups");
+        if (tail_N > 0) return fail("tile.alg = 5 cannot carry a fused tail");
+        if (t.tw != 28) return fail("tile.alg = 5 needs tw = 28");
+        if (t.cch < d.C || t.cch - d.C >= t.cch / t.wk) return fail("tile.alg = 5 takes all input channels in one pass without an idle wave");
+        if ((long long)t.cch * d.H * d.W * 4 >= (1LL << 31)) return fail("image too large for tile.alg = 5");
+    }
     if (t.alg == 4) {
         // 3x3 convolution streamed from global memory: 16 channels x 16 pixels per workgroup, the input channels
         // split over wk waves in groups of four, everything in one pass
@@ -192,6 +211,11 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
         g.TW = 2 * g.TWt;
         g.TH = 2 * g.THt;
         g.PT = 4 * lanes;   // pixels the workgroup's lanes stand for
+    } else if (t.alg == 5) {
+        g.ktaps = 16;
+        g.TW = 28;
+        g.TH = 2;
+        g.PT = 64;          // two rows of 32 columns in the parked tile (28 of them real)
     } else {
         g.PT = t.mf * t.nb * t.wn;
         // (the streamed 1x1 kernel walks the output in runs of 16 consecutive pixels, whatever the image's rows are)
@@ -257,7 +281,7 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
     const long long stage_bytes = (long long)g.nstage * g.stage_floats * 4;
     // (the Winograd path always parks its output tiles in LDS, also without a split over waves)
     // (... and so does the streamed 3x3 kernel with several pixel blocks per wave: all its threads share the final store)
-    const long long red_bytes = (t.wk > 1 || t.alg == 1 || (t.alg == 4 && t.nb > 1)) ? (long long)t.wk * g.MT * g.PT * 4 : 0;
+    const long long red_bytes = (t.wk > 1 || t.alg == 1 || t.alg == 5 || (t.alg == 4 && t.nb > 1)) ? (long long)t.wk * g.MT * g.PT * 4 : 0;
     long long lds = std::max(stage_bytes, red_bytes);
     if (tail_N > 0) {
         // A fused 1x1 tail needs every output channel of the convolution in one workgroup; its tile is parked
@@ -329,7 +353,7 @@ void pack_weights(const tdc_conv_desc &d, const tdc_tile &t, const Geometry &g, 
                     }
         return;
     }
-    if (g.wino) {
+    if (g.wino || t.alg == 5) {
         // Winograd F(2x2,3x3): U = G g G^T per (output channel, input channel), G = [1 0 0; .5 .5 .5; .5 -.5 .5; 0 0 1].
         // Per (channel tile, pass, M block, channel group): [q = 0..3][64 lanes][e = 0..3] holding U[q][e] of
         // (n = l % 16, c = l / 16), so that one 128-bit LDS read fetches the A operands of four of the 16 MFMAs.
@@ -467,8 +491,21 @@ KernelId kernel_id_with_head(const tdc_tile &t) {
     return k;
 }
 
+int wino_stream_max_waves(int groups) { return (groups >= 1 && groups <= 3) ? 16 : groups == 4 ? 12 : 0; }
+
 KernelId kernel_id_for(const tdc_tile &t, int KH, int KW, int dilation, int stride, bool extras) {
     KernelId k;
+    if (t.alg == 5) {
+        if (extras || KH != 3 || KW != 3 || dilation != 1 || stride != 1 || t.mf != 16 || t.mb != 1 || t.nb != 1 || t.wn != 1 ||
+            t.wm < 1 || t.wk < 1 || t.ks != 1 || t.cch % (4 * t.wk) != 0)
+            return k;
+        const int cg = t.cch / (4 * t.wk);
+        const int maxw = wino_stream_max_waves(cg);
+        if (!maxw || t.wm * t.wk > maxw) return k;
+        k.family = KernelId::STREAM_WINO;
+        k.p[0] = cg; k.p[1] = maxw;
+        return k;
+    }
     if (t.alg == 4) {
         // (`extras` can only mean a fused tail here, which the one kernel carries)
         if (KH != 3 || KW != 3 || dilation != 1 || t.mf != 16 || t.mb != 1 || t.wm < 1 || t.wn != 1 || t.wk < 1 ||
@@ -535,6 +572,9 @@ std::string kernel_name(const KernelId &k) {
         case KernelId::STREAM_3x3:
             if (k.p[3] > 1) std::snprintf(buf, sizeof buf, "tdc_conv3x3_stream_rownb_kernel<%d, %d>", k.p[0], k.p[3]);
             else std::snprintf(buf, sizeof buf, "tdc_conv3x3_stream_kernel<%d, %s, %d>", k.p[0], tf[k.p[1] != 0], k.p[2]);
+            break;
+        case KernelId::STREAM_WINO:
+            std::snprintf(buf, sizeof buf, "tdc_wino3x3_stream_kernel<%d, %d>", k.p[0], k.p[1]);
             break;
         default: return "";
     }
@@ -621,6 +661,23 @@ bool model_evaluate(const tdc_conv_desc &d, const tdc_tile &t, tdc_tile_info &in
     const int comp_waves_per_simd = ceil_div(ncomp, m.simds_per_cu);
 
     auto wg_time = [&](int r, long long concurrent_wgs) {
+        if (t.alg == 5) {
+            // like the streamed direct kernel: set-up, one round trip, the bytes at the achieved fill rate, the requests
+            // of a wave one after the other, its own MFMA chain with the transform's vector work, the reduction, the store.
+            // Per input channel and 16 output channels 1 KiB of transformed weights; per input channel four rows of 128 bytes.
+            const double chip_share =
+                MC.l2_bytes_per_clk / std::max<double>(1.0, (double)std::min<long long>(concurrent_wgs, m.cus));
+            const double rate = std::min(0.59 * MC.copy_bytes_per_clk, chip_share);
+            const double bytes = (double)t.cch * (t.wm * 1024.0 + 512.0) * r;
+            const double groups = (double)t.cch / (4.0 * t.wk);
+            const double waves_simd = std::ceil((double)g.waves * r / m.simds_per_cu);
+            double clk = MC.stream_setup_clk + MC.stream_latency_clk + 65.0 * (waves_simd - 1.0) + bytes / rate +
+                         groups * 8.0 * 21.4 + waves_simd * groups * 16.0 * (mfma_clk + MC.wino_kstep_clk);
+            clk += 1.6 * MC.sync_clk + 200.0;   // output transform, park, barrier
+            const double rounds = std::ceil((double)g.MT * 32.0 / g.threads);
+            clk += rounds * (110.0 + 8.0 * t.wk) + out_bytes * r / 200.0;
+            return clk;
+        }
         if (t.alg == 4) {
             // as below; per input channel 576 bytes of weights and nine 64-byte rows of input (the rows of
             // neighbouring taps mostly hit in the L1, so they count for less than their size)
@@ -796,6 +853,23 @@ std::vector<tdc_tile> model_enumerate(const tdc_conv_desc &d, int tail_N) {
                                 out.push_back(t);
                         }
                 }
+            }
+        }
+    }
+    // streamed Winograd candidates: 3x3 / stride 1 / pad 1, even width, all input channels in one pass
+    if (d.KH == 3 && d.KW == 3 && d.stride == 1 && d.dilation == 1 && d.pad == 1 && d.W % 2 == 0 && tail_N == 0 &&
+        !std::getenv("TDC_EXPERIMENT_NO_STREAMED_WINOGRAD")) {
+        const int groups_total = ceil_div(d.C, 4);
+        for (int wm : {1, 2}) {
+            if (16 * wm > round_up(d.N, 16)) continue;
+            for (int per_wave : {4, 3, 2, 1}) {
+                if (per_wave > groups_total) continue;
+                const int wk = ceil_div(groups_total, per_wave);
+                if (wm * wk > wino_stream_max_waves(per_wave)) continue;
+                if (per_wave * wk - groups_total >= per_wave) continue;   // an idle wave
+                tdc_tile t{16, 1, 1, wm, 1, wk, 4 * per_wave * wk, 28, 1, 0, 5};
+                Geometry g;
+                if (make_geometry(d, t, g, nullptr, 0)) out.push_back(t);
             }
         }
     }

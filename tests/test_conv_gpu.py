@@ -218,6 +218,47 @@ def test_every_streamed_3x3_tile(shape, stride, pad):
         assert (got[:, :4] == 7.0).all() and (got[:, 4 + N:] == 7.0).all()
 
 
+@pytest.mark.parametrize("shape", [(1, 16, 16, 7, 8), (2, 13, 20, 9, 12), (1, 64, 32, 28, 28), (1, 40, 24, 13, 30),
+                                   (2, 20, 33, 9, 58), (1, 96, 40, 6, 30), (1, 130, 48, 5, 56), (1, 16, 20, 4, 44),
+                                   (1, 180, 17, 3, 14), (3, 5, 3, 2, 2), (1, 48, 96, 11, 84)])
+def test_every_streamed_winograd_tile(shape):
+    """The Winograd path that streams both operands from global memory into registers (tile.alg = 5): every launchable
+    tile (1 to 4 channel groups per wave, one or two channel blocks per workgroup) on images whose rows have one, two or
+    three 28-column blocks, the last one partial; odd heights (a tile row with one output row), ragged channel counts,
+    batches; plain, and with bias + residual + ReLU written into a channel slice whose addresses are only 4-byte aligned."""
+    from ctypes import c_void_p
+    B, C, N, H, W = shape
+    x, w = case(2700 + C * N + H, B, C, N, H, W, 3)
+    g = seeded(2701)
+    bias = torch.randn(N, generator=g)
+    want = ref.conv2d_c(x.numpy(), w.numpy(), stride=1, pad=1)
+    resid = torch.randn(B, N, H, W, generator=g)
+    want_full = (torch.from_numpy(want) + bias.view(1, -1, 1, 1) + resid).clamp_min(0).numpy()
+    tiles = [t for t in tdc_amd.model_enumerate(tdc_amd.conv_desc(B, C, N, H, W, 3, 3, 1, 1)) if t.alg == 5]
+    assert tiles
+    if C >= 16:
+        assert len({t.cch // (4 * t.wk) for t in tiles}) >= 2
+    for t in tiles:
+        announce("streamed winograd", shape, t)
+        assert_close(run_conv(x, w, pad=1, tile=t), want, f"{shape} {t}")
+        plan = tdc_amd.Conv2dPlan(B, C, N, H, W, 3, 3, 1, 1, 1, True, True, tile=t).set_weights(w, bias)
+        for shift in (0, 1):   # shift 1: the output and residual images start on an odd float
+            xin = torch.zeros(B * (C + 3) * H * W + 1, device="cuda")
+            xv = xin[shift:shift + B * (C + 3) * H * W].view(B, C + 3, H, W); xv[:, 1:1 + C] = x.cuda()
+            rbuf = torch.zeros(B * (N + 2) * H * W + 1, device="cuda")
+            rv = rbuf[shift:shift + B * (N + 2) * H * W].view(B, N + 2, H, W); rv[:, 2:] = resid.cuda()
+            obuf = torch.full((B * (N + 5) * H * W + 1,), 7.0, device="cuda")
+            ov = obuf[shift:shift + B * (N + 5) * H * W].view(B, N + 5, H, W)
+            tdc_amd._lib.check(tdc_amd.lib().tdc_conv_forward_strided(
+                plan._h, c_void_p(xv[:, 1:].data_ptr()), (C + 3) * H * W, c_void_p(rv[:, 2:].data_ptr()), (N + 2) * H * W,
+                c_void_p(ov[:, 4:].data_ptr()), (N + 5) * H * W, c_void_p(torch.cuda.current_stream().cuda_stream)))
+            torch.cuda.synchronize()
+            got = ov.cpu()
+            assert_close(got[:, 4:4 + N].numpy(), want_full, f"slices {shape} {t} shift {shift}")
+            assert (got[:, :4] == 7.0).all() and (got[:, 4 + N:] == 7.0).all()
+        plan.close()
+
+
 @pytest.mark.parametrize("W,c0", [(16, 0), (16, 3), (14, 3), (13, 1)])
 def test_winograd_into_channel_slices(W, c0):
     """A Winograd tile reading from, adding a residual from, and writing into channel slices of wider buffers (the
