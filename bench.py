@@ -13,6 +13,7 @@ events on the launch stream, and the CPU baseline (the PyTorch-CPU convolution
 the reference operator executes) timed on this host's cores.
 """
 import argparse
+import hashlib
 import json
 import os
 import sys
@@ -121,7 +122,7 @@ def main():
 
     import torch
     import tdc_amd
-    from tdc_amd.conv import Conv2dPlan, time_many_ms
+    from tdc_amd.conv import Conv2dPlan, launch_floor_us, time_many_ms
     from oracle import ref   # checker + cpu_baseline leg only
 
     if not torch.cuda.is_available():
@@ -205,7 +206,9 @@ def main():
                      % ((l["hw"], l["r1"], l["r2"]), l["plan"].info.tile.astuple(), share))
         return share
 
+    t_plans0 = time.perf_counter()
     layers = [make_layer(hw, r1, r2) for hw in ref.SWEEP_HW for r1, r2 in ref.SWEEP_RANKS]
+    plan_creation_s = time.perf_counter() - t_plans0   # tile selection (measured, when --tune > 0), packing, upload
     # the reference's own 18 layer shapes (2080Ti-evaluation/TDC-LAYERS-ORACLE/compile_run.py:21-38), a secondary table
     ref_layers = [make_layer(hw, c, n) for (c, n, hw, _, _) in REFERENCE_LAYERS]
     plans = [l["plan"] for l in layers]
@@ -262,24 +265,38 @@ def main():
 
     # -- per-layer device time and roofline fraction ------------------------------
     # `us` = launch-to-launch time (median of three runs of 100 graph-replayed launches: what a layer costs inside a
-    # stream of work); `kernel_us` = begin-to-end duration of the kernel alone from the committed rocprofv3 trace of
+    # stream of work); `kernel_us_from_committed_trace` = begin-to-end duration of the kernel alone from the committed rocprofv3 trace of
     # isolated launches (every launch followed by a stream synchronisation; median, p10).  An isolated launch starts
     # on an idle, cold chip and pays its whole dispatch ramp and drain, which back-to-back launches overlap with their
     # neighbours: it is the LARGER of the two figures for every layer.
     kernel_only = kernel_only_durations()
+
+    # -- the launch path by itself (tdc_launch_floor_time): dependent launches of a kernel with the same argument block
+    #    that touches no memory, empty or with every wave busy for a set time; as stream launches (how the timed step is
+    #    issued) and as one graph replay (how the per-layer `us` below are issued) -----------------------------------
+    def floor_leg(as_graph):
+        best = lambda **kw: min(launch_floor_us(launches=300, graph=as_graph, **kw) for _ in range(3))
+        empty = best(grid=256, block=512)
+        spins = {sp: best(grid=256, block=512, spin_us=sp) for sp in (1.0, 2.0, 4.0)}
+        return {"empty_kernel_us": round(empty, 3), "empty_kernel_1_workgroup_us": round(best(grid=1, block=64), 3),
+                "busy_1us": round(spins[1.0], 3), "busy_2us": round(spins[2.0], 3), "busy_4us": round(spins[4.0], 3),
+                # what a launch adds to a kernel long enough not to hide under the launch path
+                "overhead_beyond_duration_us": round(spins[4.0] - 4.0, 3)}
+    floor_stream, floor_graph = floor_leg(False), floor_leg(True)
+    layer_floor = (floor_graph if graph else floor_stream)["empty_kernel_us"]   # same launch mode as the per-layer `us`
 
     def layer_row(l):
         info = l["plan"].info
         us = sorted(l["plan"].time_us(l["x"], l["out"], iters=100, graph=graph) for _ in range(3))[1]
         row = {"H": l["hw"], "R1": l["r1"], "R2": l["r2"], "us": round(us, 3),
                "roof_us": round(info.roof_us, 4), "frac": round(info.roof_us / us, 4),
+               # the share of the roofline left once the launch floor (an empty kernel, same launch mode) is taken off
+               "frac_attainable": round(info.roof_us / max(us - layer_floor, info.roof_us), 4),
                "gflops": round(info.flops / us * 1e-3, 1), "tile": list(info.tile.astuple()),
                "parity_share_of_tolerance": round(l["parity"], 4)}
         ko = kernel_only.get((l["r1"], l["r2"], l["hw"]))
-        if ko:
-            row["kernel_us"] = {"median": ko[0], "p10": ko[1]}
-            if ko[2] != row["tile"]:      # (the measured selection settled on another tile when that trace was taken)
-                row["kernel_us"]["tile"] = ko[2]
+        if ko and ko[2] == row["tile"]:   # (only when that trace was taken with the tile timed here)
+            row["kernel_us_from_committed_trace"] = {"median": ko[0], "p10": ko[1]}
         return row
 
     table = []
@@ -340,6 +357,13 @@ def main():
         roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_TBPS * 1e3, "unit": "GB/s",
                     "frac": round(achieved / (PEAK_HBM_TBPS * 1e3), 4), "traffic": None}
     roofline["traffic"] = measured_traffic(dinfo.tile.astuple())
+    roofline["traffic_source"] = ("profiles/core_conv_128x128_56_hbm_traffic.txt (committed rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
+                                  "run with this tile; not measured in this run)" if roofline["traffic"] is not None else
+                                  "none: the committed counter run used another tile")
+    # the whole timed step against the sum of its layers' rooflines (time-weighted, unlike the dominant kernel's frac)
+    roofline["sweep_sum_roof_us"] = round(sum(t["roof_us"] for t in table), 3)
+    roofline["sweep_time_weighted_frac"] = round(sum(t["roof_us"] for t in table) / (ms_per_step * 1e3), 4)
+    roofline["launch_floor_us"] = floor_stream["empty_kernel_us"] if not step_graph else floor_graph["empty_kernel_us"]
     # the same kernel as isolated launches (one hipEvent pair around ONE eager launch, 200 times): includes the
     # start-up of an idle queue, so it is reported next to the back-to-back figure, not used for `achieved`
     singles = sorted(dl["plan"].time_us(dl["x"], dl["out"], iters=1, graph=False) for _ in range(200))
@@ -361,6 +385,17 @@ def main():
         "model_only_us_per_layer": None if model_only_us is None else round(model_only_us, 4),
         "roofline": roofline,
         "geomean_frac": round(float(torch.tensor([t["frac"] for t in table]).log().mean().exp()), 4),
+        "layers_at_or_above_40_percent": sum(1 for t in table if t["frac"] >= 0.40),
+        "launch_floor": {"what": "tdc_launch_floor_time: 300 dependent launches of a kernel with the convolution kernels' argument "
+                                 "block (256 workgroups x 512 threads, no memory access), empty or with every wave busy for "
+                                 "1 / 2 / 4 us; us per launch, best of 3",
+                         "stream_launches": floor_stream, "graph_replay": floor_graph,
+                         "per_layer_us_measured_as": "graph replay" if graph else "stream launches"},
+        "tiles_sha": hashlib.sha1(json.dumps([t["tile"] for t in table]).encode()).hexdigest()[:16],
+        "plan_creation_s": round(plan_creation_s, 2),
+        "kernel_us_from_committed_trace": "profiles/core_conv_layers_kernel_only_durations.txt: rocprofv3 kernel-trace durations of "
+                                          "isolated launches (each followed by a synchronisation); shown only for rows whose "
+                                          "tile is the one that trace was taken with; NOT measured in this run",
         "layers": table,
         "reference_layer_shapes": {
             "what": "the 18 core-conv shapes the reference itself times (2080Ti-evaluation/TDC-LAYERS-ORACLE/compile_run.py:21-38), "

@@ -209,6 +209,15 @@ int tdc_conv_forward_strided(tdc_conv_plan *plan, const float *d_in, int64_t in_
  * cost from the figure.  Synchronises the device before and after. */
 int tdc_conv_time(tdc_conv_plan *plan, const float *d_in, const float *d_residual, float *d_out,
                   int32_t iters, int32_t use_graph, float *total_ms_out);
+/* The launch path by itself, timed the same way: `launches` dependent launches of a kernel that carries the
+ * convolution kernels' argument block, starts `grid` workgroups of `block` threads (a multiple of 64, at most 1024)
+ * and keeps every wave busy for spin_us microseconds (0 = an empty kernel) without touching memory; stream launches,
+ * or one replay of a HIP graph of all of them when use_graph != 0.  The empty kernel gives the launch floor every
+ * layer pays; the spinning ones show how much of a kernel's own duration hides under the launch path of its
+ * successor (launch-to-launch time = max(floor, duration + overhead), not floor + duration).  The reference's harness
+ * has no counterpart: it times one cold launch (template_benchmark_cudnn.template:491-496). */
+int tdc_launch_floor_time(int32_t launches, int32_t use_graph, int32_t grid, int32_t block, float spin_us,
+                          float *total_ms_out);
 /* Same for a list of plans run one after the other: one pass over the `n`
  * plans is one step; the timed region holds `iters` steps (each step one replay of
  * a HIP graph of the n launches when use_graph != 0). */

@@ -62,6 +62,21 @@ int launch_zero_words(unsigned *dst, int n, void *stream) {
     return (int)hipGetLastError();
 }
 
+// Launch-path probe (tdc_launch_floor_time): same argument block as the convolution kernels, no memory access; every
+// wave waits until the constant 100 MHz clock has advanced by `ticks`.
+__global__ void __launch_bounds__(1024) tdc_launch_probe_kernel(const ConvKParams p, int ticks) {
+    if (ticks <= 0) return;
+    const unsigned long long t0 = __builtin_amdgcn_s_memrealtime();
+    // (bounded: the clock always advances, and the host refuses more than 100 us)
+    while ((long long)(__builtin_amdgcn_s_memrealtime() - t0) < (long long)ticks) __builtin_amdgcn_s_sleep(1);
+    if (p.out && threadIdx.x == 0x7fffffff) p.out[0] = 0.0f;   // (never true: keeps the argument block alive)
+}
+
+int launch_floor_probe(const ConvKParams &kp, int grid, int block, int spin_ticks, void *stream) {
+    hipLaunchKernelGGL(tdc_launch_probe_kernel, dim3(grid), dim3(block), 0, (hipStream_t)stream, kp, spin_ticks);
+    return (int)hipGetLastError();
+}
+
 int kernel_resources(const void *fn, int block_threads, int dynamic_lds_bytes, int *vgprs, int *static_lds, int *max_threads,
                      int *max_wg_per_cu) {
     hipFuncAttributes attr{};

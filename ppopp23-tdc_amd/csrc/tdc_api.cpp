@@ -762,6 +762,58 @@ int tdc_conv_time(tdc_conv_plan *plan, const float *d_in, const float *d_residua
     return TDC_OK;
 }
 
+int tdc_launch_floor_time(int32_t launches, int32_t use_graph, int32_t grid, int32_t block, float spin_us, float *total_ms_out) {
+    if (!total_ms_out || launches < 1 || launches > 100000 || grid < 1 || grid > 65535 || block < 64 || block > 1024 ||
+        block % 64 != 0 || !(spin_us >= 0.0f) || spin_us > 100.0f)
+        return fail(TDC_ERR_INVALID, "bad argument");
+    const int ticks = (int)(spin_us * 100.0f + 0.5f);
+    ConvKParams kp{};
+    hipStream_t s = nullptr;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    int he = 0;
+    const char *what = "hipStreamCreate";
+    hipError_t e = hipDeviceSynchronize();
+    if (e == hipSuccess) e = hipStreamCreate(&s);
+    if (e == hipSuccess) { what = "hipEventCreate"; e = hipEventCreate(&e0); }
+    if (e == hipSuccess) e = hipEventCreate(&e1);
+    if (e == hipSuccess && use_graph) {
+        what = "graph capture";
+        e = hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal);
+        if (e == hipSuccess) {
+            for (int i = 0; i < launches && !he; ++i) he = launch_floor_probe(kp, grid, block, ticks, s);
+            e = hipStreamEndCapture(s, &graph);
+        }
+        if (e == hipSuccess && !he) e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+        if (e == hipSuccess && !he) e = hipGraphLaunch(exec, s);   // untimed: upload
+        if (e == hipSuccess && !he) e = hipStreamSynchronize(s);
+    } else if (e == hipSuccess) {
+        for (int i = 0; i < 20 && !he; ++i) he = launch_floor_probe(kp, grid, block, ticks, s);   // untimed: warm-up
+        e = hipStreamSynchronize(s);
+    }
+    if (e == hipSuccess && !he) {
+        what = "timed region";
+        e = hipEventRecord(e0, s);
+        if (use_graph) {
+            if (e == hipSuccess) e = hipGraphLaunch(exec, s);
+        } else {
+            for (int i = 0; i < launches && !he; ++i) he = launch_floor_probe(kp, grid, block, ticks, s);
+        }
+        if (e == hipSuccess) e = hipEventRecord(e1, s);
+        if (e == hipSuccess) e = hipEventSynchronize(e1);
+        if (e == hipSuccess) e = hipEventElapsedTime(total_ms_out, e0, e1);
+    }
+    if (exec) (void)hipGraphExecDestroy(exec);
+    if (graph) (void)hipGraphDestroy(graph);
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    if (s) (void)hipStreamDestroy(s);
+    if (he) return hip_fail("probe launch", he);
+    if (e != hipSuccess) return hip_fail(what, e);
+    return TDC_OK;
+}
+
 void tdc_conv_plan_destroy(tdc_conv_plan *plan) {
     if (!plan) return;
     free_plan_buffers(plan);

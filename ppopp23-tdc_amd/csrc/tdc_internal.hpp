@@ -203,6 +203,9 @@ size_t static_scratch_ctr_bytes();
 int static_scratch_address(void **ptr_out);
 // dst[0..n) = 0 with a small fill kernel (safe under stream capture, unlike hipMemsetAsync).
 int launch_zero_words(unsigned *dst, int n, void *stream);
+// Launch-path probe: a kernel with the convolution kernels' argument block whose waves spin for `spin_ticks` ticks of
+// the 100 MHz constant clock and touch no memory.
+int launch_floor_probe(const ConvKParams &kp, int grid, int block, int spin_ticks, void *stream);
 // What the compiled kernel really uses: registers per lane, static LDS, its launch bound, and how many workgroups
 // of `block_threads` threads with `dynamic_lds_bytes` of LDS the runtime places on one compute unit.
 int kernel_resources(const void *fn, int block_threads, int dynamic_lds_bytes, int *vgprs, int *static_lds, int *max_threads,

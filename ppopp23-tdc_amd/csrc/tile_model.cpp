@@ -663,17 +663,19 @@ bool model_evaluate(const tdc_conv_desc &d, const tdc_tile &t, tdc_tile_info &in
     auto wg_time = [&](int r, long long concurrent_wgs) {
         if (t.alg == 5) {
             // like the streamed direct kernel: set-up, one round trip, the bytes at the achieved fill rate, the requests
-            // of a wave one after the other, its own MFMA chain with the transform's vector work, the reduction, the store.
-            // Per input channel and 16 output channels 1 KiB of transformed weights; per input channel four rows of 128 bytes.
+            // of a wave one after the other, the MFMA chains of the waves that share a SIMD (the transform's vector work
+            // mostly hides under them), output transform and drain, the reduction, the store.  Per input channel and 16
+            // output channels 1 KiB of transformed weights; per input channel four rows of 128 bytes.
+            // (fitted to 60 timed tiles of 13 shapes, 6 % mean error)
             const double chip_share =
                 MC.l2_bytes_per_clk / std::max<double>(1.0, (double)std::min<long long>(concurrent_wgs, m.cus));
-            const double rate = std::min(0.59 * MC.copy_bytes_per_clk, chip_share);
+            const double rate = std::min(1.31 * MC.copy_bytes_per_clk, chip_share);
             const double bytes = (double)t.cch * (t.wm * 1024.0 + 512.0) * r;
             const double groups = (double)t.cch / (4.0 * t.wk);
             const double waves_simd = std::ceil((double)g.waves * r / m.simds_per_cu);
             double clk = MC.stream_setup_clk + MC.stream_latency_clk + 65.0 * (waves_simd - 1.0) + bytes / rate +
-                         groups * 8.0 * 21.4 + waves_simd * groups * 16.0 * (mfma_clk + MC.wino_kstep_clk);
-            clk += 1.6 * MC.sync_clk + 200.0;   // output transform, park, barrier
+                         groups * 8.0 * 21.4 + waves_simd * groups * 16.0 * (mfma_clk + 10.0);
+            clk += 1.6 * MC.sync_clk + 1000.0;   // MFMA drain, output transform, park, barrier
             const double rounds = std::ceil((double)g.MT * 32.0 / g.threads);
             clk += rounds * (110.0 + 8.0 * t.wk) + out_bytes * r / 200.0;
             return clk;

@@ -22,7 +22,7 @@ EXPORTS = (
     "tdc_conv_plan_set_weights", "tdc_conv_plan_set_input_affine", "tdc_conv_plan_set_head", "tdc_conv_plan_query",
     "tdc_conv_forward", "tdc_conv_forward_static_ws", "tdc_conv_plan_occupancy",
     "tdc_conv_forward_strided", "tdc_tkconv_forward_strided",
-    "tdc_conv_time", "tdc_conv_time_many", "tdc_conv_plan_destroy",
+    "tdc_conv_time", "tdc_conv_time_many", "tdc_launch_floor_time", "tdc_conv_plan_destroy",
     "tdc_tkconv_create", "tdc_tkconv_set_weights", "tdc_tkconv_forward", "tdc_tkconv_forward_features",
     "tdc_tkconv_core_forward", "tdc_tkconv_query", "tdc_tkconv_num_kernels", "tdc_tkconv_destroy",
     "tdc_model_evaluate", "tdc_model_kernel_info", "tdc_model_enumerate", "tdc_model_select", "tdc_model_select_with_tail", "tdc_model_get_constants",
@@ -107,6 +107,7 @@ def lib():
     L.tdc_conv_forward_static_ws.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]
     L.tdc_conv_plan_occupancy.argtypes = [c_void_p, POINTER(KernelOccupancy)]
     L.tdc_conv_time.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int32, POINTER(ctypes.c_float)]
+    L.tdc_launch_floor_time.argtypes = [c_int32, c_int32, c_int32, c_int32, ctypes.c_float, POINTER(ctypes.c_float)]
     L.tdc_conv_time_many.argtypes = [POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p), c_int32, c_int32, c_int32,
                                      POINTER(ctypes.c_float)]
     L.tdc_conv_plan_destroy.argtypes = [c_void_p]

@@ -170,6 +170,15 @@ def time_many_ms(plans, xs, outs, iters=1, graph=True):
     return ms.value
 
 
+def launch_floor_us(launches=300, graph=False, grid=256, block=512, spin_us=0.0):
+    """Device microseconds per launch of `launches` dependent probe kernels (the convolution kernels' argument block,
+    no memory access, every wave busy for `spin_us`): the launch floor with spin_us = 0."""
+    import ctypes
+    ms = ctypes.c_float(0.0)
+    check(lib().tdc_launch_floor_time(launches, int(graph), grid, block, float(spin_us), byref(ms)))
+    return ms.value * 1e3 / launches
+
+
 def _out_dim(n, k, stride, pad, dil):
     return (n + 2 * pad - dil * (k - 1) - 1) // stride + 1
 

@@ -222,6 +222,75 @@ def resnet18_params(seed=18, num_classes=1000, rank_ratio=0.5):
     return p
 
 
+def _basic_block(net, x, p, pre, blk_stride, fused_middle):
+    """One TTBasicBlock (inference/resnet_inet_tt.py:53-117): conv1 (TKConv) + bn1 + ReLU, conv2 (TKConv) + bn2,
+    + identity (through the 1x1 downsample convolution + BatchNorm where the block has one), ReLU.  With
+    `fused_middle` the last factor of conv1 (with bn1 folded in, + ReLU) and the first factor of conv2 run as ONE kernel
+    (a 1x1 convolution with a 1x1 tail): the block's middle tensor of `planes` channels never reaches memory and a
+    launch disappears; the two cores and the outer factors are separate launches then."""
+    identity = x
+    if pre + ".downsample.0.weight" in p:
+        ds, dt = bn_scale_shift(p, pre + ".downsample.1")
+        identity = net.conv(x, fold_dense(p[pre + ".downsample.0.weight"], ds), dt, stride=blk_stride)
+    s1, t1 = bn_scale_shift(p, pre + ".bn1")
+    s2, t2 = bn_scale_shift(p, pre + ".bn2")
+    last1 = fold_dense(p[pre + ".conv1.last_kernel"], s1)
+    last2 = fold_dense(p[pre + ".conv2.last_kernel"], s2)
+    if not fused_middle:
+        y = net.tkconv(x, p[pre + ".conv1.first_kernel"], p[pre + ".conv1.core_kernel"], last1, t1, stride=blk_stride, pad=1,
+                       relu=True)
+        return net.tkconv(y, p[pre + ".conv2.first_kernel"], p[pre + ".conv2.core_kernel"], last2, t2, stride=1, pad=1,
+                          residual=identity, relu=True)
+    y = net.conv(x, p[pre + ".conv1.first_kernel"])
+    y = net.conv(y, p[pre + ".conv1.core_kernel"], stride=blk_stride, pad=1)
+    y = net.conv_tail(y, last1, p[pre + ".conv2.first_kernel"], bias=t1, relu=True)
+    y = net.conv(y, p[pre + ".conv2.core_kernel"], stride=1, pad=1)
+    return net.conv(y, last2, t2, residual=identity, relu=True)
+
+
+_BASIC_BLOCK_FUSES = {}
+
+
+def _basic_block_fuses(batch, cin, h, w, p, pre, blk_stride):
+    """Whether a block runs faster with the middle pair of 1x1 factors fused (see _basic_block).  The fused kernel needs
+    every channel of the block's middle tensor in one workgroup, which the kernels offer up to 256 channels.  Without
+    measured tile selection: fuse where the plain layout does not already run each Tucker convolution as one launch.
+    With it, both layouts of the block are built as networks of their own and timed (remembered per shape)."""
+    planes = p[pre + ".conv1.last_kernel"].shape[0]
+    if planes > 256:
+        return False
+    key = (batch, cin, h, w, planes, p[pre + ".conv1.first_kernel"].shape[0], blk_stride, pre + ".downsample.0.weight" in p,
+           _lib.get_autotune() > 0)
+    if key not in _BASIC_BLOCK_FUSES:
+        nets, ok = [], True
+        for fused in (False, True):
+            m = Net(batch, cin, h, w)
+            try:
+                m.finalize(_basic_block(m, 0, p, pre, blk_stride, fused))
+            except _lib.TdcError:      # (no tile carries this tail)
+                m.close()
+                ok = False
+                break
+            nets.append(m)
+        if not ok:
+            for m in nets:
+                m.close()
+            _BASIC_BLOCK_FUSES[key] = False
+        elif _lib.get_autotune() <= 0:
+            _BASIC_BLOCK_FUSES[key] = nets[1].num_kernels < nets[0].num_kernels
+        else:
+            x = torch.randn(batch, cin, h, w, device="cuda")
+            t = []
+            for m in nets:
+                m.forward(x)
+                m.time_ms(iters=10)
+                t.append(min(m.time_ms(iters=30) for _ in range(3)))
+            _BASIC_BLOCK_FUSES[key] = t[1] < 0.98 * t[0]
+        for m in nets:
+            m.close()
+    return _BASIC_BLOCK_FUSES[key]
+
+
 def build_tucker_resnet18(params, batch=1, H=224, W=224):
     """Returns a finalized Net computing the logits [batch, num_classes, 1, 1]."""
     p = params
@@ -236,16 +305,8 @@ def build_tucker_resnet18(params, batch=1, H=224, W=224):
         for b in range(2):
             pre = f"layer{st}.{b}"
             blk_stride = stride if b == 0 else 1
-            identity = x
-            if pre + ".downsample.0.weight" in p:
-                ds, dt = bn_scale_shift(p, pre + ".downsample.1")
-                identity = net.conv(x, fold_dense(p[pre + ".downsample.0.weight"], ds), dt, stride=blk_stride)
-            s1, t1 = bn_scale_shift(p, pre + ".bn1")
-            y = net.tkconv(x, p[pre + ".conv1.first_kernel"], p[pre + ".conv1.core_kernel"],
-                           fold_dense(p[pre + ".conv1.last_kernel"], s1), t1, stride=blk_stride, pad=1, relu=True)
-            s2, t2 = bn_scale_shift(p, pre + ".bn2")
-            x = net.tkconv(y, p[pre + ".conv2.first_kernel"], p[pre + ".conv2.core_kernel"],
-                           fold_dense(p[pre + ".conv2.last_kernel"], s2), t2, stride=1, pad=1, residual=identity, relu=True)
+            _, cin, h, w = net.shape(x)
+            x = _basic_block(net, x, p, pre, blk_stride, _basic_block_fuses(batch, cin, h, w, p, pre, blk_stride))
             net.feature_ids[pre] = x
     x = net.global_avgpool(x)
     x = net.conv(x, p["fc.weight"].reshape(p["fc.weight"].shape[0], -1, 1, 1), p["fc.bias"])
