@@ -85,33 +85,11 @@ struct Mfma<16> {
 
 constexpr int OOB_OFFSET = 0x7ffffff0;  // beyond any buffer: the load returns zero
 
-// Output stores.  TDC_STORE_WT (experiment builds): written through the die's L2 at once (device-scope store) instead
-// of staying dirty there until the kernel ends.
-#ifndef TDC_STORE_WT
-#define TDC_STORE_WT 0
-#endif
-__device__ __forceinline__ void store_out(float *p, float v) {
-#if TDC_STORE_WT
-    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-#else
-    *p = v;
-#endif
-}
-__device__ __forceinline__ void store_out(float *p, f4_t v) {
-#if TDC_STORE_WT
-    asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
-#else
-    *reinterpret_cast<f4_t *>(p) = v;
-#endif
-}
+// Output stores (plain: the lines stay in the die's L2 until the kernel ends).
+__device__ __forceinline__ void store_out(float *p, float v) { *p = v; }
+__device__ __forceinline__ void store_out(float *p, f4_t v) { *reinterpret_cast<f4_t *>(p) = v; }
 typedef float f2_store_t __attribute__((ext_vector_type(2)));
-__device__ __forceinline__ void store_out(float *p, f2_store_t v) {
-#if TDC_STORE_WT
-    asm volatile("global_store_dwordx2 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
-#else
-    *reinterpret_cast<f2_store_t *>(p) = v;
-#endif
-}
+__device__ __forceinline__ void store_out(float *p, f2_store_t v) { *reinterpret_cast<f2_store_t *>(p) = v; }
 
 __device__ __forceinline__ int fdiv(int n, const FastDiv &f) {
     return (int)(__umulhi((unsigned)n, f.m) + ((unsigned)n & f.pass));

@@ -304,9 +304,6 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
     // of every pass is requested before the wait and the barrier of that pass and is in registers when they end.
     f4_t wu0[WINO ? 4 : 1];
     auto wino_load_a = [&](int chunk, int g, f4_t(&u)[4]) {
-#if defined(TDC_PROBE) && (TDC_PROBE & 1)
-        if (g > 0) return;   // timing probe (wrong results): no weight requests inside the loop
-#endif
         const int soff = (int)(w_byte_base + (unsigned)chunk * w_pass_bytes) + ((wm * ncg_pass + wk * ncgw + g) * 16) * 256;
 #pragma unroll
         for (int q = 0; q < 4; ++q)
@@ -425,21 +422,12 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_conv_mfma_kernel(const ConvKPar
             float v0[16], v1[16];
             f4_t u1[4];
             auto load_patch = [&](int g, float(&v)[16]) {
-#if defined(TDC_PROBE) && (TDC_PROBE & 2)
-                if (g > 0) return;   // timing probe (wrong results): no patch reads and no input transform inside the loop
-#endif
                 const float *b = praw + g * gstep;
                 float d[4][4];
 #pragma unroll
                 for (int r = 0; r < 4; ++r)
 #pragma unroll
                     for (int c = 0; c < 4; ++c) d[r][c] = b[r * RS + c];
-#if defined(TDC_PROBE) && (TDC_PROBE & 4)
-                // timing probe (wrong results): the patch is read but not transformed
-#pragma unroll
-                for (int i = 0; i < 16; ++i) v[i] = d[i >> 2][i & 3];
-                return;
-#endif
                 float tr[4][4];   // B^T d: rows
 #pragma unroll
                 for (int c = 0; c < 4; ++c) {

@@ -147,14 +147,12 @@ class TKConv2dC(nn.Module):
         return out
 
     def _versions(self):
+        """What the native copies were packed from: storage address and autograd version counter of every parameter.
+        No element is read (a device-resident parameter would cost a blocking copy per forward, and forward would fail
+        under stream capture).  Writes the version counter does not see — ``p.data.copy_(w)``, ``p.data = w`` with the
+        same storage — need ``invalidate()``; ``load_kernels``, ``load_state_dict`` and ``.to()`` call it themselves."""
         ps = [self.first_kernel, self.core_kernel, self.last_kernel] + ([self.bias] if self.bias is not None else [])
-        # (storage address and version counter; writes through .data bump neither, hence the first/last elements as a
-        #  cheap additional check — a full comparison would cost more than the convolution)
-        stamp = []
-        for p in ps:
-            flat = p.detach().reshape(-1)
-            stamp.append((p.data_ptr(), p._version, float(flat[0]), float(flat[-1])))
-        return tuple(stamp)
+        return tuple((p.data_ptr(), p._version) for p in ps)
 
     def _op_for(self, x):
         if x.dim() != 4 or x.shape[1] != self.in_channels:

@@ -254,11 +254,18 @@ _BASIC_BLOCK_FUSES = {}
 def _basic_block_fuses(batch, cin, h, w, p, pre, blk_stride):
     """Whether a block runs faster with the middle pair of 1x1 factors fused (see _basic_block).  The fused kernel needs
     every channel of the block's middle tensor in one workgroup, which the kernels offer up to 256 channels.  Without
-    measured tile selection: fuse where the plain layout does not already run each Tucker convolution as one launch.
-    With it, both layouts of the block are built as networks of their own and timed (remembered per shape)."""
+    measured tile selection the tile model decides (the fused kernel predicted at 0.7 of the two launches or less: timed
+    at batch 1 it takes 1.4-3.7x of what two launches take — 64 -> 128 -> 64 @28x28: 7.9 us against 2.7 + 2.8;
+    128 -> 256 -> 128 @14x14: 22.9 against 2.9 + 3.1 — because one workgroup per 16-64 pixels owns every channel).  With
+    it, both layouts of the block are built as networks of their own and timed (remembered per shape)."""
     planes = p[pre + ".conv1.last_kernel"].shape[0]
+    r2 = p[pre + ".conv1.last_kernel"].shape[1]
     if planes > 256:
         return False
+    if _lib.get_autotune() <= 0:
+        ho, wo = (h + 2 - 3) // blk_stride + 1, (w + 2 - 3) // blk_stride + 1
+        d1 = _lib.conv_desc(batch, r2, planes, ho, wo, 1, 1, 1, 0, 1, True, True)
+        return _lib.fused_tail_pays(d1, p[pre + ".conv2.first_kernel"].shape[0], margin=0.7)
     key = (batch, cin, h, w, planes, p[pre + ".conv1.first_kernel"].shape[0], blk_stride, pre + ".downsample.0.weight" in p,
            _lib.get_autotune() > 0)
     if key not in _BASIC_BLOCK_FUSES:
@@ -273,11 +280,7 @@ def _basic_block_fuses(batch, cin, h, w, p, pre, blk_stride):
                 break
             nets.append(m)
         if not ok:
-            for m in nets:
-                m.close()
             _BASIC_BLOCK_FUSES[key] = False
-        elif _lib.get_autotune() <= 0:
-            _BASIC_BLOCK_FUSES[key] = nets[1].num_kernels < nets[0].num_kernels
         else:
             x = torch.randn(batch, cin, h, w, device="cuda")
             t = []

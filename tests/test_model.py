@@ -88,6 +88,43 @@ def test_streamed_tiles_only_where_they_apply():
     assert not any(t.alg >= 3 for t in tdc_amd.model_enumerate(tdc_amd.conv_desc(1, 3, 64, 32, 32, 7, 7, 2, 3)))
 
 
+def test_streamed_winograd_tiles_only_where_they_apply():
+    """tile.alg = 5: Winograd F(2x2,3x3) with both operands read from global memory; 3x3 / stride 1 / pad 1 / even width,
+    a tile-row block of 2 x 28 pixels per workgroup, every input channel in one pass, 1 to 4 groups of four per wave."""
+    d = conv3(64, 64, 56)
+    ok = tdc_amd.model_evaluate(d, tdc_amd.Tile(16, 1, 1, 1, 1, 8, 64, 28, 1, 0, 5))
+    assert (ok.grid_x, ok.grid_y, ok.th, ok.block_threads, ok.lds_bytes, ok.nchunks) == (56, 4, 2, 512, 8 * 16 * 64 * 4, 1)
+    from tdc_amd import _lib
+    name, regs, waves = _lib.model_kernel_info(d, ok.tile, False)
+    assert name == "tdc_wino3x3_stream_kernel<2, 16>" and regs <= 128 and waves >= 4
+    wide = tdc_amd.model_evaluate(d, tdc_amd.Tile(16, 1, 1, 2, 1, 4, 64, 28, 1, 0, 5))     # two blocks of 16 channels, four groups per wave
+    assert (wide.grid_x, wide.grid_y, wide.block_threads) == (56, 2, 512)
+    ragged = tdc_amd.model_evaluate(conv3(50, 20, 30), tdc_amd.Tile(16, 1, 1, 1, 1, 13, 52, 28, 1, 0, 5))   # 13 groups, one per wave
+    assert (ragged.grid_x, ragged.grid_y) == (2 * 15, 2)
+    for dd, t in [(d, tdc_amd.Tile(16, 1, 1, 1, 1, 2, 64, 28, 1, 0, 5)),        # eight groups per wave
+                  (d, tdc_amd.Tile(16, 1, 1, 1, 1, 8, 32, 28, 1, 0, 5)),        # not all channels in one pass
+                  (d, tdc_amd.Tile(16, 1, 1, 1, 1, 16, 128, 28, 1, 0, 5)),      # half of the waves without channels
+                  (d, tdc_amd.Tile(16, 1, 1, 1, 1, 8, 64, 14, 1, 0, 5)),        # tw must be 28
+                  (d, tdc_amd.Tile(16, 1, 1, 1, 1, 8, 64, 28, 2, 0, 5)),        # no split across workgroups
+                  (d, tdc_amd.Tile(16, 1, 1, 1, 1, 8, 64, 28, 1, 2, 5)),        # no loader waves
+                  (d, tdc_amd.Tile(16, 1, 1, 1, 2, 8, 64, 28, 1, 0, 5)),        # one block per wave set
+                  (d, tdc_amd.Tile(16, 1, 1, 4, 1, 4, 64, 28, 1, 0, 5)),        # four groups per wave: at most 12 waves
+                  (conv3(64, 64, 7), tdc_amd.Tile(16, 1, 1, 1, 1, 8, 64, 28, 1, 0, 5)),                 # odd width
+                  (conv3(64, 64, 56, stride=2), tdc_amd.Tile(16, 1, 1, 1, 1, 8, 64, 28, 1, 0, 5)),      # stride 2
+                  (tdc_amd.conv_desc(1, 64, 64, 56, 56, 3, 3, 1, 0), tdc_amd.Tile(16, 1, 1, 1, 1, 8, 64, 28, 1, 0, 5)),     # pad 0
+                  (tdc_amd.conv_desc(1, 64, 64, 56, 56, 3, 3, 1, 2, 2), tdc_amd.Tile(16, 1, 1, 1, 1, 8, 64, 28, 1, 0, 5)),  # dilation
+                  (tdc_amd.conv_desc(1, 64, 64, 56, 56, 1, 1, 1, 0), tdc_amd.Tile(16, 1, 1, 1, 1, 8, 64, 28, 1, 0, 5))]:
+        with pytest.raises(tdc_amd.TdcError):
+            tdc_amd.model_evaluate(dd, t)
+    assert any(t.alg == 5 for t in tdc_amd.model_enumerate(d))
+    assert not any(t.alg == 5 for t in tdc_amd.model_enumerate(conv3(64, 64, 7)))
+    assert not any(t.alg == 5 for t in tdc_amd.model_enumerate(conv3(64, 64, 56, stride=2)))
+    assert not any(t.alg == 5 for t in tdc_amd.model_enumerate(d, ) if t.ks != 1 or t.wl != 0)
+    # the model takes it where it was measured faster: the mid-size 56 x 56 layers
+    assert tdc_amd.model_select(d).tile.alg == 5 and tdc_amd.model_select(conv3(64, 128, 56)).tile.alg == 5
+    assert tdc_amd.model_select(conv3(16, 16, 56)).tile.alg == 4 and tdc_amd.model_select(conv3(128, 128, 28)).tile.alg == 4
+
+
 def test_winograd_tiles_only_where_the_algorithm_applies():
     """tile.alg needs a 3x3 / stride 1 / dilation 1 convolution and one 16x16 block per wave; the model hands the
     large 56x56 layers to it and keeps the small ones on the direct path."""

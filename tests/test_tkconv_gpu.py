@@ -113,7 +113,7 @@ def test_module_forward_matches_reference_forward():
                              1, 1, 1)
     assert_close(m(x2.cuda()).cpu().numpy(), want2.numpy(), "module after update")
     # writes through .data do not bump the version counter: invalidate() (or load_state_dict / load_kernels) re-packs
-    m.last_kernel.data[1:-1].mul_(-2.0)          # (first and last element untouched: the cheap stamp cannot see it)
+    m.last_kernel.data[1:-1].mul_(-2.0)          # (the stamp — storage address and version counter — cannot see it)
     m.invalidate()
     want3 = ref.tkconv_torch(x2, m.first_kernel.detach(), m.core_kernel.detach(), m.last_kernel.detach(), m.bias.detach(),
                              1, 1, 1)
@@ -122,6 +122,12 @@ def test_module_forward_matches_reference_forward():
     m.load_state_dict(sd)
     want4 = ref.tkconv_torch(x2, sd["first_kernel"], sd["core_kernel"], sd["last_kernel"], sd["bias"], 1, 1, 1)
     assert_close(m(x2.cuda()).cpu().numpy(), want4.numpy(), "module after load_state_dict")
+    # a module moved to the device works too, and a forward with unchanged parameters reads no parameter element
+    # (the stamp is addresses and version counters only), so it can run with the device's copy engines busy or idle alike
+    m.cuda()
+    assert_close(m(x2.cuda()).cpu().numpy(), want4.numpy(), "module after .cuda()")
+    assert all(isinstance(v, int) for pair in m._versions() for v in pair)
+    m.cpu()
     # the per-shape operator cache is bounded
     for hw in range(5, 5 + m.MAX_CACHED_SHAPES + 3):
         m(torch.randn(1, 40, hw, hw).cuda())

@@ -81,3 +81,41 @@ def test_plans_without_a_split_need_no_scratch():
     torch.cuda.synchronize()
     assert torch.equal(a, b)
     plan.close()
+
+
+def test_static_workspace_entry_point_allocates_nothing_and_replays_from_a_graph():
+    """The two properties the entry point exists for: no device allocation per call (free device memory as the driver
+    reports it does not move over many calls), and usable under stream capture — the captured graph is replayed several
+    times with the program's own eager work and synchronisations in between and inputs that change between replays, and
+    every replay is compared bit for bit with the eager entry point.  The symbol address of the static array is resolved
+    by the eager call in front of the capture."""
+    B, C, N, H, W = 1, 256, 256, 7, 7
+    x, w, bias, resid = _case(7100, B, C, N, H, W, 3)
+    tile = _split_tile(tdc_amd.conv_desc(B, C, N, H, W, 3, 3, 1, 1), 4)
+    plan = tdc_amd.Conv2dPlan(B, C, N, H, W, 3, 3, 1, 1, 1, True, True, tile=tile).set_weights(w, bias)
+    xd, rd = x.cuda(), resid.cuda()
+    got = torch.empty(B, N, H, W, device="cuda")
+    want = torch.empty(B, N, H, W, device="cuda")
+    plan.forward_static_ws(xd, rd, out=got)      # eager: also resolves the address of this device's copy of the array
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    for _ in range(50):
+        plan.forward_static_ws(xd, rd, out=got)
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before, "free device memory moved across 50 calls"
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            plan.forward_static_ws(xd, rd, out=got)
+    g = seeded(7101)
+    for rep in range(4):
+        xd.copy_((torch.rand(B, C, H, W, generator=g) * 2 - 1).cuda())     # eager work between the replays
+        plan.forward(xd, rd, out=want)
+        got.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), f"replay {rep}: graph-replayed static-workspace result differs from tdc_conv_forward"
+    del graph
+    plan.close()
