@@ -126,14 +126,14 @@ __device__ __forceinline__ void finish_four_channels(const f4_t &acc, int ch0, i
 // then loads the values in, it hits the scalar cache.
 __device__ __forceinline__ void touch_kernel_arguments() {
     if constexpr (TDC_TOUCH_KERNARGS) {
-        static_assert(sizeof(ConvKParams) <= 8 * 64, "touch more lines");
+        static_assert(sizeof(ConvKParams) > 8 * 64 && sizeof(ConvKParams) <= 9 * 64, "touch exactly the lines of the argument block");
         const auto kargs = __builtin_amdgcn_kernarg_segment_ptr();
-        unsigned t0, t1, t2, t3, t4, t5, t6, t7;
+        unsigned t0, t1, t2, t3, t4, t5, t6, t7, t8;
         asm volatile(
-            "s_load_dword %0, %8, 0x0\n\ts_load_dword %1, %8, 0x40\n\ts_load_dword %2, %8, 0x80\n\t"
-            "s_load_dword %3, %8, 0xc0\n\ts_load_dword %4, %8, 0x100\n\ts_load_dword %5, %8, 0x140\n\t"
-            "s_load_dword %6, %8, 0x180\n\ts_load_dword %7, %8, 0x1c0\n\ts_waitcnt lgkmcnt(0)"
-            : "=&s"(t0), "=&s"(t1), "=&s"(t2), "=&s"(t3), "=&s"(t4), "=&s"(t5), "=&s"(t6), "=&s"(t7)
+            "s_load_dword %0, %9, 0x0\n\ts_load_dword %1, %9, 0x40\n\ts_load_dword %2, %9, 0x80\n\t"
+            "s_load_dword %3, %9, 0xc0\n\ts_load_dword %4, %9, 0x100\n\ts_load_dword %5, %9, 0x140\n\t"
+            "s_load_dword %6, %9, 0x180\n\ts_load_dword %7, %9, 0x1c0\n\ts_load_dword %8, %9, 0x200\n\ts_waitcnt lgkmcnt(0)"
+            : "=&s"(t0), "=&s"(t1), "=&s"(t2), "=&s"(t3), "=&s"(t4), "=&s"(t5), "=&s"(t6), "=&s"(t7), "=&s"(t8)
             : "s"(kargs)
             : "memory");
     }

@@ -64,6 +64,37 @@ __device__ __forceinline__ bool stream_join_slices(const ConvKParams &p, float *
     return true;
 }
 
+// The partial blocks of the WK waves that split the input channels lie in LDS as [wave][register 0-3][lane].  Sum of
+// register `i` over the WK slices from `first` on, in slice order (the result does not depend on timing), eight reads in
+// flight at a time: read one by one, every slice would cost this wave a whole LDS round trip.
+__device__ __forceinline__ float sum_slices(const float *lds, int first, int WK, int i, int lane) {
+    const float *src = lds + (first * 4 + i) * 64 + lane;
+    float sum = 0.0f;
+    for (int w0 = 0; w0 < WK; w0 += 8) {
+        float part[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) part[u] = src[min(w0 + u, WK - 1) * 256];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (w0 + u < WK) sum += part[u];
+    }
+    return sum;
+}
+
+// One output channel `ch` of pixel `pix` (a lane of a wave that finishes ONE accumulator register of the block):
+// + bias, + residual, ReLU, store.
+__device__ __forceinline__ void finish_one_channel(float val, int ch, int N, long long P, long long pix,
+                                                   const float *__restrict__ bias, const float *__restrict__ resid, int relu,
+                                                   float *__restrict__ out) {
+    if (ch >= N) return;
+    const float bv = bias ? bias[ch] : 0.0f;
+    const float rv = resid ? resid[(long long)ch * P + pix] : 0.0f;
+    val += bv;
+    val += rv;
+    if (relu) val = fmaxf(val, 0.0f);
+    store_out(out + ((long long)ch * P + pix), val);
+}
+
 // ---------------------------------------------------------------------------
 // 1x1 convolution with many input channels over few pixels (tile.alg = 3): no LDS stage, no passes, no barrier
 // before the reduction.  One workgroup owns a 16-channel x 16-pixel block of the output; its WK waves split the
@@ -162,11 +193,19 @@ __global__ void __launch_bounds__(NQ == 8 ? 512 : 1024) tdc_conv1x1_stream_kerne
 #pragma unroll
         for (int i = 0; i < 4; ++i) lds[(wave * 4 + i) * 64 + lane] = acc[i];
         __syncthreads();
+        if constexpr (!SPLIT) {
+            if (p.WK >= 4) {
+                // the first four waves share the final sum and the store: wave w finishes accumulator register w
+                // (output channel 4k + w of its lanes' pixels)
+                if (wave >= 4 || px >= p.P) return;
+                finish_one_channel(sum_slices(lds, 0, p.WK, wave, lane), by * 16 + 4 * k + wave, p.N, p.P, px, p.bias, resid,
+                                   p.relu, out);
+                return;
+            }
+        }
         if (wave == 0) {
-            acc = (f4_t){0.0f, 0.0f, 0.0f, 0.0f};
-            for (int w = 0; w < p.WK; ++w)
 #pragma unroll
-                for (int i = 0; i < 4; ++i) acc[i] += lds[(w * 4 + i) * 64 + lane];
+            for (int i = 0; i < 4; ++i) acc[i] = sum_slices(lds, 0, p.WK, i, lane);
         }
     }
     if constexpr (SPLIT) {
@@ -184,16 +223,25 @@ __global__ void __launch_bounds__(NQ == 8 ? 512 : 1024) tdc_conv1x1_stream_kerne
 // tile.alg = 2: two 128-bit loads and one 32-bit load); padding, channels past C and lanes past the tile present an
 // out-of-range offset and read zero without a memory access.
 // ---------------------------------------------------------------------------
-// ROW (stride 1 and a tile of one row of 14 pixels): the 16 lanes of a quarter load the 16 consecutive input pixels
-// that the row of outputs touches, once per filter row, and the three taps of a row are lane shifts of that value
-// (three requests per group of channels instead of nine).
+// INP: how a wave gets its pixel operands.
+//   0  nine 32-bit requests per group of channels, one per tap;
+//   1  (stride 1 and a tile of one row of 14 pixels) the 16 lanes of a quarter load the 16 consecutive input pixels
+//      that the row of outputs touches, once per filter row, and the three taps of a row are lane shifts of that value
+//      (three requests per group of channels instead of nine);
+//   2  (tile.alg = 6) the tile's input WINDOW — (TH-1)*stride+3 rows of up to 24 columns, from the 4-column boundary
+//      at or left of its first column — is loaded with ONE or two 128-bit requests per group of four channels (lane n
+//      of a quarter takes four consecutive columns of one window row), masked where it leaves the image, and left in a
+//      wave-private piece of LDS, from which every lane reads its nine taps.  The compute unit's address path takes
+//      about as long for a 32-bit request of a wave as for a 128-bit one (12 against 16-17 cycles, measured), so the
+//      window costs it a ninth (a third, against INP = 1) of the time; LDS reads are several times cheaper.  No
+//      workgroup barrier is involved: a wave only reads what it wrote itself.
 // MODE: 0 = plain, 1 = input channels dealt to p.KS workgroups, 2 = with the fused 1x1 tail, 3 = with a fused 1x1 head in
 // front as well (a whole Tucker convolution in one launch: the workgroup first computes the first factor on its window of
 // (TH + 2) x (TW + 2) pixels into LDS, which the core loop then reads instead of global memory).  Separate instantiations:
 // code a launch never runs still costs it (0.13 us per launch measured for the split's code inside the plain kernel).
-template <int CG, bool ROW, int MODE>
+template <int CG, int INP, int MODE>
 __global__ void __launch_bounds__(1024) tdc_conv3x3_stream_kernel(const ConvKParams p) {
-    constexpr bool SPLIT = MODE == 1, TAIL = MODE == 2 || MODE == 3, HEAD = MODE == 3;
+    constexpr bool SPLIT = MODE == 1, TAIL = MODE == 2 || MODE == 3, HEAD = MODE == 3, ROW = INP == 1, WINDOW = INP == 2;
     extern __shared__ __align__(16) float lds[];
     touch_kernel_arguments();
     const int tid = threadIdx.x;
@@ -299,8 +347,66 @@ __global__ void __launch_bounds__(1024) tdc_conv3x3_stream_kernel(const ConvKPar
 #pragma unroll
             for (int t = 0; t < 9; ++t)
                 b[g][t] = Fk[4 * g * p.head_ld + min((jy + t / 3) * p.head_ww + jx + t % 3, wmax)];
-    } else
-    if constexpr (ROW) {
+    } else if constexpr (WINDOW) {
+        // The window of this tile: rows iyw0 .. iyw0 + win_rows - 1, columns from ixa (a multiple of four, at or left of
+        // the tile's first input column) in win_L segments of four.  Lane n of a quarter takes slot q * 16 + n of its
+        // channel, slot = row * win_L + segment; slots past the window and segments left or right of the image row, or in
+        // a row above or below the image, present the out-of-range offset and read zeros; a segment that straddles the
+        // right edge is loaded whole and masked.
+        const int L = p.win_L, NS = p.win_ns;
+        const int ixw0 = tile_x * p.TW * p.stride - p.pad;
+        const int ixa = (ixw0 >> 2) << 2;                 // (arithmetic shift: floors negative columns too)
+        const int iyw0 = tile_y * p.TH * p.stride - p.pad;
+        constexpr int NREQ = 2;
+        float *win = lds + p.win_off + wave * (CG * 4 * NS) + k * NS;     // this lane's channel of group 0
+        unsigned soff[NREQ];
+        int wslot[NREQ], ncol[NREQ];
+#pragma unroll
+        for (int q = 0; q < NREQ; ++q) {
+            const int slot = q * 16 + n;
+            const int row = fdiv(slot, p.fd_winL);
+            const int cs = ixa + 4 * (slot - row * L);
+            const bool ok = row < p.win_rows && (unsigned)(iyw0 + row) < (unsigned)p.H && (unsigned)cs < (unsigned)p.W;
+            const unsigned m = ok ? 0xffffffffu : 0u;
+            soff[q] = ((unsigned)((iyw0 + row) * p.W + cs) * 4u & m) | ((unsigned)OOB_OFFSET & ~m);
+            wslot[q] = row < p.win_rows ? slot * 4 : -1;          // where this lane's four columns go (floats), or nowhere
+            ncol[q] = p.W - cs;                                   // columns of the segment inside the row
+        }
+        f4_t wv[CG][NREQ];
+#pragma unroll
+        for (int g = 0; g < CG; ++g) {
+#pragma unroll
+            for (int q = 0; q < NREQ; ++q)
+                if (q == 0 || p.win_nreq > 1)
+                    wv[g][q] = __builtin_bit_cast(f4_t, __builtin_amdgcn_raw_buffer_load_b128(
+                        in_rsrc, (int)(soff[q] + base + (unsigned)(4 * g) * chan_bytes), 0, 0));
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int g = 0; g < CG; ++g)
+#pragma unroll
+            for (int q = 0; q < NREQ; ++q)
+                if ((q == 0 || p.win_nreq > 1) && wslot[q] >= 0) {
+                    f4_t v = wv[g][q];
+#pragma unroll
+                    for (int e = 1; e < 4; ++e) v[e] = e < ncol[q] ? v[e] : 0.0f;
+                    *reinterpret_cast<f4_t *>(win + g * 4 * NS + wslot[q]) = v;
+                }
+        // (the lanes of a wave exchange data through LDS here: its LDS instructions complete in order, and nothing may be
+        //  moved across this point by the compiler)
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        const int jyc = min(jy, p.TH - 1);   // (lanes past the tile re-read its last row; they are never stored)
+        const float *rd = win + (jyc * p.stride) * (4 * L) + jx * p.stride + (ixw0 - ixa);
+#pragma unroll
+        for (int g = 0; g < CG; ++g)
+#pragma unroll
+            for (int r = 0; r < 3; ++r)
+#pragma unroll
+                for (int c = 0; c < 3; ++c) b[g][r * 3 + c] = rd[g * 4 * NS + r * (4 * L) + c];
+    } else if constexpr (ROW) {
         // lane n of a quarter: input column (tile's first column - pad + n) of the three input rows
         const int iyr = tile_y - p.pad, ixr = tile_x * 14 - p.pad + n;
         unsigned roff[3];
@@ -371,18 +477,26 @@ __global__ void __launch_bounds__(1024) tdc_conv3x3_stream_kernel(const ConvKPar
     f4_t acc = acc0 + acc1;
     // lane l holds rows 4*(l/16) .. +3 (output channels) of column l%16 (pixel); the slices of a channel block are
     // added by its first wave, in slice order
+    const int pp = oy * p.Wo + ox;
     if (p.WK > 1) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) lds[(wave * 4 + i) * 64 + lane] = acc[i];
         __syncthreads();
+        if constexpr (MODE == 0) {
+            if (p.WK >= 4) {
+                // the first four waves of a channel block share the final sum and the store: wave w finishes
+                // accumulator register w (output channel 4k + w of its lanes' pixels)
+                if (wki >= 4 || !live) return;
+                finish_one_channel(sum_slices(lds, wave - wki, p.WK, wki, lane), mblk * 16 + 4 * k + wki, p.N, p.P, pp, p.bias,
+                                   resid, p.relu, out);
+                return;
+            }
+        }
         if (wki == 0) {
-            acc = (f4_t){0.0f, 0.0f, 0.0f, 0.0f};
-            for (int w = 0; w < p.WK; ++w)
 #pragma unroll
-                for (int i = 0; i < 4; ++i) acc[i] += lds[((wave + w) * 4 + i) * 64 + lane];
+            for (int i = 0; i < 4; ++i) acc[i] = sum_slices(lds, wave, p.WK, i, lane);
         }
     }
-    const int pp = oy * p.Wo + ox;
     if constexpr (TAIL) {
         // Fused 1x1 tail, out2 = W2 * act(conv + bias): the workgroup owns every output channel of the convolution
         // (the host guarantees it).  The finished 16-pixel columns are parked in LDS as f[channel][pixel] — the B operand
@@ -621,12 +735,12 @@ static kernel_fn pick_stream(int nq) {
     }
 }
 
-template <bool ROW, int MODE>
+template <int INP, int MODE>
 static kernel_fn pick_stream3(int groups) {
     switch (groups) {
-        case 1: return tdc_conv3x3_stream_kernel<1, ROW, MODE>;
-        case 2: return tdc_conv3x3_stream_kernel<2, ROW, MODE>;
-        case 4: return tdc_conv3x3_stream_kernel<4, ROW, MODE>;
+        case 1: return tdc_conv3x3_stream_kernel<1, INP, MODE>;
+        case 2: return tdc_conv3x3_stream_kernel<2, INP, MODE>;
+        case 4: return tdc_conv3x3_stream_kernel<4, INP, MODE>;
         default: return nullptr;
     }
 }
@@ -650,9 +764,10 @@ const void *stream_kernel_function(const KernelId &k) {
         }
     } else if (k.family == KernelId::STREAM_3x3) {
         const int cg = k.p[0], mode = k.p[2];
-        if (k.p[1]) fn = mode == 2 ? pick_stream3<true, 2>(cg) : mode == 1 ? pick_stream3<true, 1>(cg) : mode == 0 ? pick_stream3<true, 0>(cg) : nullptr;
-        else fn = mode == 3 ? pick_stream3<false, 3>(cg) : mode == 2 ? pick_stream3<false, 2>(cg) : mode == 1 ? pick_stream3<false, 1>(cg)
-                : mode == 0 ? pick_stream3<false, 0>(cg) : nullptr;
+        if (k.p[1] == 2) fn = mode == 2 ? pick_stream3<2, 2>(cg) : mode == 1 ? pick_stream3<2, 1>(cg) : mode == 0 ? pick_stream3<2, 0>(cg) : nullptr;
+        else if (k.p[1] == 1) fn = mode == 2 ? pick_stream3<1, 2>(cg) : mode == 1 ? pick_stream3<1, 1>(cg) : mode == 0 ? pick_stream3<1, 0>(cg) : nullptr;
+        else fn = mode == 3 ? pick_stream3<0, 3>(cg) : mode == 2 ? pick_stream3<0, 2>(cg) : mode == 1 ? pick_stream3<0, 1>(cg)
+                : mode == 0 ? pick_stream3<0, 0>(cg) : nullptr;
     }
     return reinterpret_cast<const void *>(fn);
 }

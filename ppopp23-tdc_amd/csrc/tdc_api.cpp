@@ -603,6 +603,8 @@ static int forward_impl(tdc_conv_plan *plan, const float *d_in, int64_t in_batch
     kp.head_w = plan->d_head_w;
     kp.head_C = plan->head_C; kp.head_runs = plan->head_runs; kp.head_mblk = plan->head_mblk; kp.head_npb = plan->head_npb;
     kp.head_ww = plan->head_ww; kp.head_wq = plan->head_wq; kp.head_ld = plan->head_ld; kp.head_f_off = plan->head_f_off;
+    kp.win_rows = g.win_rows; kp.win_L = g.win_L; kp.win_nreq = g.win_nreq; kp.win_ns = g.win_ns; kp.win_off = g.win_off;
+    kp.fd_winL = make_fastdiv(std::max(g.win_L, 1));
     kp.fd_hww = make_fastdiv(std::max(plan->head_ww, 1));
     kp.fd_hnpb = make_fastdiv(std::max(plan->head_npb, 1));
     kp.fd_npx = make_fastdiv(g.PT / 16);
@@ -998,10 +1000,14 @@ int tdc_tkconv_create(const tdc_tkconv_desc *desc, tdc_tkconv **op_out) {
         // The first factor too, recomputed per workgroup on its window (streamed 3x3 kernel, stride 1).  Every
         // workgroup then pulls the whole first factor through its compute unit, so this only pays while that factor is
         // small: without measurement, up to 16 KiB of its weights and 64 input channels.
-        if (op->core_last && op->core_last->tile.alg == 4 && desc->K == 3 && desc->stride == 1 && desc->dilation == 1 &&
+        if (op->core_last && (op->core_last->tile.alg == 4 || op->core_last->tile.alg == 6) && desc->K == 3 && desc->stride == 1 && desc->dilation == 1 &&
             !std::getenv("TDC_EXPERIMENT_NO_FUSED_HEAD") &&
             (measure ? (long long)desc->C * desc->R1 <= 32768 : ((long long)desc->C * desc->R1 <= 4096 && desc->C <= 64))) {
-            st = tdc_conv_plan_create_with_tail(&d2, desc->N, desc->has_bias, desc->relu, &op->core_last->tile, &op->whole);
+            // (the same tile; the head's output is read from LDS, so a tile that passes its input window through LDS
+            //  becomes the plain streamed one)
+            tdc_tile head_tile = op->core_last->tile;
+            head_tile.alg = 4;
+            st = tdc_conv_plan_create_with_tail(&d2, desc->N, desc->has_bias, desc->relu, &head_tile, &op->whole);
             if (st == TDC_OK) {
                 const std::vector<float> zeros((size_t)desc->R1 * desc->C, 0.0f);
                 st = tdc_conv_plan_set_head(op->whole, desc->C, zeros.data());

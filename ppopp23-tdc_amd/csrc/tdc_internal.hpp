@@ -55,6 +55,10 @@ struct Geometry {
     int wslab_floats = 0;            // weights of one pass of one channel tile
     int aff_floats = 0;              // room for the scale/shift of an input affine (1x1 convolutions without padding)
     int tail_N = 0, tail_ng = 0, tail_ld = 0, tail_f_off = 0;   // fused 1x1 tail (0 = none)
+    // tile.alg = 6: the input window a wave leaves in its own piece of LDS — rows, 4-column segments per row, requests per
+    // group of channels (1 or 2), floats per channel (padded so that the four channel quarters fall into different banks),
+    // and where the pieces start (floats)
+    int win_rows = 0, win_L = 0, win_nreq = 0, win_ns = 0, win_off = 0;
     int stage_floats = 0;
     int nstage = 1;
     int lds_bytes = 0;
@@ -136,6 +140,8 @@ struct ConvKParams {
     int head_mblk, head_npb;   // ... 16-row blocks of its output (the core's input channels), 16-pixel blocks of the window
     int head_ww, head_wq;      // ... window width (TW + 2) and pixels ((TH + 2) * (TW + 2))
     int head_ld, head_f_off;   // ... row stride and offset (floats) of its output in LDS
+    int win_rows, win_L, win_nreq, win_ns, win_off;   // tile.alg = 6: the wave-private input window in LDS (see Geometry)
+    FastDiv fd_winL;
     FastDiv fd_hww, fd_hnpb;
     FastDiv fd_npx;            // 16-pixel blocks per tile
     FastDiv fd_csv, fd_rsv;      // LDS channel slot / row, in copy elements
@@ -159,7 +165,7 @@ enum : int { TAPS_GENERIC = 0, TAPS_1x1 = 1, TAPS_3x3 = 9, TAPS_3x3G = 10, TAPS_
 // launcher and the occupancy probe all speak of the same function.
 //   STAGED      tdc_conv_mfma_kernel<MF, MB, NB, TAPS, MAXW, EXT>     p = {MF, MB, NB, TAPS, MAXW, EXT}
 //   STREAM_1x1  tdc_conv1x1_stream_kernel<NQ, AFF, MODE>              p = {NQ, AFF, MODE}
-//   STREAM_3x3  tdc_conv3x3_stream_kernel<CG, ROW, MODE>              p = {CG, ROW, MODE, 1}
+//   STREAM_3x3  tdc_conv3x3_stream_kernel<CG, INP, MODE>              p = {CG, INP, MODE, 1}   (INP: 0 taps, 1 row shifts, 2 window in LDS)
 //               tdc_conv3x3_stream_rownb_kernel<CG, NB>               p = {CG, 1, 0, NB}   (NB = 2 or 4 pixel blocks per wave)
 //   STREAM_WINO tdc_wino3x3_stream_kernel<CG, MAXW>                   p = {CG, MAXW}
 struct KernelId {

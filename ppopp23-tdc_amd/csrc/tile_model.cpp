@@ -142,7 +142,7 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
     g.taps = d.KH * d.KW;
     g.ktaps = g.taps;
     g.MT = t.mf * t.mb * t.wm;
-    if (t.alg < 0 || t.alg > 5) return fail("tile.alg must be in [0, 5]");
+    if (t.alg < 0 || t.alg > 6) return fail("tile.alg must be in [0, 6]");
     if (t.alg == 5) {
         // Winograd F(2x2,3x3) streamed from global memory: 16*wm channels of one tile row block (2 rows x 28 columns) per
         // workgroup, the input channels split over wk waves in groups of four, everything in one pass
@@ -156,9 +156,11 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
         if (t.cch < d.C || t.cch - d.C >= t.cch / t.wk) return fail("tile.alg = 5 takes all input channels in one pass without an idle wave");
         if ((long long)t.cch * d.H * d.W * 4 >= (1LL << 31)) return fail("image too large for tile.alg = 5");
     }
-    if (t.alg == 4) {
+    if (t.alg == 6 && (t.nb != 1 || d.pad > 1 || d.stride > 2))
+        return fail("tile.alg = 6 needs nb = 1, pad <= 1 and stride <= 2");
+    if (t.alg == 4 || t.alg == 6) {
         // 3x3 convolution streamed from global memory: 16 channels x 16 pixels per workgroup, the input channels
-        // split over wk waves in groups of four, everything in one pass
+        // split over wk waves in groups of four, everything in one pass (alg 6: the tile's input window through LDS)
         if (d.KH != 3 || d.KW != 3 || d.dilation != 1) return fail("tile.alg = 4 needs a 3x3 / dilation 1 convolution");
         if (t.mf != 16 || t.mb != 1 || t.wn != 1) return fail("tile.alg = 4 needs mf = 16, mb = 1, wn = 1");
         if (t.nb != 1) {
@@ -223,7 +225,7 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
         if (t.tw < 1 || t.tw > g.PT || (!runs && t.tw > g.Wo)) return fail("tile.tw must be in [1, min(Wo, pixel lanes)]");
         g.TW = t.tw;
         g.TH = runs ? 1 : std::min(g.PT / t.tw, g.Ho);
-        if (t.alg == 4) g.TH = std::min(16 / t.tw, g.Ho);   // (a block is 16 pixel lanes, whatever nb is)
+        if (t.alg == 4 || t.alg == 6) g.TH = std::min(16 / t.tw, g.Ho);   // (a block is 16 pixel lanes, whatever nb is)
     }
     g.ntx = ceil_div(g.Wo, g.TW);
     if (t.alg == 4 && t.nb > 1) g.ntx = ceil_div(g.ntx, t.nb);   // a workgroup takes nb neighbouring tiles of a row
@@ -297,6 +299,20 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
         lds = std::max(lds, ((long long)g.tail_f_off + (long long)g.MT * g.tail_ld) * 4);
     }
     if (t.alg >= 3 && t.ks > 1) lds = std::max<long long>(lds, 16);   // the drawn ticket is passed through LDS
+    if (t.alg == 6) {
+        // The input window of a tile: (TH-1)*stride+3 rows; columns from the multiple of four at or left of the tile's first
+        // input column (up to three more than the (TW-1)*stride+3 the taps touch), in segments of four.  One slot per lane
+        // of a channel quarter and request.
+        g.win_rows = (g.TH - 1) * d.stride + 3;
+        g.win_L = ceil_div((g.TW - 1) * d.stride + 3 + 3, 4);
+        g.win_nreq = ceil_div(g.win_rows * g.win_L, 16);
+        if (g.win_nreq > 2) return fail("tile.alg = 6: the input window of this tile needs more than two requests per group");
+        if (d.W < 4) return fail("tile.alg = 6 needs an image at least four columns wide");
+        g.win_ns = g.win_rows * g.win_L * 4;
+        while (g.win_ns % 32 != 16) g.win_ns += 4;
+        g.win_off = (int)((lds + 15) / 16 * 4);
+        lds = (long long)g.win_off * 4 + (long long)g.waves * (t.cch / t.wk) * g.win_ns * 4;
+    }
     if (lds > machine().lds_bytes_per_cu) return fail("tile needs more than 160 KiB of LDS");
     g.lds_bytes = (int)lds;
     if (const char *e = std::getenv("TDC_EXPERIMENT_MIN_LDS")) g.lds_bytes = std::max(g.lds_bytes, std::atoi(e));
@@ -325,7 +341,7 @@ void pack_weights(const tdc_conv_desc &d, const tdc_tile &t, const Geometry &g, 
     const int ncg = t.cch / g.kc;
     const int taps = g.taps;
     float *dst = packed;
-    if (t.alg == 2 || t.alg == 4) {
+    if (t.alg == 2 || t.alg == 4 || t.alg == 6) {
         // per (channel tile, pass, M block, channel group): [taps 0-3][lane][4] [taps 4-7][lane][4] [tap 8][lane]
         for (int by = 0; by < g.grid_y; ++by)
             for (int chunk = 0; chunk < g.nchunks; ++chunk)
@@ -506,7 +522,7 @@ KernelId kernel_id_for(const tdc_tile &t, int KH, int KW, int dilation, int stri
         k.p[0] = cg; k.p[1] = maxw;
         return k;
     }
-    if (t.alg == 4) {
+    if (t.alg == 4 || t.alg == 6) {
         // (`extras` can only mean a fused tail here, which the one kernel carries)
         if (KH != 3 || KW != 3 || dilation != 1 || t.mf != 16 || t.mb != 1 || t.wm < 1 || t.wn != 1 || t.wk < 1 ||
             t.wm * t.wk > 16 || t.cch % (4 * t.wk) != 0)
@@ -516,11 +532,11 @@ KernelId kernel_id_for(const tdc_tile &t, int KH, int KW, int dilation, int stri
         const bool row = stride == 1 && t.tw == 14;   // one row of 14 pixels: the taps of a filter row are lane shifts
         if (t.nb != 1) {
             // several pixel blocks per wave: row tiles, no extras, no split across workgroups
-            if ((t.nb != 2 && t.nb != 4) || !row || extras || t.ks > 1) return k;
+            if ((t.nb != 2 && t.nb != 4) || !row || extras || t.ks > 1 || t.alg == 6) return k;
         }
         k.family = KernelId::STREAM_3x3;
         k.p[0] = cg;
-        k.p[1] = row;
+        k.p[1] = t.alg == 6 ? 2 : row;
         k.p[2] = extras ? 2 : t.ks > 1 ? 1 : 0;
         k.p[3] = t.nb;
         return k;
@@ -571,7 +587,7 @@ std::string kernel_name(const KernelId &k) {
             break;
         case KernelId::STREAM_3x3:
             if (k.p[3] > 1) std::snprintf(buf, sizeof buf, "tdc_conv3x3_stream_rownb_kernel<%d, %d>", k.p[0], k.p[3]);
-            else std::snprintf(buf, sizeof buf, "tdc_conv3x3_stream_kernel<%d, %s, %d>", k.p[0], tf[k.p[1] != 0], k.p[2]);
+            else std::snprintf(buf, sizeof buf, "tdc_conv3x3_stream_kernel<%d, %d, %d>", k.p[0], k.p[1], k.p[2]);
             break;
         case KernelId::STREAM_WINO:
             std::snprintf(buf, sizeof buf, "tdc_wino3x3_stream_kernel<%d, %d>", k.p[0], k.p[1]);
@@ -680,7 +696,7 @@ bool model_evaluate(const tdc_conv_desc &d, const tdc_tile &t, tdc_tile_info &in
             clk += rounds * (110.0 + 8.0 * t.wk) + out_bytes * r / 200.0;
             return clk;
         }
-        if (t.alg == 4) {
+        if (t.alg == 4 || t.alg == 6) {
             // as below; per input channel 576 bytes of weights and nine 64-byte rows of input (the rows of
             // neighbouring taps mostly hit in the L1, so they count for less than their size)
             const double chip_share =
@@ -691,13 +707,17 @@ bool model_evaluate(const tdc_conv_desc &d, const tdc_tile &t, tdc_tile_info &in
             const double rate = std::min(0.59 * MC.copy_bytes_per_clk, chip_share);
             const bool row_mode = d.stride == 1 && t.tw == 14;
             // (nb pixel blocks per wave: the input rows of every block, the weights once)
-            const double bytes = (double)t.cch * t.wm * (576.0 + t.nb * (row_mode ? 0.28 : 0.66) * 576.0) * r;
+            // (alg 6: the window of the tile once, 16 bytes per slot)
+            const double in_bytes_ch = t.alg == 6 ? 16.0 * g.win_rows * g.win_L : t.nb * (row_mode ? 0.28 : 0.66) * 576.0;
+            const double bytes = (double)t.cch * t.wm * (576.0 + in_bytes_ch) * r;
             const double groups = (double)t.cch / (4.0 * t.wk);
             const double waves_simd = std::ceil((double)g.waves * r / m.simds_per_cu);
             // a wave issues its requests one after the other (about 21 cycles each): fewer groups per wave start sooner
             // (288 cycles per group: a wave's own nine MFMAs per block run one after the other)
+            // (alg 6: one or two requests per group for the window, then its way through LDS: a write, nine reads)
+            const double in_requests = t.alg == 6 ? (double)g.win_nreq : t.nb * (row_mode ? 3.0 : 9.0);
             double clk = MC.stream_setup_clk + MC.stream_latency_clk + 288.0 * groups + 65.0 * (waves_simd - 1.0) + bytes / rate +
-                         groups * (3.0 + t.nb * (row_mode ? 3.0 : 9.0)) * 21.4;
+                         groups * (3.0 + in_requests) * 21.4 + (t.alg == 6 ? 150.0 + 40.0 * groups : 0.0);
             // the MFMAs of the extra blocks no longer hide under the requests: the matrix pipe of a SIMD serves its waves in turn
             if (t.nb > 1) {
                 clk += waves_simd * groups * 9.0 * (t.nb - 1) * mfma_clk;
@@ -844,6 +864,12 @@ std::vector<tdc_tile> model_enumerate(const tdc_conv_desc &d, int tail_N) {
                     if (!make_geometry(d, t, g, nullptr, tail_N)) continue;
                     if (ks > 1 && (long long)g.grid_x * g.grid_y * g.grid_z > 2LL * machine().cus) continue;
                     out.push_back(t);
+                    // the same tile with its input window loaded in 128-bit pieces and passed through LDS
+                    if (d.pad <= 1 && d.stride <= 2 && !std::getenv("TDC_EXPERIMENT_NO_STREAMED_WINDOW")) {
+                        tdc_tile t6 = t;
+                        t6.alg = 6;
+                        if (make_geometry(d, t6, g, nullptr, tail_N)) out.push_back(t6);
+                    }
                     // the same tile with 2 or 4 neighbouring 14-pixel row tiles per workgroup, sharing the weights in
                     // registers (where the image row has that many)
                     if (tw == 14 && d.stride == 1 && ks == 1 && tail_N == 0 && !std::getenv("TDC_EXPERIMENT_NO_STREAMED_NB"))

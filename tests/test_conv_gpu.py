@@ -183,7 +183,8 @@ def test_streamed_1x1_with_stride(shape, stride):
                                               ((3, 5, 3, 4, 3), 1, 0), ((1, 250, 17, 5, 5), 2, 1), ((2, 20, 33, 9, 58), 1, 1),
                                               ((1, 96, 40, 6, 30), 1, 1), ((1, 64, 48, 5, 56), 1, 0), ((1, 16, 20, 4, 44), 1, 1)])
 def test_every_streamed_3x3_tile(shape, stride, pad):
-    """The 3x3 path that streams both operands from global memory into registers (tile.alg = 4): every launchable tile
+    """The 3x3 path that streams both operands from global memory into registers (tile.alg = 4, and 6 with the input
+    window loaded in 128-bit pieces and passed through LDS): every launchable tile
     (1, 2 or 4 channel groups per wave, 1 to 16 waves, every shape of the 16-pixel tile; 2 or 4 neighbouring 14-pixel row
     tiles per workgroup where the rows are wide enough, including rows whose last workgroup has blocks past the image),
     stride 2, wide and no padding, ragged channel counts, batches; plain, and with bias + residual + ReLU written into a
@@ -197,10 +198,12 @@ def test_every_streamed_3x3_tile(shape, stride, pad):
     Ho, Wo = want.shape[2], want.shape[3]
     resid = torch.randn(B, N, Ho, Wo, generator=g)
     want_full = (torch.from_numpy(want) + bias.view(1, -1, 1, 1) + resid).clamp_min(0).numpy()
-    tiles = [t for t in tdc_amd.model_enumerate(tdc_amd.conv_desc(B, C, N, H, W, 3, 3, stride, pad)) if t.alg == 4]
+    tiles = [t for t in tdc_amd.model_enumerate(tdc_amd.conv_desc(B, C, N, H, W, 3, 3, stride, pad)) if t.alg in (4, 6)]
     assert tiles
     if stride == 1 and Wo > 14:
         assert {t.nb for t in tiles} == ({1, 2, 4} if Wo > 42 else {1, 2})
+    # (tile.alg = 6, the input window in 128-bit pieces through LDS, wherever padding and stride allow it and the image has four columns)
+    assert any(t.alg == 6 for t in tiles) == (pad <= 1 and W >= 4)
     for t in tiles:
         announce("streamed 3x3", shape, stride, pad, t)
         assert_close(run_conv(x, w, stride=stride, pad=pad, tile=t), want, f"{shape} s{stride} p{pad} {t}")
