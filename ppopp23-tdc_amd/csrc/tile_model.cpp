@@ -884,8 +884,11 @@ std::vector<tdc_tile> model_enumerate(const tdc_conv_desc &d, int tail_N) {
             }
         }
     }
-    // streamed Winograd candidates: 3x3 / stride 1 / pad 1, even width, all input channels in one pass
-    if (d.KH == 3 && d.KW == 3 && d.stride == 1 && d.dilation == 1 && d.pad == 1 && d.W % 2 == 0 && tail_N == 0 &&
+    // streamed Winograd candidates: 3x3 / stride 1 / pad 1, even width, all input channels in one pass.  Offered for single
+    // images only: the kernel is built for the latency of one small launch, and at batch 8 its timing alone misleads the
+    // measured selection (DenseNet-121's 64 -> 16 @56x56 core at batch 8: 6.9 us alone against 8.1 us for the staged
+    // Winograd tile, but the network ran 2.5 % slower with it); a forced tile still runs any batch.
+    if (d.batch == 1 && d.KH == 3 && d.KW == 3 && d.stride == 1 && d.dilation == 1 && d.pad == 1 && d.W % 2 == 0 && tail_N == 0 &&
         !std::getenv("TDC_EXPERIMENT_NO_STREAMED_WINOGRAD")) {
         const int groups_total = ceil_div(d.C, 4);
         for (int wm : {1, 2}) {

@@ -237,8 +237,9 @@ def test_every_streamed_winograd_tile(shape):
     want = ref.conv2d_c(x.numpy(), w.numpy(), stride=1, pad=1)
     resid = torch.randn(B, N, H, W, generator=g)
     want_full = (torch.from_numpy(want) + bias.view(1, -1, 1, 1) + resid).clamp_min(0).numpy()
-    tiles = [t for t in tdc_amd.model_enumerate(tdc_amd.conv_desc(B, C, N, H, W, 3, 3, 1, 1)) if t.alg == 5]
-    assert tiles
+    # (the enumeration offers these tiles for single images; forced, they run any batch)
+    tiles = [t for t in tdc_amd.model_enumerate(tdc_amd.conv_desc(1, C, N, H, W, 3, 3, 1, 1)) if t.alg == 5]
+    assert tiles and not any(t.alg == 5 for t in tdc_amd.model_enumerate(tdc_amd.conv_desc(2, C, N, H, W, 3, 3, 1, 1)))
     if C >= 16:
         assert len({t.cch // (4 * t.wk) for t in tiles}) >= 2
     for t in tiles:
