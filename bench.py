@@ -234,6 +234,12 @@ def main():
     # tdc_conv_forward launches on a stream (what a caller of the library does; it needs a host that issues a launch
     # in under ~4 us).  Which one the timed region uses is decided BEFORE it, from the warm-up steps of both; the
     # other is timed afterwards and reported beside it.
+    # (spin-up, untimed and not counted as warm-up steps: the same step for ~0.2 s, so that the W warm-up steps and the K
+    #  timed steps run at the clocks of a busy GPU; the parity checks above leave it idle for hundreds of milliseconds,
+    #  and with the driver's K = 20 the timed region is only 2.5 ms long)
+    t_spin = time.perf_counter()
+    while time.perf_counter() - t_spin < 0.2:
+        time_many_ms(plans, xs, outs, iters=50, graph=False)
     warm = {}
     for mode in ([True, False] if graph else [False]):
         time_many_ms(plans, xs, outs, iters=2, graph=mode)

@@ -578,7 +578,10 @@ __global__ void __launch_bounds__(1024) tdc_conv3x3_stream_kernel(const ConvKPar
 // of the WK waves meet in LDS as [wave][block][register][lane] and ALL threads share the final sum (in wave order, so
 // the result does not depend on timing) and the store.
 // ---------------------------------------------------------------------------
-template <int CG, int NB>
+// WIN (tile.alg = 6): the three input rows under all NB blocks — 14 NB + 2 columns, from the 4-column boundary at or left
+// of the first — come as two (NB = 2) or three (NB = 4) 128-bit requests per group of channels instead of 3 NB 32-bit
+// ones, through a wave-private piece of LDS, from which every lane reads the nine taps of each of its blocks.
+template <int CG, int NB, bool WIN>
 __global__ void __launch_bounds__(1024) tdc_conv3x3_stream_rownb_kernel(const ConvKParams p) {
     extern __shared__ __align__(16) float lds[];
     TDC_STAMP_DECL;
@@ -626,30 +629,88 @@ __global__ void __launch_bounds__(1024) tdc_conv3x3_stream_rownb_kernel(const Co
     const unsigned base = (unsigned)(wki * (4 * CG) + k) * chan_bytes;   // this lane's first channel
     // lane n of a quarter: input column (block's first column - pad + n) of the three input rows under the output row
     const int iyr = tile_y - p.pad;
-    unsigned roff[NB][3];
+    float rowv[WIN ? 1 : CG][NB][3];
+    float bwin[WIN ? CG : 1][NB][9];
+    if constexpr (WIN) {
+        // slot = row * win_L + segment of four columns from ixa on; lane n of a quarter takes slot q * 16 + n of its channel
+        constexpr int NREQ = NB == 2 ? 2 : 3;
+        const int L = p.win_L, NS = p.win_ns;
+        const int ixw0 = tile_x * NB * 14 - p.pad;
+        const int ixa = (ixw0 >> 2) << 2;                 // (arithmetic shift: floors negative columns too)
+        float *win = lds + p.win_off + wave * (CG * 4 * NS) + k * NS;     // this lane's channel of group 0
+        unsigned soff[NREQ];
+        int wslot[NREQ], ncol[NREQ];
 #pragma unroll
-    for (int blk = 0; blk < NB; ++blk) {
-        const int ixr = (tile_x * NB + blk) * 14 - p.pad + n;
-#pragma unroll
-        for (int r = 0; r < 3; ++r) {
-            const bool ok = (unsigned)(iyr + r) < (unsigned)p.H && (unsigned)ixr < (unsigned)p.W;
+        for (int q = 0; q < NREQ; ++q) {
+            const int slot = q * 16 + n;
+            const int row = fdiv(slot, p.fd_winL);
+            const int cs = ixa + 4 * (slot - row * L);
+            const bool ok = row < 3 && (unsigned)(iyr + row) < (unsigned)p.H && (unsigned)cs < (unsigned)p.W;
             const unsigned m = ok ? 0xffffffffu : 0u;
-            roff[blk][r] = ((unsigned)((iyr + r) * p.W + ixr) * 4u & m) | ((unsigned)OOB_OFFSET & ~m);
+            soff[q] = ((unsigned)((iyr + row) * p.W + cs) * 4u & m) | ((unsigned)OOB_OFFSET & ~m);
+            wslot[q] = row < 3 ? slot * 4 : -1;
+            ncol[q] = p.W - cs;
         }
+        f4_t wv[CG][NREQ];
+#pragma unroll
+        for (int g = 0; g < CG; ++g) {
+#pragma unroll
+            for (int q = 0; q < NREQ; ++q)
+                wv[g][q] = __builtin_bit_cast(f4_t, __builtin_amdgcn_raw_buffer_load_b128(
+                    in_rsrc, (int)(soff[q] + base + (unsigned)(4 * g) * chan_bytes), 0, 0));
+            __builtin_amdgcn_sched_barrier(0);   // requests in the order the MFMAs consume them
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        TDC_STAMP(1);   // every request issued
+#pragma unroll
+        for (int g = 0; g < CG; ++g)
+#pragma unroll
+            for (int q = 0; q < NREQ; ++q)
+                if (wslot[q] >= 0) {
+                    f4_t v = wv[g][q];
+#pragma unroll
+                    for (int e = 1; e < 4; ++e) v[e] = e < ncol[q] ? v[e] : 0.0f;
+                    *reinterpret_cast<f4_t *>(win + g * 4 * NS + wslot[q]) = v;
+                }
+        // (the lanes of a wave exchange data through LDS here: its LDS instructions complete in order, and nothing may be
+        //  moved across this point by the compiler)
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        const float *rd = win + min(n, 13) + (ixw0 - ixa);   // (lanes 14 and 15 of a block re-read pixel 13; never stored)
+#pragma unroll
+        for (int g = 0; g < CG; ++g)
+#pragma unroll
+            for (int blk = 0; blk < NB; ++blk)
+#pragma unroll
+                for (int r = 0; r < 3; ++r)
+#pragma unroll
+                    for (int c = 0; c < 3; ++c) bwin[g][blk][r * 3 + c] = rd[g * 4 * NS + r * (4 * L) + blk * 14 + c];
+    } else {
+        unsigned roff[NB][3];
+#pragma unroll
+        for (int blk = 0; blk < NB; ++blk) {
+            const int ixr = (tile_x * NB + blk) * 14 - p.pad + n;
+#pragma unroll
+            for (int r = 0; r < 3; ++r) {
+                const bool ok = (unsigned)(iyr + r) < (unsigned)p.H && (unsigned)ixr < (unsigned)p.W;
+                const unsigned m = ok ? 0xffffffffu : 0u;
+                roff[blk][r] = ((unsigned)((iyr + r) * p.W + ixr) * 4u & m) | ((unsigned)OOB_OFFSET & ~m);
+            }
+        }
+#pragma unroll
+        for (int g = 0; g < CG; ++g) {
+#pragma unroll
+            for (int blk = 0; blk < NB; ++blk)
+#pragma unroll
+                for (int r = 0; r < 3; ++r)
+                    rowv[g][blk][r] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                        in_rsrc, (int)(roff[blk][r] + base + (unsigned)(4 * g) * chan_bytes), 0, 0));
+            __builtin_amdgcn_sched_barrier(0);   // requests in the order the MFMAs consume them
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        TDC_STAMP(1);   // every request issued
     }
-    float rowv[CG][NB][3];
-#pragma unroll
-    for (int g = 0; g < CG; ++g) {
-#pragma unroll
-        for (int blk = 0; blk < NB; ++blk)
-#pragma unroll
-            for (int r = 0; r < 3; ++r)
-                rowv[g][blk][r] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
-                    in_rsrc, (int)(roff[blk][r] + base + (unsigned)(4 * g) * chan_bytes), 0, 0));
-        __builtin_amdgcn_sched_barrier(0);   // requests in the order the MFMAs consume them
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    TDC_STAMP(1);   // every request issued
     f4_t acc[NB];
 #pragma unroll
     for (int blk = 0; blk < NB; ++blk) acc[blk] = (f4_t){0.0f, 0.0f, 0.0f, 0.0f};
@@ -663,11 +724,16 @@ __global__ void __launch_bounds__(1024) tdc_conv3x3_stream_rownb_kernel(const Co
                 const float av = t < 4 ? a0[g][t] : t < 8 ? a1[g][t - 4] : a8[g];
 #pragma unroll
                 for (int blk = 0; blk < NB; ++blk) {
-                    const int v = __builtin_bit_cast(int, rowv[g][blk][r]);
-                    // row_shl:c within the 16 lanes of a quarter: lane n takes the value of lane n + c
-                    const float bv = c == 0 ? rowv[g][blk][r]
-                                   : c == 1 ? __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, v, 0x101, 0xf, 0xf, true))
-                                            : __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, v, 0x102, 0xf, 0xf, true));
+                    float bv;
+                    if constexpr (WIN) {
+                        bv = bwin[g][blk][t];
+                    } else {
+                        const int v = __builtin_bit_cast(int, rowv[g][blk][r]);
+                        // row_shl:c within the 16 lanes of a quarter: lane n takes the value of lane n + c
+                        bv = c == 0 ? rowv[g][blk][r]
+                           : c == 1 ? __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, v, 0x101, 0xf, 0xf, true))
+                                    : __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, v, 0x102, 0xf, 0xf, true));
+                    }
                     acc[blk] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, bv, acc[blk], 0, 0, 0);
                 }
             }
@@ -754,13 +820,19 @@ const void *stream_kernel_function(const KernelId &k) {
     } else if (k.family == KernelId::STREAM_3x3 && k.p[3] > 1) {
         // NB pixel blocks per wave: rows of 14 pixels, plain mode only
         const int cg = k.p[0], nb = k.p[3];
-        if (k.p[1] && k.p[2] == 0) {
-            if (nb == 2) fn = cg == 1 ? static_cast<kernel_fn>(tdc_conv3x3_stream_rownb_kernel<1, 2>)
-                            : cg == 2 ? static_cast<kernel_fn>(tdc_conv3x3_stream_rownb_kernel<2, 2>)
-                            : cg == 4 ? static_cast<kernel_fn>(tdc_conv3x3_stream_rownb_kernel<4, 2>) : nullptr;
-            if (nb == 4) fn = cg == 1 ? static_cast<kernel_fn>(tdc_conv3x3_stream_rownb_kernel<1, 4>)
-                            : cg == 2 ? static_cast<kernel_fn>(tdc_conv3x3_stream_rownb_kernel<2, 4>)
-                            : cg == 4 ? static_cast<kernel_fn>(tdc_conv3x3_stream_rownb_kernel<4, 4>) : nullptr;
+        if (k.p[1] == 1 && k.p[2] == 0) {
+            if (nb == 2) fn = cg == 1 ? static_cast<kernel_fn>(tdc_conv3x3_stream_rownb_kernel<1, 2, false>)
+                            : cg == 2 ? static_cast<kernel_fn>(tdc_conv3x3_stream_rownb_kernel<2, 2, false>)
+                            : cg == 4 ? static_cast<kernel_fn>(tdc_conv3x3_stream_rownb_kernel<4, 2, false>) : nullptr;
+            if (nb == 4) fn = cg == 1 ? static_cast<kernel_fn>(tdc_conv3x3_stream_rownb_kernel<1, 4, false>)
+                            : cg == 2 ? static_cast<kernel_fn>(tdc_conv3x3_stream_rownb_kernel<2, 4, false>)
+                            : cg == 4 ? static_cast<kernel_fn>(tdc_conv3x3_stream_rownb_kernel<4, 4, false>) : nullptr;
+        } else if (k.p[1] == 2 && k.p[2] == 0) {      // the rows of all blocks as one window through LDS
+            if (nb == 2) fn = cg == 1 ? static_cast<kernel_fn>(tdc_conv3x3_stream_rownb_kernel<1, 2, true>)
+                            : cg == 2 ? static_cast<kernel_fn>(tdc_conv3x3_stream_rownb_kernel<2, 2, true>)
+                            : cg == 4 ? static_cast<kernel_fn>(tdc_conv3x3_stream_rownb_kernel<4, 2, true>) : nullptr;
+            if (nb == 4) fn = cg == 1 ? static_cast<kernel_fn>(tdc_conv3x3_stream_rownb_kernel<1, 4, true>)
+                            : cg == 2 ? static_cast<kernel_fn>(tdc_conv3x3_stream_rownb_kernel<2, 4, true>) : nullptr;
         }
     } else if (k.family == KernelId::STREAM_3x3) {
         const int cg = k.p[0], mode = k.p[2];

@@ -114,7 +114,7 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
     };
     if (!check_desc(d, why)) return false;
     if (t.mf != 32 && t.mf != 16) return fail("tile.mf must be 16 or 32");
-    if (t.mb < 1 || t.mb > 2 || t.nb < 1 || (t.nb > 2 && !(t.alg == 4 && t.nb == 4)))
+    if (t.mb < 1 || t.mb > 2 || t.nb < 1 || (t.nb > 2 && !((t.alg == 4 || t.alg == 6) && t.nb == 4)))
         return fail("tile.mb / tile.nb must be 1 or 2 (tile.nb may be 4 for tile.alg = 4)");
     if (t.wm < 1 || t.wn < 1 || t.wk < 1) return fail("tile.wm / wn / wk must be >= 1");
     g = Geometry();
@@ -156,8 +156,8 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
         if (t.cch < d.C || t.cch - d.C >= t.cch / t.wk) return fail("tile.alg = 5 takes all input channels in one pass without an idle wave");
         if ((long long)t.cch * d.H * d.W * 4 >= (1LL << 31)) return fail("image too large for tile.alg = 5");
     }
-    if (t.alg == 6 && (t.nb != 1 || d.pad > 1 || d.stride > 2))
-        return fail("tile.alg = 6 needs nb = 1, pad <= 1 and stride <= 2");
+    if (t.alg == 6 && (d.pad > 1 || d.stride > 2)) return fail("tile.alg = 6 needs pad <= 1 and stride <= 2");
+    if (t.alg == 6 && t.nb == 4 && t.cch / std::max(t.wk, 1) > 8) return fail("tile.alg = 6 with nb = 4 takes at most two groups per wave");
     if (t.alg == 4 || t.alg == 6) {
         // 3x3 convolution streamed from global memory: 16 channels x 16 pixels per workgroup, the input channels
         // split over wk waves in groups of four, everything in one pass (alg 6: the tile's input window through LDS)
@@ -228,7 +228,7 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
         if (t.alg == 4 || t.alg == 6) g.TH = std::min(16 / t.tw, g.Ho);   // (a block is 16 pixel lanes, whatever nb is)
     }
     g.ntx = ceil_div(g.Wo, g.TW);
-    if (t.alg == 4 && t.nb > 1) g.ntx = ceil_div(g.ntx, t.nb);   // a workgroup takes nb neighbouring tiles of a row
+    if ((t.alg == 4 || t.alg == 6) && t.nb > 1) g.ntx = ceil_div(g.ntx, t.nb);   // a workgroup takes nb neighbouring tiles of a row
     g.nty = ceil_div(g.Ho, g.TH);
     if (t.alg == 3 && !flat) {
         g.ntx = ceil_div(g.P, 16);
@@ -283,7 +283,7 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
     const long long stage_bytes = (long long)g.nstage * g.stage_floats * 4;
     // (the Winograd path always parks its output tiles in LDS, also without a split over waves)
     // (... and so does the streamed 3x3 kernel with several pixel blocks per wave: all its threads share the final store)
-    const long long red_bytes = (t.wk > 1 || t.alg == 1 || t.alg == 5 || (t.alg == 4 && t.nb > 1)) ? (long long)t.wk * g.MT * g.PT * 4 : 0;
+    const long long red_bytes = (t.wk > 1 || t.alg == 1 || t.alg == 5 || ((t.alg == 4 || t.alg == 6) && t.nb > 1)) ? (long long)t.wk * g.MT * g.PT * 4 : 0;
     long long lds = std::max(stage_bytes, red_bytes);
     if (tail_N > 0) {
         // A fused 1x1 tail needs every output channel of the convolution in one workgroup; its tile is parked
@@ -304,9 +304,9 @@ bool make_geometry(const tdc_conv_desc &d, const tdc_tile &t, Geometry &g, std::
         // input column (up to three more than the (TW-1)*stride+3 the taps touch), in segments of four.  One slot per lane
         // of a channel quarter and request.
         g.win_rows = (g.TH - 1) * d.stride + 3;
-        g.win_L = ceil_div((g.TW - 1) * d.stride + 3 + 3, 4);
+        g.win_L = ceil_div((g.TW * t.nb - 1) * d.stride + 3 + 3, 4);   // (nb > 1: the blocks lie side by side in one window)
         g.win_nreq = ceil_div(g.win_rows * g.win_L, 16);
-        if (g.win_nreq > 2) return fail("tile.alg = 6: the input window of this tile needs more than two requests per group");
+        if (g.win_nreq > (t.nb == 4 ? 3 : 2)) return fail("tile.alg = 6: the input window of this tile needs too many requests per group");
         if (d.W < 4) return fail("tile.alg = 6 needs an image at least four columns wide");
         g.win_ns = g.win_rows * g.win_L * 4;
         while (g.win_ns % 32 != 16) g.win_ns += 4;
@@ -532,7 +532,8 @@ KernelId kernel_id_for(const tdc_tile &t, int KH, int KW, int dilation, int stri
         const bool row = stride == 1 && t.tw == 14;   // one row of 14 pixels: the taps of a filter row are lane shifts
         if (t.nb != 1) {
             // several pixel blocks per wave: row tiles, no extras, no split across workgroups
-            if ((t.nb != 2 && t.nb != 4) || !row || extras || t.ks > 1 || t.alg == 6) return k;
+            if ((t.nb != 2 && t.nb != 4) || !row || extras || t.ks > 1) return k;
+            if (t.alg == 6 && t.nb == 4 && cg == 4) return k;
         }
         k.family = KernelId::STREAM_3x3;
         k.p[0] = cg;
@@ -586,7 +587,7 @@ std::string kernel_name(const KernelId &k) {
             std::snprintf(buf, sizeof buf, "tdc_conv1x1_stream_kernel<%d, %s, %d>", k.p[0], tf[k.p[1] != 0], k.p[2]);
             break;
         case KernelId::STREAM_3x3:
-            if (k.p[3] > 1) std::snprintf(buf, sizeof buf, "tdc_conv3x3_stream_rownb_kernel<%d, %d>", k.p[0], k.p[3]);
+            if (k.p[3] > 1) std::snprintf(buf, sizeof buf, "tdc_conv3x3_stream_rownb_kernel<%d, %d, %s>", k.p[0], k.p[3], tf[k.p[1] == 2]);
             else std::snprintf(buf, sizeof buf, "tdc_conv3x3_stream_kernel<%d, %d, %d>", k.p[0], k.p[1], k.p[2]);
             break;
         case KernelId::STREAM_WINO:
@@ -708,7 +709,7 @@ bool model_evaluate(const tdc_conv_desc &d, const tdc_tile &t, tdc_tile_info &in
             const bool row_mode = d.stride == 1 && t.tw == 14;
             // (nb pixel blocks per wave: the input rows of every block, the weights once)
             // (alg 6: the window of the tile once, 16 bytes per slot)
-            const double in_bytes_ch = t.alg == 6 ? 16.0 * g.win_rows * g.win_L : t.nb * (row_mode ? 0.28 : 0.66) * 576.0;
+            const double in_bytes_ch = t.alg == 6 ? 16.0 * g.win_rows * g.win_L * 0.7 : t.nb * (row_mode ? 0.28 : 0.66) * 576.0;
             const double bytes = (double)t.cch * t.wm * (576.0 + in_bytes_ch) * r;
             const double groups = (double)t.cch / (4.0 * t.wk);
             const double waves_simd = std::ceil((double)g.waves * r / m.simds_per_cu);
@@ -717,7 +718,7 @@ bool model_evaluate(const tdc_conv_desc &d, const tdc_tile &t, tdc_tile_info &in
             // (alg 6: one or two requests per group for the window, then its way through LDS: a write, nine reads)
             const double in_requests = t.alg == 6 ? (double)g.win_nreq : t.nb * (row_mode ? 3.0 : 9.0);
             double clk = MC.stream_setup_clk + MC.stream_latency_clk + 288.0 * groups + 65.0 * (waves_simd - 1.0) + bytes / rate +
-                         groups * (3.0 + in_requests) * 21.4 + (t.alg == 6 ? 150.0 + 40.0 * groups : 0.0);
+                         groups * (3.0 + in_requests) * 21.4 + (t.alg == 6 ? 150.0 + 40.0 * groups * (t.nb > 1 ? 1.5 * t.nb : 1.0) : 0.0);
             // the MFMAs of the extra blocks no longer hide under the requests: the matrix pipe of a SIMD serves its waves in turn
             if (t.nb > 1) {
                 clk += waves_simd * groups * 9.0 * (t.nb - 1) * mfma_clk;
@@ -879,6 +880,14 @@ std::vector<tdc_tile> model_enumerate(const tdc_conv_desc &d, int tail_N) {
                             if (make_geometry(d, t, g, nullptr, 0) &&
                                 kernel_id_for(t, 3, 3, 1, 1, false).family != KernelId::NONE)
                                 out.push_back(t);
+                            // ... and with the rows of all blocks loaded as one window through LDS
+                            if (d.pad <= 1 && !std::getenv("TDC_EXPERIMENT_NO_STREAMED_WINDOW")) {
+                                tdc_tile t6 = t;
+                                t6.alg = 6;
+                                if (make_geometry(d, t6, g, nullptr, 0) &&
+                                    kernel_id_for(t6, 3, 3, 1, 1, false).family != KernelId::NONE)
+                                    out.push_back(t6);
+                            }
                         }
                 }
             }
