@@ -102,7 +102,7 @@ typedef struct tdc_tile {
                      5 = Winograd F(2x2,3x3) with BOTH operands read from global memory straight into registers
                          (3x3 / stride 1 / pad 1 / dilation 1, even image width): a workgroup owns 16 * wm channels of
                          one tile-row block (2 output rows x 28 columns, tw = 28), its wk waves split the input
-                         channels in groups of four, cch = 4 * wk * {1, 2, 3, 4} >= C (one pass; at most 16 / 16 / 16 / 12
+                         channels in groups of four, cch = 4 * wk * {1, 2, 3, 4} >= C (one pass; at most 16
                          waves per workgroup); the input rows are loaded as column pairs, once per lane, and the
                          patch columns a tile shares with its neighbours are lane shifts; mf = 16, mb = nb = wn = 1,
                          ks = 1, wl = 0.  No fused tail.

@@ -29,8 +29,12 @@ __device__ __forceinline__ float shl1(float v) {
     return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x101, 0xf, 0xf, true));
 }
 
+// Four groups per wave would need 142 registers per lane with everything requested up front; the operands of the third
+// and fourth group are requested when the first and second have been consumed instead, which keeps the kernel inside
+// the 128 registers that let two 8-wave workgroups share a compute unit.
 template <int CG, int MAXW>
 __global__ void __launch_bounds__(MAXW * 64) tdc_wino3x3_stream_kernel(const ConvKParams p) {
+    constexpr int NOW = CG < 4 ? CG : 2;   // groups requested before the first MFMA
     extern __shared__ __align__(16) float lds[];
     TDC_STAMP_DECL;
     TDC_STAMP(0);   // entry
@@ -85,13 +89,16 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_wino3x3_stream_kernel(const Con
         const unsigned m = ok ? 0xffffffffu : 0u;
         roff[r] = ((unsigned)((iy0 + r) * p.W + ix) * 4u & m) | ((unsigned)OOB_OFFSET & ~m);
     }
-#pragma unroll
-    for (int g = 0; g < CG; ++g) {
-        if (g > 0) load_weights(g);
+    auto load_input = [&](int g) {
 #pragma unroll
         for (int r = 0; r < 4; ++r)   // (the whole offset goes through the range-checked vector operand)
             xin[g][r] = __builtin_bit_cast(f2_t, __builtin_amdgcn_raw_buffer_load_b64(
                 in_rsrc, (int)(roff[r] + base + (unsigned)(4 * g) * chan_bytes), 0, 0));
+    };
+#pragma unroll
+    for (int g = 0; g < NOW; ++g) {
+        if (g > 0) load_weights(g);
+        load_input(g);
         __builtin_amdgcn_sched_barrier(0);   // requests in the order the MFMAs consume them
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -122,6 +129,11 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_wino3x3_stream_kernel(const Con
         for (int x = 0; x < 16; ++x)
             acc[x] = __builtin_amdgcn_mfma_f32_16x16x4f32(u[g][x >> 2][x & 3], v[x], acc[x], 0, 0, 0);
         __builtin_amdgcn_sched_barrier(0);   // group by group, as the data arrives
+        if (g + NOW < CG) {                  // this group's registers are free: request the group NOW further on
+            load_weights(g + NOW);
+            load_input(g + NOW);
+            __builtin_amdgcn_sched_barrier(0);
+        }
     }
     TDC_STAMP(4);   // MFMAs issued
     // Output transform Y = A^T M A, A^T = [1 1 1 0; 0 1 -1 -1], per accumulator register (= output channel); parked as
@@ -191,8 +203,8 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_wino3x3_stream_kernel(const Con
 }
 
 // ---------------------------------------------------------------------------
-// Instantiation table: KernelId{STREAM_WINO, {CG, MAXW}} -> function.  Up to three groups per wave are built for 16 waves
-// per workgroup (128 registers per lane), four for 12.
+// Instantiation table: KernelId{STREAM_WINO, {CG, MAXW}} -> function, all built for 16 waves per workgroup (128 registers
+// per lane).
 // ---------------------------------------------------------------------------
 typedef void (*kernel_fn)(const ConvKParams);
 
@@ -203,7 +215,7 @@ const void *wino_stream_kernel_function(const KernelId &k) {
         if (cg == 1 && maxw == 16) fn = tdc_wino3x3_stream_kernel<1, 16>;
         if (cg == 2 && maxw == 16) fn = tdc_wino3x3_stream_kernel<2, 16>;
         if (cg == 3 && maxw == 16) fn = tdc_wino3x3_stream_kernel<3, 16>;
-        if (cg == 4 && maxw == 12) fn = tdc_wino3x3_stream_kernel<4, 12>;
+        if (cg == 4 && maxw == 16) fn = tdc_wino3x3_stream_kernel<4, 16>;
     }
     return reinterpret_cast<const void *>(fn);
 }

@@ -507,7 +507,7 @@ KernelId kernel_id_with_head(const tdc_tile &t) {
     return k;
 }
 
-int wino_stream_max_waves(int groups) { return (groups >= 1 && groups <= 3) ? 16 : groups == 4 ? 12 : 0; }
+int wino_stream_max_waves(int groups) { return (groups >= 1 && groups <= 4) ? 16 : 0; }
 
 KernelId kernel_id_for(const tdc_tile &t, int KH, int KW, int dilation, int stride, bool extras) {
     KernelId k;

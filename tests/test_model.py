@@ -108,7 +108,7 @@ def test_streamed_winograd_tiles_only_where_they_apply():
                   (d, tdc_amd.Tile(16, 1, 1, 1, 1, 8, 64, 28, 2, 0, 5)),        # no split across workgroups
                   (d, tdc_amd.Tile(16, 1, 1, 1, 1, 8, 64, 28, 1, 2, 5)),        # no loader waves
                   (d, tdc_amd.Tile(16, 1, 1, 1, 2, 8, 64, 28, 1, 0, 5)),        # one block per wave set
-                  (d, tdc_amd.Tile(16, 1, 1, 4, 1, 4, 64, 28, 1, 0, 5)),        # four groups per wave: at most 12 waves
+                  (d, tdc_amd.Tile(16, 1, 1, 8, 1, 4, 64, 28, 1, 0, 5)),        # 32 waves
                   (conv3(64, 64, 7), tdc_amd.Tile(16, 1, 1, 1, 1, 8, 64, 28, 1, 0, 5)),                 # odd width
                   (conv3(64, 64, 56, stride=2), tdc_amd.Tile(16, 1, 1, 1, 1, 8, 64, 28, 1, 0, 5)),      # stride 2
                   (tdc_amd.conv_desc(1, 64, 64, 56, 56, 3, 3, 1, 0), tdc_amd.Tile(16, 1, 1, 1, 1, 8, 64, 28, 1, 0, 5)),     # pad 0
@@ -148,7 +148,9 @@ def test_winograd_tiles_only_where_the_algorithm_applies():
                  (conv3(64, 64, 28), tdc_amd.Tile(16, 1, 1, 1, 1, 4, 64, 7, 1, 0, 3))]:
         with pytest.raises(tdc_amd.TdcError):
             tdc_amd.model_evaluate(d, t)
-    assert tdc_amd.model_select(conv3(128, 128, 56)).tile.alg == 1
+    # (the staged Winograd tiles keep the large layers where the streamed one does not apply: batches, 112 x 112 images)
+    assert tdc_amd.model_select(tdc_amd.conv_desc(4, 128, 128, 56, 56, 3, 3, 1, 1)).tile.alg == 1
+    assert tdc_amd.model_select(conv3(128, 128, 56)).tile.alg == 5
     assert tdc_amd.model_select(conv3(32, 32, 14)).tile.alg != 1
     assert not any(t.alg == 1 for t in tdc_amd.model_enumerate(conv3(64, 64, 56, stride=2)))
 
