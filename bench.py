@@ -93,6 +93,8 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="issue launches on a plain stream instead of a HIP graph")
     ap.add_argument("--only-dominant", action="store_true",
                     help="profiling aid: launch only the dominant layer (128->128 @56), `steps` times, and exit")
+    ap.add_argument("--only-launch-floor", action="store_true",
+                    help="time only the launch path (empty and spinning kernels, stream launches and graph replay), for profiling")
     ap.add_argument("--only-e2e", action="store_true",
                     help="profiling aid: run only the end-to-end Tucker ResNet-18 forward, `steps` times, and exit")
     ap.add_argument("--e2e-batch", type=int, default=1, help="with --only-e2e: images per forward")
@@ -137,6 +139,18 @@ def main():
         for _ in range(5):
             dst.copy_(src)
         torch.cuda.synchronize()
+
+    def floor_leg(as_graph):
+        best = lambda **kw: min(launch_floor_us(launches=300, graph=as_graph, **kw) for _ in range(3))
+        empty = best(grid=256, block=512)
+        spins = {sp: best(grid=256, block=512, spin_us=sp) for sp in (1.0, 2.0, 4.0)}
+        return {"empty_kernel_us": round(empty, 3), "empty_kernel_1_workgroup_us": round(best(grid=1, block=64), 3),
+                "busy_1us": round(spins[1.0], 3), "busy_2us": round(spins[2.0], 3), "busy_4us": round(spins[4.0], 3),
+                # what a launch adds to a kernel long enough not to hide under the launch path
+                "overhead_beyond_duration_us": round(spins[4.0] - 4.0, 3)}
+    if a.only_launch_floor:
+        print(json.dumps({"only_launch_floor": True, "stream_launches": floor_leg(False), "graph_replay": floor_leg(True)}))
+        return
 
     if a.only_e2e:
         from tdc_amd import nets
@@ -280,14 +294,6 @@ def main():
     # -- the launch path by itself (tdc_launch_floor_time): dependent launches of a kernel with the same argument block
     #    that touches no memory, empty or with every wave busy for a set time; as stream launches (how the timed step is
     #    issued) and as one graph replay (how the per-layer `us` below are issued) -----------------------------------
-    def floor_leg(as_graph):
-        best = lambda **kw: min(launch_floor_us(launches=300, graph=as_graph, **kw) for _ in range(3))
-        empty = best(grid=256, block=512)
-        spins = {sp: best(grid=256, block=512, spin_us=sp) for sp in (1.0, 2.0, 4.0)}
-        return {"empty_kernel_us": round(empty, 3), "empty_kernel_1_workgroup_us": round(best(grid=1, block=64), 3),
-                "busy_1us": round(spins[1.0], 3), "busy_2us": round(spins[2.0], 3), "busy_4us": round(spins[4.0], 3),
-                # what a launch adds to a kernel long enough not to hide under the launch path
-                "overhead_beyond_duration_us": round(spins[4.0] - 4.0, 3)}
     floor_stream, floor_graph = floor_leg(False), floor_leg(True)
     layer_floor = (floor_graph if graph else floor_stream)["empty_kernel_us"]   # same launch mode as the per-layer `us`
 

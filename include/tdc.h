@@ -66,11 +66,12 @@ typedef struct tdc_conv_desc {
  * as many rows as fit in the workgroup's mf*nb*wn pixel lanes); its wm*wn*wk
  * computing wavefronts split output channels, pixels and input channels; input channels
  * are staged through LDS `cch` at a time, double-buffered (alg 0-2), or requested from
- * global memory into registers all at once (alg 3-4). */
+ * global memory into registers all at once (alg 3-6). */
 typedef struct tdc_tile {
     int32_t mf;   /* MFMA block edge: 32 (v_mfma_f32_32x32x2_f32) or 16 (16x16x4) */
     int32_t mb;   /* MFMA blocks per wave along output channels (1 or 2)        */
-    int32_t nb;   /* MFMA blocks per wave along pixels (1 or 2)                 */
+    int32_t nb;   /* MFMA blocks per wave along pixels (1 or 2; alg 4 and 6 also 4: the
+                     workgroup's tile is nb 16-pixel blocks side by side along a row)  */
     int32_t wm;   /* waves along output channels                               */
     int32_t wn;   /* waves along pixels                                        */
     int32_t wk;   /* waves along input channels (in-workgroup split-K)          */
@@ -105,8 +106,14 @@ typedef struct tdc_tile {
                          channels in groups of four, cch = 4 * wk * {1, 2, 3, 4} >= C (one pass; at most 16
                          waves per workgroup); the input rows are loaded as column pairs, once per lane, and the
                          patch columns a tile shares with its neighbours are lane shifts; mf = 16, mb = nb = wn = 1,
-                         ks = 1, wl = 0.  No fused tail.
-                     The model offers 3, 4 and 5 where launch and latency dominate (few channels or few pixels); the
+                         ks = 1, wl = 0.  No fused tail.  Offered for single images only (batch 1).
+                     6 = alg 4 with the input taken as a WINDOW: every lane requests 128-bit pieces of the input rows
+                         its workgroup's tile covers (two or three requests per channel instead of one per filter row
+                         or tap), the pieces cross a wave-private LDS buffer, and each lane reads its nine taps back
+                         from there.  3x3 / dilation 1, pad <= 1, stride <= 2; same shapes, cch / wk / ks rules and
+                         fused tail as alg 4 (nb = 4: at most two channel groups per wave).  The input base address
+                         and row pitch need not be 16-byte aligned: the requests are element-masked at the row ends.
+                     The model offers 3 to 6 where launch and latency dominate (few channels or few pixels); the
                      staged paths keep the layers whose operands are worth sharing through the LDS. */
 } tdc_tile;
 

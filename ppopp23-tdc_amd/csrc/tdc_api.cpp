@@ -47,6 +47,7 @@ struct tdc_conv_plan {
     tdc_tile_info info{};
     Geometry geo{};
     const void *kernel = nullptr;
+    void *kernel_handle = nullptr;   // the kernel's module function on the plan's device: what a forward launches
     float *d_wpk = nullptr;
     float *d_bias = nullptr;
     float *d_ws = nullptr;        // tile.ks > 1: partial tiles [batch][ks][N][P]
@@ -357,8 +358,8 @@ int tdc_conv_plan_create_with_tail(const tdc_conv_desc *desc, int32_t tail_N, in
     if (!make_geometry(*desc, p->tile, p->geo, &why, tail_N)) return fail(TDC_ERR_INVALID, why);
     p->kernel = conv_kernel_for(p->tile, desc->KH, desc->KW, desc->dilation, desc->stride, tail_N > 0);
     if (!p->kernel) return fail(TDC_ERR_UNSUPPORTED, "no kernel instantiated for this tile");
-    int he = prepare_conv_kernel(p->kernel, p->geo);
-    if (he) return hip_fail("hipFuncSetAttribute(MaxDynamicSharedMemorySize)", he);
+    int he = prepare_conv_kernel(p->kernel, p->geo, &p->kernel_handle);
+    if (he) return hip_fail("kernel set-up (hipFuncSetAttribute / hipGetFuncBySymbol)", he);
     const size_t wfloats = packed_weight_floats(p->geo);
     e = hipMalloc((void **)&p->d_wpk, wfloats * sizeof(float));
     if (e != hipSuccess) return hip_fail("hipMalloc(packed weights)", e);
@@ -465,7 +466,7 @@ int tdc_conv_plan_set_input_affine(tdc_conv_plan *plan, const float *scale, cons
     // from now on this plan needs the kernel instantiation that carries the extras
     plan->kernel = conv_kernel_for(plan->tile, d.KH, d.KW, d.dilation, d.stride, true);
     if (!plan->kernel) return fail(TDC_ERR_UNSUPPORTED, "no kernel instantiated for this tile");
-    if (int he = prepare_conv_kernel(plan->kernel, plan->geo)) return hip_fail("hipFuncSetAttribute(MaxDynamicSharedMemorySize)", he);
+    if (int he = prepare_conv_kernel(plan->kernel, plan->geo, &plan->kernel_handle)) return hip_fail("kernel set-up (hipFuncSetAttribute / hipGetFuncBySymbol)", he);
     plan->in_relu = relu != 0;
     return TDC_OK;
 }
@@ -507,7 +508,7 @@ int tdc_conv_plan_set_head(tdc_conv_plan *plan, int32_t head_C, const float *w_h
     g.lds_bytes = std::max(g.lds_bytes, (int)lds);
     plan->info.lds_bytes = g.lds_bytes;
     plan->kernel = kernel;
-    if (int he = prepare_conv_kernel(plan->kernel, g)) return hip_fail("hipFuncSetAttribute(MaxDynamicSharedMemorySize)", he);
+    if (int he = prepare_conv_kernel(plan->kernel, g, &plan->kernel_handle)) return hip_fail("kernel set-up (hipFuncSetAttribute / hipGetFuncBySymbol)", he);
     plan->head_C = head_C; plan->head_runs = runs; plan->head_mblk = mblk; plan->head_npb = npb;
     plan->head_ww = ww; plan->head_wq = wq; plan->head_ld = ld; plan->head_f_off = f_off;
     return TDC_OK;
@@ -650,7 +651,7 @@ static int forward_impl(tdc_conv_plan *plan, const float *d_in, int64_t in_batch
 #if defined(TDC_STAMPS) && TDC_STAMPS
     kp.stamps = plan->d_stamps;
 #endif
-    int he = launch_conv(plan->kernel, g, kp, stream);
+    int he = launch_conv(plan->kernel_handle, g, kp, stream);
     if (he) return hip_fail("kernel launch", he);
     return TDC_OK;
 }
@@ -777,6 +778,8 @@ int tdc_launch_floor_time(int32_t launches, int32_t use_graph, int32_t grid, int
     hipGraph_t graph = nullptr;
     hipGraphExec_t exec = nullptr;
     int he = 0;
+    void *probe = nullptr;
+    if (int pe = launch_floor_probe_handle(&probe)) return hip_fail("hipGetFuncBySymbol(launch probe)", pe);
     const char *what = "hipStreamCreate";
     hipError_t e = hipDeviceSynchronize();
     if (e == hipSuccess) e = hipStreamCreate(&s);
@@ -786,14 +789,14 @@ int tdc_launch_floor_time(int32_t launches, int32_t use_graph, int32_t grid, int
         what = "graph capture";
         e = hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal);
         if (e == hipSuccess) {
-            for (int i = 0; i < launches && !he; ++i) he = launch_floor_probe(kp, grid, block, ticks, s);
+            for (int i = 0; i < launches && !he; ++i) he = launch_floor_probe(probe, kp, grid, block, ticks, s);
             e = hipStreamEndCapture(s, &graph);
         }
         if (e == hipSuccess && !he) e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
         if (e == hipSuccess && !he) e = hipGraphLaunch(exec, s);   // untimed: upload
         if (e == hipSuccess && !he) e = hipStreamSynchronize(s);
     } else if (e == hipSuccess) {
-        for (int i = 0; i < 20 && !he; ++i) he = launch_floor_probe(kp, grid, block, ticks, s);   // untimed: warm-up
+        for (int i = 0; i < 20 && !he; ++i) he = launch_floor_probe(probe, kp, grid, block, ticks, s);   // untimed: warm-up
         e = hipStreamSynchronize(s);
     }
     if (e == hipSuccess && !he) {
@@ -802,7 +805,7 @@ int tdc_launch_floor_time(int32_t launches, int32_t use_graph, int32_t grid, int
         if (use_graph) {
             if (e == hipSuccess) e = hipGraphLaunch(exec, s);
         } else {
-            for (int i = 0; i < launches && !he; ++i) he = launch_floor_probe(kp, grid, block, ticks, s);
+            for (int i = 0; i < launches && !he; ++i) he = launch_floor_probe(probe, kp, grid, block, ticks, s);
         }
         if (e == hipSuccess) e = hipEventRecord(e1, s);
         if (e == hipSuccess) e = hipEventSynchronize(e1);

@@ -196,10 +196,11 @@ inline const void *conv_kernel_for(const tdc_tile &t, int KH, int KW, int dilati
     return kernel_function(kernel_id_for(t, KH, KW, dilation, stride, extras));
 }
 inline const void *conv_kernel_with_head(const tdc_tile &t) { return kernel_function(kernel_id_with_head(t)); }
-// One-time per-plan attribute setup (dynamic LDS above 64 KiB).  hipError_t as int.
-int prepare_conv_kernel(const void *fn, const Geometry &g);
+// One-time per-plan set-up: the dynamic-LDS attribute (above 64 KiB) and the kernel's module function handle on the
+// current device, which launch_conv launches.  hipError_t as int.
+int prepare_conv_kernel(const void *fn, const Geometry &g, void **handle_out);
 // Enqueue the kernel.  Returns a hipError_t as int.
-int launch_conv(const void *fn, const Geometry &g, const ConvKParams &kp, void *stream);
+int launch_conv(void *handle, const Geometry &g, const ConvKParams &kp, void *stream);
 
 // Static scratch (a device array that lives from module load to process exit, one copy per GPU) for the partial
 // tiles and ticket counters of a split across workgroups, for callers that cannot allocate.  The address is the
@@ -211,7 +212,8 @@ int static_scratch_address(void **ptr_out);
 int launch_zero_words(unsigned *dst, int n, void *stream);
 // Launch-path probe: a kernel with the convolution kernels' argument block whose waves spin for `spin_ticks` ticks of
 // the 100 MHz constant clock and touch no memory.
-int launch_floor_probe(const ConvKParams &kp, int grid, int block, int spin_ticks, void *stream);
+int launch_floor_probe_handle(void **handle_out);
+int launch_floor_probe(void *handle, const ConvKParams &kp, int grid, int block, int spin_ticks, void *stream);
 // What the compiled kernel really uses: registers per lane, static LDS, its launch bound, and how many workgroups
 // of `block_threads` threads with `dynamic_lds_bytes` of LDS the runtime places on one compute unit.
 int kernel_resources(const void *fn, int block_threads, int dynamic_lds_bytes, int *vgprs, int *static_lds, int *max_threads,

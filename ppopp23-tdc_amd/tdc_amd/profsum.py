@@ -7,6 +7,7 @@ geometry (grid, workgroup, LDS) is what tells the layers apart.
     python -m tdc_amd.profsum kernel <dir-with-*_kernel_trace.csv>
     python -m tdc_amd.profsum pmc    <dir-with-*_counter_collection.csv> [--copy-bytes N]
     python -m tdc_amd.profsum timeline <dir-with-*_kernel_trace.csv> --last N
+    python -m tdc_amd.profsum bursts <dir-with-*_kernel_trace.csv>
     python -m tdc_amd.profsum isolated <dir-with-*_kernel_trace.csv> --layers <output of bench.py --isolated-layers>
     python -m tdc_amd.profsum isolated-pmc <dir,dir,...> --layers <output of bench.py --isolated-layers> [--copy-bytes N]
 
@@ -16,6 +17,8 @@ WRITE_SIZE readings (KiB) of every kernel are also shown scaled by the reading o
 copy kernel in the same run, which is known to read and write N bytes.
 ``timeline``: the last N dispatches of the trace in launch order (one forward of a network of N kernels):
 start offset, duration, and the idle gap since the previous kernel ended.
+``bursts``: dispatches per kernel, launch geometry and duration class (nearest 0.5 us): launches, duration
+statistics and the median start-to-start interval under the tracer.
 ``isolated``: median / p10 kernel duration per benchmark layer from a trace of ``bench.py --isolated-layers``.
 ``isolated-pmc``: counters per benchmark layer from ``--pmc`` runs of the same command (one directory per counter set).
 """
@@ -32,6 +35,11 @@ import sys
 def _short(name):
     name = name.replace("void tdc::", "").replace("(tdc::ConvKParams)", "")
     return name if len(name) <= 60 else name[:57] + "..."
+
+
+def _is_conv(name):
+    """A dispatch of one of the convolution kernels (staged, streamed, streamed Winograd)."""
+    return "tdc_conv" in name or "tdc_wino" in name
 
 
 def kernel_summary(path, out=sys.stdout):
@@ -107,6 +115,39 @@ def timeline(path, last, out=sys.stdout):
         len(rows), (prev_end - t0) * 1e-3, busy, idle))
 
 
+def bursts(path, out=sys.stdout, min_len=20):
+    """Dispatches grouped by kernel, launch geometry and duration class (nearest half microsecond): what loops of
+    dependent launches of one kernel with different run times (the launch probe with its spin times) look like in a
+    trace.  The duration is the kernel alone; the start-to-start interval (median over the class, to the previous
+    dispatch in the trace) is the launch-to-launch time UNDER THE TRACER, which serialises dispatches."""
+    files = sorted(glob.glob(os.path.join(path, "**", "*kernel_trace.csv"), recursive=True))
+    if not files:
+        raise SystemExit(f"no *kernel_trace.csv under {path}")
+    rows = []
+    for f in files:
+        rows += list(csv.DictReader(open(f)))
+    rows.sort(key=lambda r: int(r["Start_Timestamp"]))
+    acc = collections.defaultdict(lambda: ([], []))
+    prev = None
+    for r in rows:
+        d = (int(r["End_Timestamp"]) - int(r["Start_Timestamp"])) * 1e-3
+        key = (_short(r["Kernel_Name"]), int(r["Grid_Size_X"]), int(r["Workgroup_Size_X"]), round(d * 2.0) / 2.0)
+        acc[key][0].append(d)
+        if prev is not None:
+            acc[key][1].append((int(r["Start_Timestamp"]) - prev) * 1e-3)
+        prev = int(r["Start_Timestamp"])
+    out.write("%-52s %9s %5s %6s %8s %9s %9s %9s %9s %15s\n" % ("kernel", "grid_x", "wg", "class", "launches", "mean_dur",
+                                                               "p10_dur", "median", "p90_dur", "start_to_start"))
+    for (name, gx, wg, cls), (d, gaps) in sorted(acc.items()):
+        if len(d) < min_len:
+            continue
+        d.sort()
+        gaps.sort()
+        out.write("%-52s %9d %5d %6.1f %8d %9.3f %9.3f %9.3f %9.3f %15.3f\n" % (
+            name[:52], gx, wg, cls, len(d), sum(d) / len(d), d[len(d) // 10], d[len(d) // 2], d[(9 * len(d)) // 10],
+            gaps[len(gaps) // 2] if gaps else float("nan")))
+
+
 def isolated(path, layers_json, out=sys.stdout):
     """Kernel-only durations per layer from a trace of ``bench.py --isolated-layers`` (every launch followed by a stream
     synchronisation, so a kernel's start-to-end time contains no other kernel): the last (layers x launches)
@@ -123,7 +164,7 @@ def isolated(path, layers_json, out=sys.stdout):
     files = sorted(glob.glob(os.path.join(path, "**", "*kernel_trace.csv"), recursive=True))
     rows = []
     for f in files:
-        rows += [r for r in csv.DictReader(open(f)) if "tdc_conv" in r["Kernel_Name"]]
+        rows += [r for r in csv.DictReader(open(f)) if _is_conv(r["Kernel_Name"])]
     rows.sort(key=lambda r: int(r["Start_Timestamp"]))
     need = per * len(info["layers"])
     if len(rows) < need:
@@ -168,7 +209,7 @@ def isolated_pmc(paths, layers_json, copy_bytes=None, out=sys.stdout):
         for f in files:
             for r in csv.DictReader(open(f)):
                 name = _short(r["Kernel_Name"])
-                if "tdc_conv" in name:
+                if _is_conv(name):
                     disp.setdefault(int(r["Dispatch_Id"]), (name, {}))[1][r["Counter_Name"]] = float(r["Counter_Value"])
                 elif "copy" in name.lower() and r["Counter_Name"] in ("FETCH_SIZE", "WRITE_SIZE"):
                     copies[r["Counter_Name"]] = max(copies[r["Counter_Name"]], float(r["Counter_Value"]))
@@ -211,7 +252,7 @@ def isolated_pmc(paths, layers_json, copy_bytes=None, out=sys.stdout):
 
 def main(argv=None):
     ap = argparse.ArgumentParser()
-    ap.add_argument("mode", choices=["kernel", "pmc", "timeline", "isolated", "isolated-pmc"])
+    ap.add_argument("mode", choices=["kernel", "pmc", "timeline", "bursts", "isolated", "isolated-pmc"])
     ap.add_argument("path")
     ap.add_argument("--copy-bytes", type=int, default=None)
     ap.add_argument("--layers", default=None, help="isolated: file holding the JSON line bench.py --isolated-layers printed")
@@ -229,6 +270,8 @@ def main(argv=None):
         kernel_summary(a.path)
     elif a.mode == "timeline":
         timeline(a.path, a.last)
+    elif a.mode == "bursts":
+        bursts(a.path)
     else:
         pmc_summary(a.path, a.copy_bytes)
 
