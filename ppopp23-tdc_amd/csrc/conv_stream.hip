@@ -243,7 +243,10 @@ template <int CG, int INP, int MODE>
 __global__ void __launch_bounds__(1024) tdc_conv3x3_stream_kernel(const ConvKParams p) {
     constexpr bool SPLIT = MODE == 1, TAIL = MODE == 2 || MODE == 3, HEAD = MODE == 3, ROW = INP == 1, WINDOW = INP == 2;
     extern __shared__ __align__(16) float lds[];
+    TDC_STAMP_DECL;
+    TDC_STAMP(0);   // entry
     touch_kernel_arguments();
+    TDC_STAMP(7);   // every line of the kernel arguments is in the scalar cache
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -463,6 +466,7 @@ __global__ void __launch_bounds__(1024) tdc_conv3x3_stream_kernel(const ConvKPar
         }
     }
     __builtin_amdgcn_sched_barrier(0);
+    TDC_STAMP(1);   // every request issued (window form: the input has crossed the LDS)
     f4_t acc0 = (f4_t){0.0f, 0.0f, 0.0f, 0.0f}, acc1 = (f4_t){0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
     for (int g = 0; g < CG; ++g) {
@@ -475,6 +479,7 @@ __global__ void __launch_bounds__(1024) tdc_conv3x3_stream_kernel(const ConvKPar
         __builtin_amdgcn_sched_barrier(0);   // group by group, as the data arrives
     }
     f4_t acc = acc0 + acc1;
+    TDC_STAMP(4);   // MFMAs issued (the last results may still be in the pipe)
     // lane l holds rows 4*(l/16) .. +3 (output channels) of column l%16 (pixel); the slices of a channel block are
     // added by its first wave, in slice order
     const int pp = oy * p.Wo + ox;
@@ -482,13 +487,16 @@ __global__ void __launch_bounds__(1024) tdc_conv3x3_stream_kernel(const ConvKPar
 #pragma unroll
         for (int i = 0; i < 4; ++i) lds[(wave * 4 + i) * 64 + lane] = acc[i];
         __syncthreads();
+        TDC_STAMP(5);   // everybody's partial blocks are in LDS
         if constexpr (MODE == 0) {
             if (p.WK >= 4) {
                 // the first four waves of a channel block share the final sum and the store: wave w finishes
                 // accumulator register w (output channel 4k + w of its lanes' pixels)
-                if (wki >= 4 || !live) return;
-                finish_one_channel(sum_slices(lds, wave - wki, p.WK, wki, lane), mblk * 16 + 4 * k + wki, p.N, p.P, pp, p.bias,
-                                   resid, p.relu, out);
+                if (wki < 4 && live)
+                    finish_one_channel(sum_slices(lds, wave - wki, p.WK, wki, lane), mblk * 16 + 4 * k + wki, p.N, p.P, pp,
+                                       p.bias, resid, p.relu, out);
+                TDC_STAMP(6);   // stores issued
+                TDC_STAMP_FLUSH(p, logical, wave, lane);
                 return;
             }
         }
@@ -563,8 +571,9 @@ __global__ void __launch_bounds__(1024) tdc_conv3x3_stream_kernel(const ConvKPar
     if constexpr (SPLIT) {
         if (!stream_join_slices(p, lds, acc, wki == 0 && live, mblk * 16 + 4 * k, pp, img, slice, by, bx)) return;
     }
-    if (wki != 0 || !live) return;
-    finish_four_channels(acc, mblk * 16 + 4 * k, p.N, p.P, pp, p.bias, resid, p.relu, out);
+    if (wki == 0 && live) finish_four_channels(acc, mblk * 16 + 4 * k, p.N, p.P, pp, p.bias, resid, p.relu, out);
+    TDC_STAMP(6);   // stores issued
+    TDC_STAMP_FLUSH(p, logical, wave, lane);
 }
 
 // ---------------------------------------------------------------------------
