@@ -120,7 +120,7 @@ __device__ __forceinline__ void finish_four_channels(const f4_t &acc, int ch0, i
     }
 }
 
-// The kernel arguments (about 400 bytes) are read through the scalar cache.  Left alone, the compiler fetches them in
+// The kernel arguments (about 530 bytes) are read through the scalar cache.  Left alone, the compiler fetches them in
 // several dependent batches, and every batch that touches a cache line for the first time costs a round trip to L2
 // before the first request can go out.  Touch every line of the argument block at once: whatever order the compiler
 // then loads the values in, it hits the scalar cache.
@@ -137,6 +137,25 @@ __device__ __forceinline__ void touch_kernel_arguments() {
             : "s"(kargs)
             : "memory");
     }
+}
+
+// Where image `img` of the batch starts in the input, the output and the residual.  A compute unit has ONE scalar
+// unit for all its waves, and in the streamed kernels every wave's scalar prologue sits on the path to its first
+// memory request (16 waves x ~130 scalar instructions is most of a microsecond), so the 64-bit stride products — a
+// quarter of that prologue — are skipped for the first image, which is the only one in a single-image launch.
+struct ImageBase {
+    const float *in;
+    float *out;
+    const float *resid;
+};
+__device__ __forceinline__ ImageBase image_base(const ConvKParams &p, int img) {
+    ImageBase b{p.in, p.out, p.resid};
+    if (__builtin_expect(img != 0, 0)) {   // (wave-uniform: a scalar branch)
+        b.in += (long long)img * p.in_bstride;
+        b.out += (long long)img * p.out_bstride;
+        if (b.resid) b.resid += (long long)img * p.resid_bstride;
+    }
+    return b;
 }
 
 }  // namespace tdc

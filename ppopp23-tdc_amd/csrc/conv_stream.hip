@@ -129,9 +129,10 @@ __global__ void __launch_bounds__(NQ == 8 ? 512 : 1024) tdc_conv1x1_stream_kerne
     const int KS = SPLIT ? p.KS : 1;
     const int bx = p.channel_major ? r1 : r2;  // pixel block
     const int by = p.channel_major ? r2 : r1;  // channel block
-    const float *__restrict__ in = p.in + (long long)img * p.in_bstride;
-    float *__restrict__ out = p.out + (long long)img * p.out_bstride;
-    const float *__restrict__ resid = p.resid ? p.resid + (long long)img * p.resid_bstride : nullptr;
+    const ImageBase image = image_base(p, img);
+    const float *__restrict__ in = image.in;
+    float *__restrict__ out = image.out;
+    const float *__restrict__ resid = image.resid;
     const __amdgpu_buffer_rsrc_t in_rsrc =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(in), (short)0, (int)p.in_image_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t w_rsrc =
@@ -263,9 +264,10 @@ __global__ void __launch_bounds__(1024) tdc_conv3x3_stream_kernel(const ConvKPar
     const int by = p.channel_major ? r2 : r1;  // channel block
     const int tile_y = fdiv(bx, p.fd_ntx);
     const int tile_x = bx - tile_y * p.ntx;
-    const float *__restrict__ in = p.in + (long long)img * p.in_bstride;
-    float *__restrict__ out = p.out + (long long)img * p.out_bstride;
-    const float *__restrict__ resid = p.resid ? p.resid + (long long)img * p.resid_bstride : nullptr;
+    const ImageBase image = image_base(p, img);
+    const float *__restrict__ in = image.in;
+    float *__restrict__ out = image.out;
+    const float *__restrict__ resid = image.resid;
     const __amdgpu_buffer_rsrc_t in_rsrc =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(in), (short)0, (int)p.in_image_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t w_rsrc =
@@ -610,9 +612,10 @@ __global__ void __launch_bounds__(1024) tdc_conv3x3_stream_rownb_kernel(const Co
     const int by = p.channel_major ? r2 : r1;  // channel tile
     const int tile_y = fdiv(bx, p.fd_ntx);     // = output row (tiles are one row high)
     const int tile_x = bx - tile_y * p.ntx;
-    const float *__restrict__ in = p.in + (long long)img * p.in_bstride;
-    float *__restrict__ out = p.out + (long long)img * p.out_bstride;
-    const float *__restrict__ resid = p.resid ? p.resid + (long long)img * p.resid_bstride : nullptr;
+    const ImageBase image = image_base(p, img);
+    const float *__restrict__ in = image.in;
+    float *__restrict__ out = image.out;
+    const float *__restrict__ resid = image.resid;
     const __amdgpu_buffer_rsrc_t in_rsrc =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(in), (short)0, (int)p.in_image_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t w_rsrc =

@@ -53,9 +53,10 @@ __global__ void __launch_bounds__(MAXW * 64) tdc_wino3x3_stream_kernel(const Con
     const int by = p.channel_major ? r2 : r1;  // channel tile
     const int tile_y = fdiv(bx, p.fd_ntx);     // tile row: output rows 2*tile_y, 2*tile_y + 1
     const int tile_x = bx - tile_y * p.ntx;    // block of 28 output columns in that row
-    const float *__restrict__ in = p.in + (long long)img * p.in_bstride;
-    float *__restrict__ out = p.out + (long long)img * p.out_bstride;
-    const float *__restrict__ resid = p.resid ? p.resid + (long long)img * p.resid_bstride : nullptr;
+    const ImageBase image = image_base(p, img);
+    const float *__restrict__ in = image.in;
+    float *__restrict__ out = image.out;
+    const float *__restrict__ resid = image.resid;
     const __amdgpu_buffer_rsrc_t in_rsrc =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(in), (short)0, (int)p.in_image_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t w_rsrc =
