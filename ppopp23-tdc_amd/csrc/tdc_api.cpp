@@ -62,6 +62,11 @@ struct tdc_conv_plan {
     bool have_tail_weights = false;
     int in_relu = 0;
     bool have_weights = false;
+    // The kernel arguments of a launch, but for what a call brings (buffers, batch strides, copy width): built when the
+    // plan is created and again whenever a setter changes what they depend on, so that a forward copies and patches
+    // them instead of recomputing two dozen divisions — host time per launch is what bounds small back-to-back kernels.
+    ConvKParams kp{};
+    FastDiv fd_csv1{}, fd_rsv1{};   // the two arguments that differ when the input is copied with 4-byte elements
 #if defined(TDC_STAMPS) && TDC_STAMPS
     unsigned long long *d_stamps = nullptr;   // profiling build: per-wave time stamps of the last launch
     size_t stamp_words = 0;
@@ -323,6 +328,66 @@ int tdc_set_autotune(int32_t classes) {
 
 int tdc_get_autotune(void) { return g_autotune.load(); }
 
+// Everything in the kernel arguments that the plan fixes (see tdc_conv_plan::kp).
+static void refresh_launch_params(tdc_conv_plan *plan) {
+    const tdc_conv_desc &d = plan->desc;
+    const Geometry &g = plan->geo;
+    ConvKParams kp{};
+    kp.wpk = plan->d_wpk;
+    kp.bias = plan->d_bias;
+    kp.in_aff = plan->d_in_aff;
+    kp.tail_w = plan->tail_N > 0 ? plan->d_tail_w : nullptr;
+    kp.tail_bias = plan->d_tail_bias;
+    kp.tail_N = plan->tail_N; kp.tail_mblk = (plan->tail_N + 15) / 16; kp.tail_ng = g.tail_ng; kp.tail_relu = plan->tail_relu;
+    kp.tail_ld = g.tail_ld; kp.tail_f_off = g.tail_f_off;
+    kp.head_w = plan->d_head_w;
+    kp.head_C = plan->head_C; kp.head_runs = plan->head_runs; kp.head_mblk = plan->head_mblk; kp.head_npb = plan->head_npb;
+    kp.head_ww = plan->head_ww; kp.head_wq = plan->head_wq; kp.head_ld = plan->head_ld; kp.head_f_off = plan->head_f_off;
+    kp.win_rows = g.win_rows; kp.win_L = g.win_L; kp.win_nreq = g.win_nreq; kp.win_ns = g.win_ns; kp.win_off = g.win_off;
+    kp.fd_winL = make_fastdiv(std::max(g.win_L, 1));
+    kp.fd_hww = make_fastdiv(std::max(plan->head_ww, 1));
+    kp.fd_hnpb = make_fastdiv(std::max(plan->head_npb, 1));
+    kp.fd_npx = make_fastdiv(g.PT / 16);
+    kp.in_relu = plan->in_relu;
+    const long long in_image = (long long)(plan->head_C > 0 ? plan->head_C : d.C) * d.H * d.W;
+    kp.in_image_bytes = (unsigned)(in_image * 4);
+    kp.C = d.C; kp.H = g.He; kp.W = g.We; kp.N = d.N;
+    kp.Ho = g.Ho; kp.Wo = g.Wo; kp.P = g.P;
+    kp.KH = d.KH; kp.KW = d.KW; kp.stride = d.stride; kp.pad = d.pad; kp.dil = d.dilation;
+    kp.TW = g.TW; kp.TH = g.TH; kp.ntx = g.ntx;
+    kp.WM = plan->tile.wm; kp.WN = plan->tile.wn; kp.WK = plan->tile.wk;
+    kp.CCH = plan->tile.cch; kp.nchunks = g.nchunks; kp.CPW = g.cpw;
+    kp.KS = g.ks; kp.cps = g.cps; kp.WL = plan->tile.wl;
+    kp.RS = g.RS; kp.CS = g.CS; kp.nrows = g.nrows;
+    kp.VW = g.VW;   // (a forward falls back to 4-byte copy elements when its input is not 16-byte aligned)
+    kp.in_stage_floats = g.in_stage_floats; kp.wslab_floats = g.wslab_floats;
+    kp.in_nblk = g.in_stage_floats / (64 * g.VW);
+    kp.stage_floats = g.stage_floats; kp.nstage = g.nstage;
+    kp.relu = d.relu;
+    kp.fd_csv = make_fastdiv(g.CS / g.VW);
+    kp.fd_rsv = make_fastdiv(g.RS / g.VW);
+    plan->fd_csv1 = make_fastdiv(g.CS);
+    plan->fd_rsv1 = make_fastdiv(g.RS);
+    kp.fd_tw = make_fastdiv(g.TW);
+    kp.fd_ntx = make_fastdiv(g.ntx);
+    kp.fd_pt = make_fastdiv(g.PT);
+    kp.fd_wtw = make_fastdiv(g.wino ? g.TWt : (plan->tile.alg == 3 && d.stride > 1) ? g.Wo : 1);
+    kp.fd_wk = make_fastdiv(plan->tile.wk);
+    kp.fd_wn = make_fastdiv(plan->tile.wn);
+    kp.fd_ks = make_fastdiv(g.ks);
+    kp.grid_x = g.grid_x; kp.grid_y = g.grid_y;
+    kp.n_wg = g.grid_x * g.grid_y * g.grid_z;
+    kp.xcd_chunk = (kp.n_wg + 7) / 8;
+    kp.channel_major = g.channel_major;
+    kp.fd_g1 = make_fastdiv(g.channel_major ? g.grid_x : g.grid_y);
+    kp.fd_g2 = make_fastdiv(g.channel_major ? g.grid_y : g.grid_x);
+    kp.wpk_bytes = (unsigned)(packed_weight_floats(g) * sizeof(float));
+#if defined(TDC_STAMPS) && TDC_STAMPS
+    kp.stamps = plan->d_stamps;
+#endif
+    plan->kp = kp;
+}
+
 int tdc_conv_plan_create(const tdc_conv_desc *desc, const tdc_tile *forced_tile, tdc_conv_plan **plan_out) {
     return tdc_conv_plan_create_with_tail(desc, 0, 0, 0, forced_tile, plan_out);
 }
@@ -399,6 +464,7 @@ int tdc_conv_plan_create_with_tail(const tdc_conv_desc *desc, int32_t tail_N, in
         return hip_fail("hipMalloc(time stamps)", e);
     }
 #endif
+    refresh_launch_params(p.get());
     *plan_out = p.release();
     return TDC_OK;
 }
@@ -468,6 +534,7 @@ int tdc_conv_plan_set_input_affine(tdc_conv_plan *plan, const float *scale, cons
     if (!plan->kernel) return fail(TDC_ERR_UNSUPPORTED, "no kernel instantiated for this tile");
     if (int he = prepare_conv_kernel(plan->kernel, plan->geo, &plan->kernel_handle)) return hip_fail("kernel set-up (hipFuncSetAttribute / hipGetFuncBySymbol)", he);
     plan->in_relu = relu != 0;
+    refresh_launch_params(plan);
     return TDC_OK;
 }
 
@@ -511,6 +578,7 @@ int tdc_conv_plan_set_head(tdc_conv_plan *plan, int32_t head_C, const float *w_h
     if (int he = prepare_conv_kernel(plan->kernel, g, &plan->kernel_handle)) return hip_fail("kernel set-up (hipFuncSetAttribute / hipGetFuncBySymbol)", he);
     plan->head_C = head_C; plan->head_runs = runs; plan->head_mblk = mblk; plan->head_npb = npb;
     plan->head_ww = ww; plan->head_wq = wq; plan->head_ld = ld; plan->head_f_off = f_off;
+    refresh_launch_params(plan);
     return TDC_OK;
 }
 
@@ -591,66 +659,22 @@ static int forward_impl(tdc_conv_plan *plan, const float *d_in, int64_t in_batch
     if ((in_batch_stride && in_batch_stride < in_image) || (out_batch_stride && out_batch_stride < out_image) ||
         (residual_batch_stride && residual_batch_stride < out_image))
         return fail(TDC_ERR_INVALID, "batch stride smaller than one image");
-    ConvKParams kp{};
+    ConvKParams kp = plan->kp;
     kp.in = d_in;
-    kp.wpk = plan->d_wpk;
-    kp.bias = plan->d_bias;
     kp.resid = d_residual;
     kp.out = d_out;
     kp.ws = ws;
-    kp.in_aff = plan->d_in_aff;
-    kp.tail_w = plan->tail_N > 0 ? plan->d_tail_w : nullptr;
-    kp.tail_bias = plan->d_tail_bias;
-    kp.tail_N = plan->tail_N; kp.tail_mblk = (plan->tail_N + 15) / 16; kp.tail_ng = g.tail_ng; kp.tail_relu = plan->tail_relu;
-    kp.tail_ld = g.tail_ld; kp.tail_f_off = g.tail_f_off;
-    kp.head_w = plan->d_head_w;
-    kp.head_C = plan->head_C; kp.head_runs = plan->head_runs; kp.head_mblk = plan->head_mblk; kp.head_npb = plan->head_npb;
-    kp.head_ww = plan->head_ww; kp.head_wq = plan->head_wq; kp.head_ld = plan->head_ld; kp.head_f_off = plan->head_f_off;
-    kp.win_rows = g.win_rows; kp.win_L = g.win_L; kp.win_nreq = g.win_nreq; kp.win_ns = g.win_ns; kp.win_off = g.win_off;
-    kp.fd_winL = make_fastdiv(std::max(g.win_L, 1));
-    kp.fd_hww = make_fastdiv(std::max(plan->head_ww, 1));
-    kp.fd_hnpb = make_fastdiv(std::max(plan->head_npb, 1));
-    kp.fd_npx = make_fastdiv(g.PT / 16);
-    kp.in_relu = plan->in_relu;
     kp.ctr = ctr;
-    kp.in_image_bytes = (unsigned)(in_image * 4);
     kp.in_bstride = in_batch_stride ? in_batch_stride : in_image;
     kp.out_bstride = out_batch_stride ? out_batch_stride : out_image;
     kp.resid_bstride = residual_batch_stride ? residual_batch_stride : out_image;
-    kp.C = d.C; kp.H = g.He; kp.W = g.We; kp.N = d.N;
-    kp.Ho = g.Ho; kp.Wo = g.Wo; kp.P = g.P;
-    kp.KH = d.KH; kp.KW = d.KW; kp.stride = d.stride; kp.pad = d.pad; kp.dil = d.dilation;
-    kp.TW = g.TW; kp.TH = g.TH; kp.ntx = g.ntx;
-    kp.WM = plan->tile.wm; kp.WN = plan->tile.wn; kp.WK = plan->tile.wk;
-    kp.CCH = plan->tile.cch; kp.nchunks = g.nchunks; kp.CPW = g.cpw;
-    kp.KS = g.ks; kp.cps = g.cps; kp.WL = plan->tile.wl;
-    kp.RS = g.RS; kp.CS = g.CS; kp.nrows = g.nrows;
     // 16-byte copy elements need every image of the batch 16-byte aligned; otherwise 4-byte elements.
-    const bool aligned = reinterpret_cast<uintptr_t>(d_in) % 16 == 0 && kp.in_bstride % 4 == 0;
-    kp.VW = (g.VW == 4 && aligned) ? 4 : 1;
-    kp.in_stage_floats = g.in_stage_floats; kp.wslab_floats = g.wslab_floats;
-    kp.in_nblk = g.in_stage_floats / (64 * kp.VW);   // (kp.VW: the element width this launch really copies with)
-    kp.stage_floats = g.stage_floats; kp.nstage = g.nstage;
-    kp.relu = d.relu;
-    kp.fd_csv = make_fastdiv(g.CS / kp.VW);
-    kp.fd_rsv = make_fastdiv(g.RS / kp.VW);
-    kp.fd_tw = make_fastdiv(g.TW);
-    kp.fd_ntx = make_fastdiv(g.ntx);
-    kp.fd_pt = make_fastdiv(g.PT);
-    kp.fd_wtw = make_fastdiv(g.wino ? g.TWt : (plan->tile.alg == 3 && d.stride > 1) ? g.Wo : 1);
-    kp.fd_wk = make_fastdiv(plan->tile.wk);
-    kp.fd_wn = make_fastdiv(plan->tile.wn);
-    kp.fd_ks = make_fastdiv(g.ks);
-    kp.grid_x = g.grid_x; kp.grid_y = g.grid_y;
-    kp.n_wg = g.grid_x * g.grid_y * g.grid_z;
-    kp.xcd_chunk = (kp.n_wg + 7) / 8;
-    kp.channel_major = g.channel_major;
-    kp.fd_g1 = make_fastdiv(g.channel_major ? g.grid_x : g.grid_y);
-    kp.fd_g2 = make_fastdiv(g.channel_major ? g.grid_y : g.grid_x);
-    kp.wpk_bytes = (unsigned)(packed_weight_floats(g) * sizeof(float));
-#if defined(TDC_STAMPS) && TDC_STAMPS
-    kp.stamps = plan->d_stamps;
-#endif
+    if (g.VW == 4 && !(reinterpret_cast<uintptr_t>(d_in) % 16 == 0 && kp.in_bstride % 4 == 0)) {
+        kp.VW = 1;
+        kp.in_nblk = g.in_stage_floats / 64;   // (copy blocks of the element width this launch really copies with)
+        kp.fd_csv = plan->fd_csv1;
+        kp.fd_rsv = plan->fd_rsv1;
+    }
     int he = launch_conv(plan->kernel_handle, g, kp, stream);
     if (he) return hip_fail("kernel launch", he);
     return TDC_OK;
