@@ -113,7 +113,10 @@ template <int NQ, bool AFF, int MODE>
 __global__ void __launch_bounds__(NQ == 8 ? 512 : 1024) tdc_conv1x1_stream_kernel(const ConvKParams p) {
     constexpr bool SPLIT = MODE == 1, STRIDED = MODE == 2;
     extern __shared__ __align__(16) float lds[];
+    TDC_STAMP_DECL;
+    TDC_STAMP(0);   // entry
     touch_kernel_arguments();
+    TDC_STAMP(7);   // every line of the kernel arguments is in the scalar cache
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // = this wave's slice of the input channels
@@ -172,6 +175,7 @@ __global__ void __launch_bounds__(NQ == 8 ? 512 : 1024) tdc_conv1x1_stream_kerne
     }
     // (every request is issued before the first MFMA: the scheduler must not sink loads into the MFMA sequence)
     __builtin_amdgcn_sched_barrier(0);
+    TDC_STAMP(1);   // every request issued
     // two accumulator chains: consecutive MFMAs do not wait for each other's result
     f4_t acc0 = (f4_t){0.0f, 0.0f, 0.0f, 0.0f}, acc1 = (f4_t){0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
@@ -189,18 +193,22 @@ __global__ void __launch_bounds__(NQ == 8 ? 512 : 1024) tdc_conv1x1_stream_kerne
         __builtin_amdgcn_sched_barrier(0);   // run by run, as the data arrives
     }
     f4_t acc = acc0 + acc1;
+    TDC_STAMP(4);   // MFMAs issued (the last results may still be in the pipe)
     // lane l holds rows 4*(l/16) .. +3 (output channels) of column l%16 (pixel)
     if (p.WK > 1) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) lds[(wave * 4 + i) * 64 + lane] = acc[i];
         __syncthreads();
+        TDC_STAMP(5);   // everybody's partial blocks are in LDS
         if constexpr (!SPLIT) {
             if (p.WK >= 4) {
                 // the first four waves share the final sum and the store: wave w finishes accumulator register w
                 // (output channel 4k + w of its lanes' pixels)
-                if (wave >= 4 || px >= p.P) return;
-                finish_one_channel(sum_slices(lds, 0, p.WK, wave, lane), by * 16 + 4 * k + wave, p.N, p.P, px, p.bias, resid,
-                                   p.relu, out);
+                if (wave < 4 && px < p.P)
+                    finish_one_channel(sum_slices(lds, 0, p.WK, wave, lane), by * 16 + 4 * k + wave, p.N, p.P, px, p.bias,
+                                       resid, p.relu, out);
+                TDC_STAMP(6);   // stores issued
+                TDC_STAMP_FLUSH(p, logical, wave, lane);
                 return;
             }
         }
@@ -213,8 +221,9 @@ __global__ void __launch_bounds__(NQ == 8 ? 512 : 1024) tdc_conv1x1_stream_kerne
         // the input channels are split over KS workgroups: whoever finishes last adds the partial blocks in slice order
         if (!stream_join_slices(p, lds, acc, wave == 0 && px < p.P, by * 16 + 4 * k, px, img, slice, by, bx)) return;
     }
-    if (wave != 0 || px >= p.P) return;
-    finish_four_channels(acc, by * 16 + 4 * k, p.N, p.P, px, p.bias, resid, p.relu, out);
+    if (wave == 0 && px < p.P) finish_four_channels(acc, by * 16 + 4 * k, p.N, p.P, px, p.bias, resid, p.relu, out);
+    TDC_STAMP(6);   // stores issued
+    TDC_STAMP_FLUSH(p, logical, wave, lane);
 }
 
 // ---------------------------------------------------------------------------

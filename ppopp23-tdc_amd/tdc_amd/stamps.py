@@ -1,11 +1,12 @@
 """Per-wave time line of one convolution launch, from the time stamps of the PROFILING build of the library.
 
     make -C ppopp23-tdc_amd/csrc STAMPS=1 OUT=/tmp/tdc_stamps/libtdc_amd.so OBJDIR=/tmp/tdc_stamps/build RESOURCES=/dev/null all
-    TDC_AMD_LIBRARY=/tmp/tdc_stamps/libtdc_amd.so python -m tdc_amd.stamps C,N,HW mf,mb,nb,wm,wn,wk,cch,tw,ks,wl,alg [tile ...]
+    TDC_AMD_LIBRARY=/tmp/tdc_stamps/libtdc_amd.so python -m tdc_amd.stamps C,N,HW[,K] mf,mb,nb,wm,wn,wk,cch,tw,ks,wl,alg [tile ...]
 
-(from ppopp23-tdc_amd, or with it on PYTHONPATH).  The profiling build compiles s_memrealtime reads (the 100 MHz
-constant clock: 10 ns per tick) into the staged kernel's Winograd path and into the streamed 3x3 kernel with several
-pixel blocks per wave, at the phase boundaries
+(from ppopp23-tdc_amd, or with it on PYTHONPATH; K = 3 (default: 3x3, pad 1) or 1 (1x1, pad 0)).  The profiling build
+compiles s_memrealtime reads (the 100 MHz constant clock: 10 ns per tick) into the staged kernel's Winograd path and into
+the streamed kernels (1x1, 3x3, 3x3 with several pixel blocks per wave, Winograd; these have no pass loop and take stamps
+0, 1, 4, 5, 6, 7 only), at the phase boundaries
 
     0 entry   1 every operand request of the first pass issued   2 this wave's copies landed   3 barrier: all landed
     4 multiply loop done   5 partial results parked in LDS, barrier   6 output stores issued   7 kernel arguments cached
@@ -28,12 +29,12 @@ PHASES = ["entry -> requests issued", "issued -> mine landed", "mine landed -> b
           "park in LDS + barrier", "store issue"]
 
 
-def timeline(c, n, hw, tile_text):
+def timeline(c, n, hw, tile_text, k=3):
     v = [int(a) for a in tile_text.split(",")]
     tile = tdc_amd.Tile(*v[:8], ks=v[8], wl=v[9], alg=v[10])
     gen = torch.Generator().manual_seed(7)
     x = torch.randn(1, c, hw, hw, generator=gen)
-    w = torch.randn(n, c, 3, 3, generator=gen) * (2.0 / (9 * c)) ** 0.5
+    w = torch.randn(n, c, k, k, generator=gen) * (2.0 / (k * k * c)) ** 0.5
     xd = x.cuda()
     out = torch.empty(1, n, hw, hw, device="cuda")
     lib = tdc_amd.lib()
@@ -41,7 +42,7 @@ def timeline(c, n, hw, tile_text):
         sys.exit("this library has no time stamps: build it with STAMPS=1 and point TDC_AMD_LIBRARY at it")
     lib.tdc_debug_read_stamps.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint64,
                                           ctypes.POINTER(ctypes.c_uint64)]
-    plan = Conv2dPlan(1, c, n, hw, hw, 3, 3, 1, 1, tile=tile).set_weights(w)
+    plan = Conv2dPlan(1, c, n, hw, hw, k, k, 1, k // 2, tile=tile).set_weights(w)
     us = min(plan.time_us(xd, out, iters=100) for _ in range(3))
     for _ in range(5):   # isolated launches; the stamps of the last one are read
         plan.forward(xd, out=out)
@@ -56,8 +57,8 @@ def timeline(c, n, hw, tile_text):
     st = s[live]                       # [waves, 8]
     t0 = st[:, 0].min()
     rel = (st - t0) * 0.01             # microseconds
-    print("== %d->%d @%d tile %s: %.2f us back to back; %d waves of %d workgroups stamped"
-          % (c, n, hw, tile_text, us, int(live.sum()), s.shape[0]))
+    print("== %d->%d @%d %s tile %s: %.2f us back to back; %d waves of %d workgroups stamped"
+          % (c, n, hw, "1x1" if k == 1 else "3x3", tile_text, us, int(live.sum()), s.shape[0]))
     print("   kernel span (first entry -> last store issue): %.2f us; entries spread over %.2f us"
           % (rel[:, 6].max(), rel[:, 0].max()))
     for i, name in enumerate(PHASES):
@@ -92,9 +93,13 @@ def timeline(c, n, hw, tile_text):
 def main():
     if len(sys.argv) < 3:
         sys.exit(__doc__)
-    c, n, hw = (int(v) for v in sys.argv[1].split(","))
+    shape = [int(v) for v in sys.argv[1].split(",")]
+    c, n, hw = shape[:3]
+    k = shape[3] if len(shape) > 3 else 3
+    if k not in (1, 3):
+        sys.exit("K must be 1 or 3")
     for tile_text in sys.argv[2:]:
-        timeline(c, n, hw, tile_text)
+        timeline(c, n, hw, tile_text, k)
 
 
 if __name__ == "__main__":
