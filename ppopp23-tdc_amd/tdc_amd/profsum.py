@@ -7,7 +7,7 @@ geometry (grid, workgroup, LDS) is what tells the layers apart.
     python -m tdc_amd.profsum kernel <dir-with-*_kernel_trace.csv>
     python -m tdc_amd.profsum pmc    <dir-with-*_counter_collection.csv> [--copy-bytes N]
     python -m tdc_amd.profsum timeline <dir-with-*_kernel_trace.csv> --last N
-    python -m tdc_amd.profsum bursts <dir-with-*_kernel_trace.csv>
+    python -m tdc_amd.profsum durations <dir-with-*_kernel_trace.csv>
     python -m tdc_amd.profsum isolated <dir-with-*_kernel_trace.csv> --layers <output of bench.py --isolated-layers>
     python -m tdc_amd.profsum isolated-pmc <dir,dir,...> --layers <output of bench.py --isolated-layers> [--copy-bytes N]
 
@@ -17,7 +17,7 @@ WRITE_SIZE readings (KiB) of every kernel are also shown scaled by the reading o
 copy kernel in the same run, which is known to read and write N bytes.
 ``timeline``: the last N dispatches of the trace in launch order (one forward of a network of N kernels):
 start offset, duration, and the idle gap since the previous kernel ended.
-``bursts``: dispatches per kernel, launch geometry and duration class (nearest 0.5 us): launches, duration
+``durations``: dispatches per kernel, launch geometry and duration class (nearest 0.5 us): launches, duration
 statistics and the median start-to-start interval under the tracer.
 ``isolated``: median / p10 kernel duration per benchmark layer from a trace of ``bench.py --isolated-layers``.
 ``isolated-pmc``: counters per benchmark layer from ``--pmc`` runs of the same command (one directory per counter set).
@@ -115,7 +115,7 @@ def timeline(path, last, out=sys.stdout):
         len(rows), (prev_end - t0) * 1e-3, busy, idle))
 
 
-def bursts(path, out=sys.stdout, min_len=20):
+def duration_classes(path, out=sys.stdout, min_len=20):
     """Dispatches grouped by kernel, launch geometry and duration class (nearest half microsecond): what loops of
     dependent launches of one kernel with different run times (the launch probe with its spin times) look like in a
     trace.  The duration is the kernel alone; the start-to-start interval (median over the class, to the previous
@@ -252,7 +252,7 @@ def isolated_pmc(paths, layers_json, copy_bytes=None, out=sys.stdout):
 
 def main(argv=None):
     ap = argparse.ArgumentParser()
-    ap.add_argument("mode", choices=["kernel", "pmc", "timeline", "bursts", "isolated", "isolated-pmc"])
+    ap.add_argument("mode", choices=["kernel", "pmc", "timeline", "durations", "isolated", "isolated-pmc"])
     ap.add_argument("path")
     ap.add_argument("--copy-bytes", type=int, default=None)
     ap.add_argument("--layers", default=None, help="isolated: file holding the JSON line bench.py --isolated-layers printed")
@@ -270,8 +270,8 @@ def main(argv=None):
         kernel_summary(a.path)
     elif a.mode == "timeline":
         timeline(a.path, a.last)
-    elif a.mode == "bursts":
-        bursts(a.path)
+    elif a.mode == "durations":
+        duration_classes(a.path)
     else:
         pmc_summary(a.path, a.copy_bytes)
 
