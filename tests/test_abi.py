@@ -84,6 +84,20 @@ def test_plan_creation_without_a_gpu_fails_loudly():
     assert b"HIP device" in tdc_amd.lib().tdc_last_error_string()
 
 
+def test_launch_floor_probe_rejects_bad_arguments():
+    """tdc_launch_floor_time checks its arguments before it touches the device."""
+    import ctypes
+    L = tdc_amd.lib()
+    ms = ctypes.c_float(-1.0)
+    for launches, graph, grid, block, spin in ((0, 0, 256, 512, 0.0), (300, 0, 0, 512, 0.0), (300, 0, 70000, 512, 0.0),
+                                                (300, 0, 256, 100, 0.0), (300, 0, 256, 2048, 0.0), (300, 1, 256, 512, -1.0),
+                                                (300, 0, 256, 512, 1000.0), (300, 0, 256, 512, float("nan"))):
+        st = L.tdc_launch_floor_time(launches, graph, grid, block, ctypes.c_float(spin), ctypes.byref(ms))
+        assert st == tdc_amd._lib.TDC_ERR_INVALID, (launches, graph, grid, block, spin, st)
+    assert L.tdc_launch_floor_time(300, 0, 256, 512, ctypes.c_float(0.0), None) == tdc_amd._lib.TDC_ERR_INVALID
+    assert ms.value == -1.0
+
+
 def test_python_operator_argument_errors_match_the_reference():
     """groups != 1 and non-zero padding modes are rejected like TKConv2dC.__init__ (inference/TKConv.py:39-42)."""
     hp = tdc_amd.ranks_dict(conv=[4, 3])

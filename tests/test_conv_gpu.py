@@ -886,6 +886,17 @@ def test_linearity_full_size():
     np.testing.assert_allclose(y, 0.5 * y1 + y2, rtol=1e-4, atol=2e-5)
 
 
+def test_launch_floor_probe():
+    """The launch-path probe: an empty kernel costs something, a kernel that keeps every wave busy for 5 us costs at
+    least those 5 us per launch and not much more, on a stream and inside a graph."""
+    from tdc_amd.conv import launch_floor_us
+    for graph in (False, True):
+        empty = min(launch_floor_us(launches=200, graph=graph) for _ in range(3))
+        busy = min(launch_floor_us(launches=200, graph=graph, spin_us=5.0) for _ in range(3))
+        assert 0.3 < empty < 20.0, (graph, empty)
+        assert 5.0 <= busy < 5.0 + max(4.0, 2.0 * empty), (graph, empty, busy)
+
+
 def test_errors():
     with pytest.raises(tdc_amd.TdcError):
         tdc_amd.Conv2dPlan(1, 4, 4, 2, 2, 5, 5, 1, 0)  # filter larger than input
